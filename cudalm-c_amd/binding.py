@@ -1,0 +1,120 @@
+"""ctypes view of libqlmx.so. Pointers may be given as ints, torch tensors (data_ptr), numpy arrays
+(host pointers, only where the C function takes host memory) or None."""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+SPAN_DTYPE = np.dtype(
+    [("pof", "<u8"), ("gof", "<u8"), ("qi0", "<u8"), ("n", "<u8"),
+     ("gi0", "<i4"), ("ngrp", "<i4"), ("sref", "<f4"), ("_pad", "<i4")])
+
+c_f, c_i, c_u64, c_vp, c_sz = C.c_float, C.c_int, C.c_ulonglong, C.c_void_p, C.c_size_t
+
+
+class QlmxError(RuntimeError):
+    pass
+
+
+def lib_path():
+    return os.path.join(HERE, "libqlmx.so")
+
+
+def _ptr(x):
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    if hasattr(x, "data_ptr"):
+        return x.data_ptr()
+    if isinstance(x, np.ndarray):
+        return x.ctypes.data
+    raise TypeError("cannot take a pointer of %r" % type(x))
+
+
+# name -> (restype, argtypes). Kept in step with include/qlmx.h; tests check every declared symbol.
+_STEP = [c_vp] * 10 + [c_i, c_i, c_i, c_f, c_f, c_f, c_f, c_f, c_vp, c_f, c_f, c_i, c_u64, c_i, c_vp, c_i, c_i, c_i, c_i, c_vp]
+SIGNATURES = {
+    "qlmx_version": (c_i, []),
+    "qlmx_init": (c_i, [c_i]),
+    "qlmx_last_error": (C.c_char_p, []),
+    "qlmx_device_name": (C.c_char_p, []),
+    "qlmx_malloc": (c_i, [C.POINTER(c_vp), c_sz]),
+    "qlmx_free": (c_i, [c_vp]),
+    "qlmx_memcpy_h2d": (c_i, [c_vp, c_vp, c_sz]),
+    "qlmx_memcpy_d2h": (c_i, [c_vp, c_vp, c_sz]),
+    "qlmx_memcpy_d2d": (c_i, [c_vp, c_vp, c_sz, c_vp]),
+    "qlmx_memset": (c_i, [c_vp, c_i, c_sz, c_vp]),
+    "qlmx_sync": (c_i, [c_vp]),
+    "qlmx_qhashu": (C.c_uint, [c_u64]),
+    "qlmx_qsri": (c_i, [c_f, c_u64, c_u64]),
+    "qlmx_qclmp": (c_i, [c_i, c_i, c_i]),
+    "qlmx_qd_get": (c_i, [c_vp, c_u64, c_i]),
+    "qlmx_qd_set_host": (None, [c_vp, c_u64, c_i, c_i]),
+    "qlmx_qd_bytes": (c_u64, [c_u64, c_i]),
+    "qlmx_encode": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_render": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_step": (c_i, _STEP),
+    "qlmx_servo": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_f, c_f, c_i, c_i, c_vp]),
+}
+
+
+class Qlmx:
+    """Loaded library. `init=True` binds device 0 and raises if that fails."""
+
+    def __init__(self, path=None, init=True, device=0):
+        path = path or lib_path()
+        if not os.path.exists(path):
+            raise QlmxError("libqlmx.so is not built (%s): run `python cudalm-c_amd/build.py`" % path)
+        self.lib = C.CDLL(path)
+        for name, (res, args) in SIGNATURES.items():
+            f = getattr(self.lib, name)
+            f.restype, f.argtypes = res, args
+        if init:
+            self.check(self.lib.qlmx_init(device))
+
+    def last_error(self):
+        return self.lib.qlmx_last_error().decode()
+
+    def check(self, rc):
+        if rc != 0:
+            raise QlmxError("libqlmx error %d: %s" % (rc, self.last_error()))
+
+    def call(self, name, *args):
+        conv = []
+        for a, t in zip(args, SIGNATURES[name][1]):
+            conv.append(_ptr(a) if t is c_vp else a)
+        rc = getattr(self.lib, name)(*conv)
+        if SIGNATURES[name][0] is c_i and name not in ("qlmx_version", "qlmx_qsri", "qlmx_qclmp", "qlmx_qd_get"):
+            self.check(rc)
+        return rc
+
+    # convenience wrappers with the reference's argument order
+    def encode(self, P, d, r, s, sp, nspan, group, dmax, packed, ngrp, stream=None):
+        self.call("qlmx_encode", P, d, r, s, sp, nspan, group, dmax, packed, ngrp, stream)
+
+    def render(self, P, d, s, sp, nspan, group, packed, gi_base, ng, stream=None):
+        self.call("qlmx_render", P, d, s, sp, nspan, group, packed, gi_base, ng, stream)
+
+    def step(self, P, G, d, r, s, m8, m8s, v8, v8s, sp, nspan, group, dmax, lr, b1, b2, wd, gscale, gsp,
+             inv_bc1, inv_sqrt_bc2, lrmode, t, adam, stat, packed, gi_base, ng, v4=0, stream=None):
+        self.call("qlmx_step", P, G, d, r, s, m8, m8s, v8, v8s, sp, nspan, group, dmax, lr, b1, b2, wd, gscale,
+                  gsp, inv_bc1, inv_sqrt_bc2, lrmode, t, adam, stat, packed, gi_base, ng, v4, stream)
+
+    def servo(self, d, r, s, sp, nspan, group, dmax, f_hi, f_lo, packed, ngrp, stream=None):
+        self.call("qlmx_servo", d, r, s, sp, nspan, group, dmax, f_hi, f_lo, packed, ngrp, stream)
+
+    def sync(self, stream=None):
+        self.call("qlmx_sync", stream)
+
+
+_cached = None
+
+
+def load(init=True):
+    global _cached
+    if _cached is None:
+        _cached = Qlmx(init=init)
+    return _cached

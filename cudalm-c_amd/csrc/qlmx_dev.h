@@ -1,0 +1,96 @@
+/* qlmx_dev.h -- device-side building blocks shared by the gfx950 kernels. */
+#ifndef QLMX_DEV_H
+#define QLMX_DEV_H
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/qlmx.h"
+
+#define QLMX_WAVE 64
+
+/* ---- error plumbing (host) ---- */
+void qlmx_set_error(const char *fmt, ...);
+int  qlmx_check_ready(void);
+#define QLMX_HIP(call, what)                                                                  \
+    do { hipError_t e_ = (call);                                                              \
+         if(e_ != hipSuccess){ qlmx_set_error("%s: %s", what, hipGetErrorString(e_));         \
+                               return QLMX_E_HIP; } } while(0)
+#define QLMX_REQUIRE(cond, ...)                                                               \
+    do { if(!(cond)){ qlmx_set_error(__VA_ARGS__); return QLMX_E_ARG; } } while(0)
+#define QLMX_LAUNCH_CHECK(what) QLMX_HIP(hipGetLastError(), what)
+
+/* ---- 64-bit hash and stochastic rounding (qlm.cuh:78-87) ----
+ * The key of element i at step t is i*KI + t*KT; callers add KI per consecutive element and a
+ * per-stream constant instead of multiplying again. */
+#define QLMX_KI 0x2545F4914F6CDD1DULL
+#define QLMX_KT 0x9E3779B97F4A7C15ULL
+
+__host__ __device__ __forceinline__ uint32_t qx_hash(uint64_t x){
+    x += 0x9E3779B97F4A7C15ULL;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ULL;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBULL;
+    return (uint32_t)(x ^ (x >> 31));
+}
+/* floor(v) + [u < frac(v)] with u = top 24 hash bits * 2^-24; `key` is the finished hash key */
+__host__ __device__ __forceinline__ int qx_sround(float v, uint64_t key){
+    float fl = floorf(v);
+    uint32_t h = qx_hash(key);
+    float u = (float)(h >> 8) * (1.0f / 16777216.0f);
+    return (int)fl + (u < (v - fl) ? 1 : 0);
+}
+__host__ __device__ __forceinline__ int qx_clamp(int v, int lo, int hi){ return v < lo ? lo : (v > hi ? hi : v); }
+
+/* signed 4-bit field k (0..7) of a 32-bit word holding 8 consecutive digits (qlm.cuh:96-101) */
+__device__ __forceinline__ int qx_nib(uint32_t w, int k){ return ((int)(w << (28 - 4*k))) >> 28; }
+
+/* ---- span lookup: the owner of group gi. The table is ascending in gi0, so a binary search
+ * returns what the reference's first-match linear scan returns (qlm.cuh:114-117). ---- */
+__device__ __forceinline__ int qx_span_of(const qlmx_span *sp, int nspan, int gi){
+    int lo = 0, hi = nspan - 1;
+    while(lo < hi){
+        int mid = (lo + hi + 1) >> 1;
+        if(sp[mid].gi0 <= gi) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+
+/* ---- DPP reductions over a row of 16 lanes ----
+ * quad_perm [1,0,3,2] = 0xB1, [2,3,0,1] = 0x4E, row_half_mirror = 0x141, row_mirror = 0x140.
+ * After the four steps every lane of the row holds the row's maximum. */
+template<int CTRL> __device__ __forceinline__ float qx_dpp(float v){
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template<int CTRL> __device__ __forceinline__ int qx_dpp_i(int v){
+    return __builtin_amdgcn_mov_dpp(v, CTRL, 0xF, 0xF, true);
+}
+__device__ __forceinline__ float qx_row16_max(float v){
+    v = fmaxf(v, qx_dpp<0xB1>(v));
+    v = fmaxf(v, qx_dpp<0x4E>(v));
+    v = fmaxf(v, qx_dpp<0x141>(v));
+    v = fmaxf(v, qx_dpp<0x140>(v));
+    return v;
+}
+__device__ __forceinline__ int qx_row16_maxi(int v){
+    v = max(v, qx_dpp_i<0xB1>(v));
+    v = max(v, qx_dpp_i<0x4E>(v));
+    v = max(v, qx_dpp_i<0x141>(v));
+    v = max(v, qx_dpp_i<0x140>(v));
+    return v;
+}
+__device__ __forceinline__ int qx_row16_sum(int v){
+    v += qx_dpp_i<0xB1>(v);
+    v += qx_dpp_i<0x4E>(v);
+    v += qx_dpp_i<0x141>(v);
+    v += qx_dpp_i<0x140>(v);
+    return v;
+}
+/* full 64-lane sum / max built from the row step plus two cross-row exchanges */
+__device__ __forceinline__ float qx_wave_sum(float v){
+    for(int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float qx_wave_max(float v){
+    for(int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+#endif

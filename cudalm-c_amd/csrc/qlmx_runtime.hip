@@ -1,0 +1,87 @@
+/* qlmx_runtime.hip -- device selection, memory helpers, error text and the host-side integer
+ * helpers of the C ABI. Mirrors what cudalm.cu does through cudaSetDevice / dmalloc / cudaMemcpy /
+ * cudaMemset / cudaDeviceSynchronize (cudalm.cu:147-154, 6628). There is no CPU fallback: without
+ * a gfx950 device every compute entry point fails with QLMX_E_NODEV. */
+#include "qlmx_dev.h"
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+static thread_local char g_err[512] = "";
+static int  g_ready = 0;
+static char g_devname[256] = "";
+
+void qlmx_set_error(const char *fmt, ...){
+    va_list ap; va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+}
+int qlmx_check_ready(void){
+    if(g_ready) return QLMX_OK;
+    qlmx_set_error("libqlmx: qlmx_init() has not succeeded (no gfx950 device bound)");
+    return QLMX_E_NODEV;
+}
+
+extern "C" int qlmx_version(void){ return QLMX_VERSION; }
+extern "C" const char *qlmx_last_error(void){ return g_err; }
+extern "C" const char *qlmx_device_name(void){ return g_devname; }
+
+extern "C" int qlmx_init(int device){
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if(e != hipSuccess || n <= 0){
+        qlmx_set_error("qlmx_init: no HIP device (%s)", e != hipSuccess ? hipGetErrorString(e) : "count 0");
+        return QLMX_E_NODEV;
+    }
+    QLMX_REQUIRE(device >= 0 && device < n, "qlmx_init: device %d of %d", device, n);
+    QLMX_HIP(hipSetDevice(device), "hipSetDevice");
+    hipDeviceProp_t pr;
+    QLMX_HIP(hipGetDeviceProperties(&pr, device), "hipGetDeviceProperties");
+    snprintf(g_devname, sizeof g_devname, "%s (%s, %d CUs)", pr.name, pr.gcnArchName, pr.multiProcessorCount);
+    if(strncmp(pr.gcnArchName, "gfx950", 6) != 0){
+        qlmx_set_error("qlmx_init: device is %s; this library carries gfx950 code only", pr.gcnArchName);
+        return QLMX_E_NODEV;
+    }
+    g_ready = 1;
+    return QLMX_OK;
+}
+
+extern "C" int qlmx_malloc(void **p, size_t bytes){
+    QLMX_REQUIRE(p, "qlmx_malloc: NULL out pointer");
+    QLMX_HIP(hipMalloc(p, bytes ? bytes : 1), "hipMalloc");
+    return QLMX_OK;
+}
+extern "C" int qlmx_free(void *p){ QLMX_HIP(hipFree(p), "hipFree"); return QLMX_OK; }
+extern "C" int qlmx_memcpy_h2d(void *dst, const void *src, size_t bytes){
+    QLMX_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice), "hipMemcpy h2d"); return QLMX_OK; }
+extern "C" int qlmx_memcpy_d2h(void *dst, const void *src, size_t bytes){
+    QLMX_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost), "hipMemcpy d2h"); return QLMX_OK; }
+extern "C" int qlmx_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream){
+    QLMX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream), "hipMemcpy d2d"); return QLMX_OK; }
+extern "C" int qlmx_memset(void *dst, int value, size_t bytes, void *stream){
+    QLMX_HIP(hipMemsetAsync(dst, value, bytes, (hipStream_t)stream), "hipMemset"); return QLMX_OK; }
+extern "C" int qlmx_sync(void *stream){
+    if(stream) QLMX_HIP(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+    else       QLMX_HIP(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    return QLMX_OK;
+}
+
+/* ---- host integer helpers (qlm.cuh:78-111) ---- */
+extern "C" unsigned int qlmx_qhashu(unsigned long long x){ return qx_hash(x); }
+extern "C" int qlmx_qsri(float v, unsigned long long i, unsigned long long t){
+    return qx_sround(v, i * QLMX_KI + t * QLMX_KT);
+}
+extern "C" int qlmx_qclmp(int v, int lo, int hi){ return qx_clamp(v, lo, hi); }
+extern "C" int qlmx_qd_get(const signed char *d, unsigned long long i, int packed){
+    if(!packed) return (int)d[i];
+    const unsigned b = (unsigned char)d[i >> 1];
+    const int v = (i & 1ULL) ? (int)(b >> 4) : (int)(b & 15u);
+    return v >= 8 ? v - 16 : v;
+}
+extern "C" void qlmx_qd_set_host(signed char *d, unsigned long long i, int v, int packed){
+    if(!packed){ d[i] = (signed char)v; return; }
+    unsigned char *b = (unsigned char *)&d[i >> 1];
+    const unsigned nib = (unsigned)v & 15u;
+    *b = (unsigned char)((i & 1ULL) ? ((*b & 0x0Fu) | (nib << 4)) : ((*b & 0xF0u) | nib));
+}
+extern "C" unsigned long long qlmx_qd_bytes(unsigned long long nq, int packed){ return packed ? (nq + 1) / 2 : nq; }

@@ -1,0 +1,284 @@
+/* qlmx_step.hip -- Integer AdamW / integer Lion update + moment requantisation for gfx950.
+ *
+ * Replaces qlm_step_launch and its two kernels (qlm.cuh:181-397; CPU twin cpu_kern.h:798-852).
+ * The arithmetic is the reference's, operation for operation and in the same order, compiled
+ * without FMA contraction: every float feeds a stochastic-rounding compare, so one ulp flips
+ * integer state. Divisions and square roots are the correctly rounded ones.
+ *
+ * Mapping. The reference gives a CUDA block (or a 32-lane warp) to each group. Here a group
+ * belongs to one DPP row (16 lanes) of a 64-lane wavefront, so a wave carries four groups and a
+ * 256-thread workgroup sixteen. With the headline group of 128 each lane owns 8 consecutive
+ * elements: one 32-bit word of packed digits, one 64-bit word each of residuals and of both
+ * moments, two 128-bit words of gradient. A lane therefore writes whole bytes it alone owns, and
+ * the reference's cross-lane nibble exchange (qlm.cuh:349-352) disappears. The two group maxima are
+ * reduced inside the row with four DPP steps. Any other group size, a short tail group or an
+ * unaligned span takes the pair-per-lane path in the same kernel (a lane still owns whole bytes).
+ *
+ * HBM traffic per weight: read G 4 + d 0.5 + r 1 + m8 1 + v8 1, write d 0.5 + r 1 + m8 1 + v8 1
+ * = 11 B, plus 20 B of scales per group (0.16 B/weight at 128) and 4 B when P is rendered.
+ */
+#include "qlmx_dev.h"
+
+struct StepParams {
+    float *P; const float *G;
+    signed char *d; signed char *r; const float *s;
+    signed char *m8; float *m8s; unsigned char *v8; float *v8s;
+    const qlmx_span *sp; int nspan, group, dmax;
+    float lr, b1, b2, wd, gscale; const float *gsp;
+    float inv_bc1, inv_sqrt_bc2; int lrmode;
+    unsigned long long t; unsigned long long *stat;
+    int packed, gi_base, ng, v4;
+    int vec_ok;      /* base pointers are aligned for the 128/64/32-bit accesses of the fast path */
+};
+
+struct GroupCtx {           /* per-group constants, uniform over the row */
+    float sg, L, dec, ms_old, vs_old, veps, gs;
+    float b1, b2, omb1, omb2, inv_bc1, inv_sqrt_bc2;
+    int dmax, v4;
+};
+
+struct ElemRes { float mn, rv; int dd, rr, idl, carry; };
+
+/* New first moment, new (stored form of the) second moment and the clamped Adam ratio u of one
+ * element: qlm.cuh:209-229. */
+template<bool ADAM>
+__device__ __forceinline__ void elem_moments(const GroupCtx &c, float graw, int m8v, int v8v,
+                                             float &mn, float &rvs, float &u){
+    float gr = graw * c.gs;
+    float mv = (float)m8v * c.ms_old;
+    if(ADAM){
+        float sv = (float)v8v * c.vs_old; if(c.v4) sv = sv * sv;
+        float vv = sv * sv;
+        mn = c.b1 * mv + c.omb1 * gr;
+        vv = c.b2 * vv + c.omb2 * gr * gr;
+        float rv = sqrtf(vv);
+        u = (mn * c.inv_bc1) / (rv * c.inv_sqrt_bc2 + c.veps);
+        u = fmaxf(-8.0f, fminf(8.0f, u));
+        rvs = c.v4 ? sqrtf(rv) : rv;
+    } else {
+        float cc = c.b1 * mv + c.omb1 * gr;
+        u = (float)((cc > 0.0f) - (cc < 0.0f));
+        mn = c.b2 * mv + c.omb2 * gr;
+        rvs = 0.0f;
+    }
+}
+
+/* One element of qlm.cuh:207-242. `key` is the finished hash key of (element, step). */
+template<bool ADAM>
+__device__ __forceinline__ ElemRes step_elem(const GroupCtx &c, float graw, int m8v, int v8v,
+                                             int dd, int rold, uint64_t key){
+    ElemRes o; float u;
+    elem_moments<ADAM>(c, graw, m8v, v8v, o.mn, o.rv, u);
+    o.idl = qx_sround(-(c.L * u + c.dec * (float)dd), key);
+    int rr = rold + o.idl;
+    int cy = 0;
+    if(rr > 64)       cy =  (((rr - 65) >> 7) + 1);
+    else if(rr < -64) cy = -((((-rr) - 65) >> 7) + 1);
+    o.carry = cy;
+    o.rr = rr - cy * 128;
+    o.dd = qx_clamp(dd + cy, -c.dmax, c.dmax);
+    return o;
+}
+
+template<bool ADAM>
+__global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
+    const int lane16 = threadIdx.x & 15;
+    const int team = (int)((blockIdx.x * (unsigned)blockDim.x + threadIdx.x) >> 4);
+    if(team >= a.ng) return;                       /* whole rows leave together */
+    const int gi = a.gi_base + team;
+    const int si = qx_span_of(a.sp, a.nspan, gi);
+    const qlmx_span S = a.sp[si];
+    const uint64_t j0 = (uint64_t)(gi - S.gi0) * (uint64_t)a.group;
+    const uint64_t left = S.n - j0;
+    const int n = (int)((uint64_t)a.group < left ? (uint64_t)a.group : left);
+    const uint64_t pof = S.pof + j0, qi0 = S.qi0 + j0, gof = S.gof + j0;
+
+    GroupCtx c;
+    c.gs = a.gsp ? *a.gsp : a.gscale;
+    c.sg = a.s[gi];
+    c.L = a.lr * 128.0f / (a.lrmode ? c.sg : S.sref);
+    c.dec = a.lr * a.wd * 128.0f;
+    c.ms_old = a.m8s[gi];
+    c.vs_old = (ADAM && a.v8s) ? a.v8s[gi] : 0.0f;
+    { float q1 = 1.0f * c.vs_old; if(a.v4) q1 = q1 * q1; c.veps = fmaxf(q1, 1e-8f); }
+    c.b1 = a.b1; c.b2 = a.b2; c.omb1 = 1.0f - a.b1; c.omb2 = 1.0f - a.b2;
+    c.inv_bc1 = a.inv_bc1; c.inv_sqrt_bc2 = a.inv_sqrt_bc2;
+    c.dmax = a.dmax; c.v4 = a.v4;
+
+    const uint64_t kt  = a.t * QLMX_KT;
+    const uint64_t ktm = kt + 0x5EEDULL * QLMX_KT;
+    const uint64_t ktv = kt + 0xBEEFULL * QLMX_KT;
+
+    unsigned long long st_carry = 0, st_rail = 0, st_zero = 0, st_idl = 0;
+    const bool want_stat = a.stat != nullptr;
+
+    const bool fast = a.vec_ok && a.group == 128 && a.packed && n == 128 && ((pof | qi0 | gof) & 7ULL) == 0;
+    if(fast){
+        const uint64_t e0 = (uint64_t)lane16 * 8;
+        const uint64_t q = qi0 + e0;
+        const float4 g0 = *(const float4 *)(a.G + gof + e0);
+        const float4 g1 = *(const float4 *)(a.G + gof + e0 + 4);
+        const uint32_t dw = *(const uint32_t *)(a.d + (q >> 1));
+        const uint2 rw = *(const uint2 *)(a.r + q);
+        const uint2 mw = *(const uint2 *)(a.m8 + q);
+        uint2 vw = make_uint2(0u, 0u);
+        if(ADAM) vw = *(const uint2 *)(a.v8 + q);
+        const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+        float mn[8], rv[8], pv[8];
+        uint32_t dnew = 0, rn0 = 0, rn1 = 0;
+        float am = 0.0f, vm = 0.0f;
+        uint64_t key = q * QLMX_KI;
+#pragma unroll
+        for(int k = 0; k < 8; k++){
+            const uint32_t rword = k < 4 ? rw.x : rw.y, mword = k < 4 ? mw.x : mw.y, vword = k < 4 ? vw.x : vw.y;
+            const int sh = 8 * (k & 3);
+            const int rold = (int)(signed char)(rword >> sh);
+            const int m8v  = (int)(signed char)(mword >> sh);
+            const int v8v  = (int)((vword >> sh) & 0xFFu);
+            const int dd   = qx_nib(dw, k);
+            ElemRes o = step_elem<ADAM>(c, gv[k], m8v, v8v, dd, rold, key + kt);
+            mn[k] = o.mn; rv[k] = o.rv;
+            pv[k] = c.sg * (float)o.dd;
+            dnew |= ((uint32_t)o.dd & 15u) << (4 * k);
+            if(k < 4) rn0 |= ((uint32_t)o.rr & 0xFFu) << sh; else rn1 |= ((uint32_t)o.rr & 0xFFu) << sh;
+            am = fmaxf(am, fabsf(o.mn)); vm = fmaxf(vm, o.rv);
+            if(want_stat){
+                unsigned ai = (unsigned)(o.idl < 0 ? -o.idl : o.idl);
+                st_idl = st_idl > ai ? st_idl : ai;
+                st_carry += (unsigned)(o.carry < 0 ? -o.carry : o.carry);
+                st_rail += (o.dd == c.dmax) | (o.dd == -c.dmax);
+                st_zero += (o.dd == 0);
+            }
+            key += QLMX_KI;
+        }
+        *(uint32_t *)(a.d + (q >> 1)) = dnew;
+        *(uint2 *)(a.r + q) = make_uint2(rn0, rn1);
+        if(a.P){
+            *(float4 *)(a.P + pof + e0)     = make_float4(pv[0], pv[1], pv[2], pv[3]);
+            *(float4 *)(a.P + pof + e0 + 4) = make_float4(pv[4], pv[5], pv[6], pv[7]);
+        }
+        am = qx_row16_max(am); vm = qx_row16_max(vm);
+        const float ms = am > 0.0f ? am / 127.0f : 1e-12f;
+        const float vs = vm > 0.0f ? vm / 255.0f : 1e-12f;
+        if(lane16 == 0){ a.m8s[gi] = ms; if(ADAM) a.v8s[gi] = vs; }
+        uint32_t mo0 = 0, mo1 = 0, vo0 = 0, vo1 = 0;
+        key = q * QLMX_KI;
+#pragma unroll
+        for(int k = 0; k < 8; k++){
+            const int sh = 8 * (k & 3);
+            int mq = qx_clamp(qx_sround(mn[k] / ms, key + ktm), -127, 127);
+            if(k < 4) mo0 |= ((uint32_t)mq & 0xFFu) << sh; else mo1 |= ((uint32_t)mq & 0xFFu) << sh;
+            if(ADAM){
+                int vq = qx_clamp(qx_sround(rv[k] / vs, key + ktv), 0, 255);
+                if(vq == 0 && rv[k] > 0.0f) vq = 1;
+                if(k < 4) vo0 |= (uint32_t)vq << sh; else vo1 |= (uint32_t)vq << sh;
+            }
+            key += QLMX_KI;
+        }
+        *(uint2 *)(a.m8 + q) = make_uint2(mo0, mo1);
+        if(ADAM) *(uint2 *)(a.v8 + q) = make_uint2(vo0, vo1);
+    } else {
+        /* pair-per-lane path: lane owns elements {2*lane16, 2*lane16+1} + 32*k, i.e. whole bytes
+         * of packed digits. Sweep one updates digits, residuals and P; sweep two recomputes the
+         * moments from m8/v8/G, which sweep one does not write (same operations, hence the same
+         * bits), and requantises them. Nothing is held in registers across the reduction. */
+        float am = 0.0f, vm = 0.0f;
+        for(int jb = 2 * lane16; jb < n; jb += 32){
+            int ddn[2] = {0, 0};
+            unsigned oldb = 0;
+            if(a.packed) oldb = (unsigned char)a.d[(qi0 + jb) >> 1];
+#pragma unroll
+            for(int h = 0; h < 2; h++){
+                const int j = jb + h;
+                if(j < n){
+                    const uint64_t qi = qi0 + j;
+                    int dd;
+                    if(a.packed){ int v = h ? (int)(oldb >> 4) : (int)(oldb & 15u); dd = v >= 8 ? v - 16 : v; }
+                    else dd = (int)a.d[qi];
+                    ElemRes o = step_elem<ADAM>(c, a.G[gof + j], (int)a.m8[qi], ADAM ? (int)a.v8[qi] : 0, dd,
+                                                (int)a.r[qi], qi * QLMX_KI + kt);
+                    a.r[qi] = (signed char)o.rr;
+                    if(a.P) a.P[pof + j] = c.sg * (float)o.dd;
+                    if(!a.packed) a.d[qi] = (signed char)o.dd;
+                    ddn[h] = o.dd;
+                    am = fmaxf(am, fabsf(o.mn)); vm = fmaxf(vm, o.rv);
+                    if(want_stat){
+                        unsigned ai = (unsigned)(o.idl < 0 ? -o.idl : o.idl);
+                        st_idl = st_idl > ai ? st_idl : ai;
+                        st_carry += (unsigned)(o.carry < 0 ? -o.carry : o.carry);
+                        st_rail += (o.dd == c.dmax) | (o.dd == -c.dmax);
+                        st_zero += (o.dd == 0);
+                    }
+                }
+            }
+            if(a.packed) a.d[(qi0 + jb) >> 1] = (signed char)(((ddn[1] & 15) << 4) | (ddn[0] & 15));
+        }
+        am = qx_row16_max(am); vm = qx_row16_max(vm);
+        const float ms = am > 0.0f ? am / 127.0f : 1e-12f;
+        const float vs = vm > 0.0f ? vm / 255.0f : 1e-12f;
+        for(int jb = 2 * lane16; jb < n; jb += 32){
+#pragma unroll
+            for(int h = 0; h < 2; h++){
+                const int j = jb + h;
+                if(j < n){
+                    const uint64_t qi = qi0 + j;
+                    float mn, rvs, u;
+                    elem_moments<ADAM>(c, a.G[gof + j], (int)a.m8[qi], ADAM ? (int)a.v8[qi] : 0, mn, rvs, u);
+                    a.m8[qi] = (signed char)qx_clamp(qx_sround(mn / ms, qi * QLMX_KI + ktm), -127, 127);
+                    if(ADAM){
+                        int vq = qx_clamp(qx_sround(rvs / vs, qi * QLMX_KI + ktv), 0, 255);
+                        if(vq == 0 && rvs > 0.0f) vq = 1;
+                        a.v8[qi] = (unsigned char)vq;
+                    }
+                }
+            }
+        }
+        /* written last: the recomputation above reads the old per-group moment scales via `c` */
+        if(lane16 == 0){ a.m8s[gi] = ms; if(ADAM) a.v8s[gi] = vs; }
+    }
+
+    if(want_stat){
+        /* row totals, then one lane per group updates the four counters */
+        unsigned sc = (unsigned)qx_row16_sum((int)st_carry), sr = (unsigned)qx_row16_sum((int)st_rail),
+                 sz = (unsigned)qx_row16_sum((int)st_zero);
+        unsigned mi = (unsigned)qx_row16_maxi((int)st_idl);
+        if(lane16 == 0){
+            atomicAdd(&a.stat[0], (unsigned long long)sc);
+            atomicAdd(&a.stat[1], (unsigned long long)sr);
+            atomicAdd(&a.stat[2], (unsigned long long)sz);
+            atomicMax(&a.stat[3], (unsigned long long)mi);
+        }
+    }
+}
+
+/* qlm_step_launch (qlm.cuh:377-397) */
+extern "C" int qlmx_step(float *P, const float *G, signed char *d, signed char *r, const float *s,
+              signed char *m8, float *m8s, unsigned char *v8, float *v8s,
+              const qlmx_span *sp, int nspan, int group, int dmax,
+              float lr, float b1, float b2, float wd, float gscale, const float *gsp,
+              float inv_bc1, float inv_sqrt_bc2, int lrmode,
+              unsigned long long t, int adam, long long *stat, int packed,
+              int gi_base, int ng, int v4, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(G && d && r && s && m8 && m8s && sp, "qlmx_step: NULL buffer");
+    QLMX_REQUIRE(!adam || (v8 && v8s), "qlmx_step: adam needs v8 and v8s");
+    QLMX_REQUIRE(nspan > 0 && ng >= 0 && gi_base >= 0, "qlmx_step: bad span/group range");
+    QLMX_REQUIRE(group >= 2 && group <= 256, "qlmx_step: group %d outside [2,256]", group);
+    QLMX_REQUIRE(!packed || (dmax <= 7 && (group & 1) == 0), "qlmx_step: packed digits need dmax<=7 and an even group");
+    QLMX_REQUIRE(dmax >= 1 && dmax <= 127, "qlmx_step: dmax %d", dmax);
+    if(ng == 0) return QLMX_OK;
+    StepParams a;
+    a.P = P; a.G = G; a.d = d; a.r = r; a.s = s; a.m8 = m8; a.m8s = m8s; a.v8 = v8; a.v8s = v8s;
+    a.sp = sp; a.nspan = nspan; a.group = group; a.dmax = dmax;
+    a.lr = lr; a.b1 = b1; a.b2 = b2; a.wd = wd; a.gscale = gscale; a.gsp = gsp;
+    a.inv_bc1 = inv_bc1; a.inv_sqrt_bc2 = inv_sqrt_bc2; a.lrmode = lrmode;
+    a.t = t; a.stat = (unsigned long long *)stat; a.packed = packed; a.gi_base = gi_base; a.ng = ng; a.v4 = v4;
+    a.vec_ok = (((uintptr_t)P | (uintptr_t)G) & 15) == 0 && (((uintptr_t)r | (uintptr_t)m8 | (uintptr_t)v8) & 7) == 0
+               && ((uintptr_t)d & 3) == 0;
+    const unsigned blocks = (unsigned)((ng + 15) / 16);
+    hipStream_t st = (hipStream_t)stream;
+    if(adam) hipLaunchKernelGGL(k_qlmx_step<true>,  dim3(blocks), dim3(256), 0, st, a);
+    else     hipLaunchKernelGGL(k_qlmx_step<false>, dim3(blocks), dim3(256), 0, st, a);
+    QLMX_LAUNCH_CHECK("qlmx_step launch");
+    return QLMX_OK;
+}

@@ -1,0 +1,103 @@
+/* qlmx.h -- C ABI of libqlmx: cudalm's QLM 4-bit weight path on MI355X (gfx950).
+ *
+ * The reference (Dsg2/cudalm-c) is one translation unit with no FFI; its backend seam is the set of
+ * call signatures cudalm.cu uses against qlm.cuh and against its own GEMM wrappers, swapped for the
+ * CPU build by cpu_rt.h / cpu_kern.h. Every entry point below replaces one of those call sites and
+ * cites it (paths relative to the reference tree). All device buffers are caller-owned; `stream`
+ * is a hipStream_t passed as void* (NULL = the default stream, which is what the reference uses).
+ * Launches are asynchronous and ordered by the stream. Every function returns 0 on success and a
+ * negative QLMX_E_* code on failure; qlmx_last_error() holds the message of the calling thread's
+ * last failure. The reference's print-and-exit(1) behaviour (ck/ckb, cudalm.cu:147-152) is kept by
+ * the C++ mirror in cudalm-c_amd/host/, not here.
+ *
+ * Plain C: pointers and sizes only, no C++ or framework types.
+ */
+#ifndef QLMX_H
+#define QLMX_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QLMX_VERSION 1
+
+#define QLMX_OK            0
+#define QLMX_E_ARG        -1   /* bad argument (shape, alignment, NULL, unsupported combination) */
+#define QLMX_E_HIP        -2   /* a HIP runtime call failed                                     */
+#define QLMX_E_NODEV      -3   /* no gfx950 device / library not initialised                    */
+#define QLMX_E_LIMIT      -4   /* a documented size limit was exceeded                          */
+
+/* One quantized span = one whole weight tensor. Same layout as QSpanD (qlm.cuh:30-38), 48 bytes. */
+typedef struct qlmx_span {
+    unsigned long long pof;   /* element offset in the rendered fp32 view P            */
+    unsigned long long gof;   /* element offset of the gradient in G                   */
+    unsigned long long qi0;   /* element offset in d / r / m8 / v8 (even when packed)  */
+    unsigned long long n;     /* elements                                              */
+    int   gi0, ngrp;          /* first scale group, number of groups                   */
+    float sref;               /* frozen mean scale for the relative-LR mode            */
+} qlmx_span;
+
+/* ---- runtime: replaces cudaSetDevice / dmalloc / cudaMemcpy / cudaMemset /
+ *      cudaDeviceSynchronize as used by cudalm.cu:147-154, 6628 and qlm.cuh:505-521 ---- */
+int         qlmx_version(void);
+int         qlmx_init(int device);
+const char *qlmx_last_error(void);
+const char *qlmx_device_name(void);
+int         qlmx_malloc(void **p, size_t bytes);
+int         qlmx_free(void *p);
+int         qlmx_memcpy_h2d(void *dst, const void *src, size_t bytes);
+int         qlmx_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int         qlmx_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
+int         qlmx_memset(void *dst, int value, size_t bytes, void *stream);
+int         qlmx_sync(void *stream);
+
+/* ---- host integer helpers: the __host__ __device__ inlines of qlm.cuh:78-111, used by the
+ *      reference's checkpoint code and selftest reference (cudalm.cu:10574-10580) ---- */
+unsigned int       qlmx_qhashu(unsigned long long x);                              /* qlm.cuh:78  */
+int                qlmx_qsri(float v, unsigned long long i, unsigned long long t);  /* qlm.cuh:83  */
+int                qlmx_qclmp(int v, int lo, int hi);                               /* qlm.cuh:88  */
+int                qlmx_qd_get(const signed char *d, unsigned long long i, int packed);          /* :96  */
+void               qlmx_qd_set_host(signed char *d, unsigned long long i, int v, int packed);    /* :102 */
+unsigned long long qlmx_qd_bytes(unsigned long long nq, int packed);                              /* :109 */
+
+/* ---- k_qlm_encode (qlm.cuh:136-167; launch at qlm.cuh:524): P -> digits, residual, scales.
+ * `sp` is the DEVICE copy of the span table, ngrp the total number of groups. group in [2,256] and
+ * even when packed; dmax <= 7 when packed. ---- */
+int qlmx_encode(const float *P, signed char *d, signed char *r, float *s,
+                const qlmx_span *sp, int nspan, int group, int dmax, int packed, int ngrp,
+                void *stream);
+
+/* ---- k_qlm_render (qlm.cuh:170-178; launches at 538, 578, 589): P = s * digit for groups
+ * gi_base .. gi_base+ng-1. ---- */
+int qlmx_render(float *P, const signed char *d, const float *s,
+                const qlmx_span *sp, int nspan, int group, int packed, int gi_base, int ng,
+                void *stream);
+
+/* ---- qlm_step_launch (qlm.cuh:377-397; called from cudalm.cu:6086, 6126, 10601, 10617):
+ * Integer AdamW (adam=1) or integer Lion (adam=0) over groups gi_base .. gi_base+ng-1, then the
+ * moments are re-quantized with fresh per-group scales. Argument order and meaning are the
+ * reference's. gsp, when not NULL, is a device pointer to the gradient clip multiplier and
+ * overrides gscale (no host round trip). stat, when not NULL, is a device long long[4]
+ * {sum |carry|, railed digits, zero digits, max |LSB step|} that is accumulated into.
+ * Differences from the reference, both additive: P may be NULL (the fp32 view is not kept when the
+ * GEMMs read the digits directly); v4 carries the QLM_V4 switch (qlm.cuh:62-67) that the reference
+ * keeps in a device global. ---- */
+int qlmx_step(float *P, const float *G, signed char *d, signed char *r, const float *s,
+              signed char *m8, float *m8s, unsigned char *v8, float *v8s,
+              const qlmx_span *sp, int nspan, int group, int dmax,
+              float lr, float b1, float b2, float wd, float gscale, const float *gsp,
+              float inv_bc1, float inv_sqrt_bc2, int lrmode,
+              unsigned long long t, int adam, long long *stat, int packed,
+              int gi_base, int ng, int v4, void *stream);
+
+/* ---- k_qlm_servo (qlm.cuh:404-441; launched from cudalm.cu:6099): rail-fraction scale servo
+ * and re-encode of (d, r) for the groups whose scale moved. ---- */
+int qlmx_servo(signed char *d, signed char *r, float *s,
+               const qlmx_span *sp, int nspan, int group, int dmax,
+               float f_hi, float f_lo, int packed, int ngrp, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QLMX_H */

@@ -1,0 +1,147 @@
+"""GPU parity for the quantized weight format and the integer optimizer: every byte of d, r, m8,
+v8, the scales and the rendered view must equal the golden vectors (written by the reference's CPU
+backend) and the CPU oracle on the same seeded inputs. All calls go through the C ABI."""
+import numpy as np
+import pytest
+
+from __graft_entry__ import load_package
+from oracle.binding import make_spans
+
+pkg = load_package()
+f32 = np.float32
+pytestmark = pytest.mark.gpu
+
+QLM_CASES = ["g128_adam_rel", "g128_adam_abs", "g128_lion", "g64_d3_v4", "g256_int8", "g96_block", "g32_ternary"]
+
+
+@pytest.fixture(scope="module")
+def q():
+    return pkg.load()
+
+
+def dev(a):
+    import torch
+    if a.dtype.names:
+        a = a.view(np.uint8)
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def beq(t, ref):
+    got = host(t) if hasattr(t, "cpu") else t
+    return np.array_equal(np.ascontiguousarray(got).view(np.uint8), np.ascontiguousarray(ref).view(np.uint8))
+
+
+@pytest.mark.parametrize("name", QLM_CASES)
+def test_golden_encode_render_step_servo(q, golden, name):
+    import torch
+    g = golden("qlm_" + name)
+    group, dmax, packed, adam, lrmode, v4 = (int(x) for x in g["cfg"])
+    tab0, nq, ng = make_spans([int(x) for x in g["sizes"]], group)
+    tab0["gof"] = g["tab"]["gof"]
+    nsp = len(tab0)
+    P = dev(g["P0"])
+    d = torch.zeros(len(g["enc_d"]), dtype=torch.int8, device="cuda")
+    r = torch.zeros(nq, dtype=torch.int8, device="cuda")
+    s = torch.zeros(ng, dtype=torch.float32, device="cuda")
+    sp = dev(tab0)
+    q.encode(P, d, r, s, sp, nsp, group, dmax, packed, ng)
+    assert beq(d, g["enc_d"]) and beq(r, g["enc_r"]) and beq(s, g["enc_s"])
+    sp = dev(g["tab"])
+    q.render(P, d, s, sp, nsp, group, packed, 0, ng)
+    assert beq(P, g["enc_P"])
+    m8 = torch.zeros(nq, dtype=torch.int8, device="cuda"); v8 = torch.zeros(nq, dtype=torch.uint8, device="cuda")
+    m8s = torch.zeros(ng, device="cuda"); v8s = torch.zeros(ng, device="cuda")
+    stat = torch.zeros(4, dtype=torch.int64, device="cuda")
+    gsp = dev(np.array([0.37], f32))
+    for t in range(1, 5):
+        hp = g["hp%d" % t]
+        if t == 2:
+            r = dev(g["t2_r_in"])
+        q.step(P, dev(g["G%d" % t]), d, r, s, m8, m8s, v8 if adam else None, v8s if adam else None, sp, nsp, group,
+               dmax, float(hp[0]), float(hp[1]), float(hp[2]), float(hp[3]), 1.0 if t != 3 else 0.0,
+               gsp if t == 3 else None, float(hp[4]), float(hp[5]), lrmode, t, adam, stat, packed, 0, ng, v4)
+        for buf, key in [(P, "P%d"), (d, "d%d"), (r, "r%d"), (m8, "m8_%d"), (m8s, "m8s_%d")]:
+            assert beq(buf, g[key % t]), (name, t, key)
+        if adam:
+            assert beq(v8, g["v8_%d" % t]) and beq(v8s, g["v8s_%d" % t]), (name, t)
+    assert np.array_equal(host(stat), g["stat"])
+    gi_base, ng2 = (int(x) for x in g["sub"])
+    q.step(P, dev(g["G5"]), d, r, s, m8, m8s, v8 if adam else None, v8s if adam else None, sp, nsp, group, dmax,
+           3e-4, 0.9, 0.95, 0.1, 1.0, None, 1.5, 1.25, lrmode, 5, adam, None, packed, gi_base, ng2, v4)
+    for buf, key in [(P, "P5"), (d, "d5"), (r, "r5"), (m8, "m8_5"), (m8s, "m8s_5")]:
+        assert beq(buf, g[key]), (name, "sub", key)
+    d2, r2, s2 = dev(g["sv_d_in"]), dev(g["sv_r_in"]), dev(g["sv_s_in"])
+    q.servo(d2, r2, s2, sp, nsp, group, dmax, float(g["sv_f"][0]), float(g["sv_f"][1]), packed, ng)
+    assert beq(d2, g["sv_d"]) and beq(r2, g["sv_r"]) and beq(s2, g["sv_s"])
+
+
+@pytest.mark.parametrize("nopview", [False, True])
+def test_step_vs_oracle_seeded_2m(q, orc, nopview):
+    """Three consecutive steps over 2M weights in two spans (one with a short tail group and a
+    shifted gradient offset), random integer state: byte-identical to the CPU oracle. With P=NULL
+    the integer state must be the same as with the view rendered."""
+    import torch
+    group, dmax = 128, 7
+    tab, nq, ng = make_spans([128 * 9000, 128 * 7000 + 66], group)
+    tab[1]["gof"] = tab[1]["pof"] + 8
+    tab["sref"] = [0.0086, 0.0091]
+    npar = nq + 8
+    hd = orc.digits(nq, 1, 20); hr = orc.int8(nq, 1, 21, -64, 64); hm8 = orc.int8(nq, 1, 22, -127, 127)
+    hv8 = orc.u8(nq, 1, 23, 0, 255)
+    hs = orc.uniform(ng, 1, 24, 0.5, 1.5) * f32(0.02 * 3 / 7)
+    hm8s = orc.uniform(ng, 1, 25, 0.5, 1.5) * f32(3e-3 / 127); hv8s = orc.uniform(ng, 1, 26, 0.5, 1.5) * f32(3e-3 / 255)
+    hP = np.zeros(npar, f32)
+    d, r, m8, v8, s, m8s, v8s = (dev(x) for x in (hd, hr, hm8, hv8, hs, hm8s, hv8s))
+    P = None if nopview else dev(hP)
+    sp = dev(tab)
+    stat = torch.zeros(4, dtype=torch.int64, device="cuda"); hstat = np.zeros(4, np.int64)
+    for t in range(1, 4):
+        hG = orc.normal(npar, 1, 30 + t, 1e-3)
+        bc1 = f32(1) - f32(0.9) ** f32(t); bc2 = f32(1) - f32(0.95) ** f32(t)
+        hp = (3e-4, 0.9, 0.95, 0.1, 1.0, None, float(f32(1) / bc1), float(f32(1) / np.sqrt(bc2)), 0, t, 1)
+        q.step(P, dev(hG), d, r, s, m8, m8s, v8, v8s, sp, 2, group, dmax, *hp, stat, 1, 0, ng)
+        orc.step(hP, hG, hd, hr, hs, hm8, hm8s, hv8, hv8s, tab, group, dmax, *hp, hstat, 1, 0, ng)
+    for got, want, nm in [(d, hd, "d"), (r, hr, "r"), (m8, hm8, "m8"), (v8, hv8, "v8"), (m8s, hm8s, "m8s"), (v8s, hv8s, "v8s")]:
+        assert beq(got, want), nm
+    if not nopview:
+        assert beq(P, hP)
+    assert np.array_equal(host(stat), hstat)
+
+
+def test_encode_render_vs_oracle_and_invariants(q, orc):
+    """4M weights: bytes equal the oracle's; rendered error <= 0.51 step; <= 15 levels per group
+    (cudalm.cu:10494-10523); render(encode(render(x))) is a fixed point."""
+    import torch
+    group, dmax = 128, 7
+    tab, nq, ng = make_spans([128 * 32768], group)
+    hP0 = orc.normal(nq, 2, 1, 0.02)
+    hP = hP0.copy(); hd = np.zeros(nq // 2, np.int8); hr = np.zeros(nq, np.int8); hs = np.zeros(ng, f32)
+    orc.encode(hP, hd, hr, hs, tab, group, dmax, 1, ng)
+    orc.render(hP, hd, hs, tab, group, 1, 0, ng)
+    P = dev(hP0); d = torch.zeros(nq // 2, dtype=torch.int8, device="cuda")
+    r = torch.zeros(nq, dtype=torch.int8, device="cuda"); s = torch.zeros(ng, device="cuda")
+    sp = dev(tab)
+    q.encode(P, d, r, s, sp, 1, group, dmax, 1, ng)
+    q.render(P, d, s, sp, 1, group, 1, 0, ng)
+    assert beq(d, hd) and beq(r, hr) and beq(s, hs) and beq(P, hP)
+    err = (P.view(ng, group) - dev(hP0).view(ng, group)).abs() / s[:, None]
+    assert float(err.max()) <= 0.51
+    d2 = torch.zeros_like(d); r2 = torch.zeros_like(r); s2 = torch.zeros_like(s); P2 = P.clone()
+    q.encode(P2, d2, r2, s2, sp, 1, group, dmax, 1, ng)
+    q.render(P2, d2, s2, sp, 1, group, 1, 0, ng)
+    assert float((P2 - P).abs().max()) <= float(s.max()) * 1e-6 and int(r2.abs().max()) <= 1
+
+
+def test_argument_errors(q):
+    import torch
+    x = torch.zeros(256, device="cuda")
+    with pytest.raises(pkg.QlmxError, match="group"):
+        q.render(x, x, x, x, 1, 1000, 1, 0, 1)
+    with pytest.raises(pkg.QlmxError, match="packed"):
+        q.encode(x, x, x, x, x, 1, 128, 127, 1, 1)
+    with pytest.raises(pkg.QlmxError, match="NULL"):
+        q.servo(None, x, x, x, 1, 128, 7, 0.1, 0.01, 1, 1)

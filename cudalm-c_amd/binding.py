@@ -18,6 +18,15 @@ class QlmxError(RuntimeError):
     pass
 
 
+class GemmProb(C.Structure):
+    """qlmx_gemm_prob of include/qlmx.h"""
+    _fields_ = [("A", c_vp), ("B", c_vp), ("C", c_vp), ("wq", c_u64), ("wg", c_u64), ("M", c_i), ("beta", c_f)]
+
+
+ACT_F32, ACT_BF16 = 0, 1
+MATH_F32, MATH_MFMA = 0, 1
+
+
 def lib_path():
     return os.path.join(HERE, "libqlmx.so")
 
@@ -25,8 +34,8 @@ def lib_path():
 def _ptr(x):
     if x is None:
         return None
-    if isinstance(x, int):
-        return x
+    if isinstance(x, (int, np.integer)):
+        return int(x)
     if hasattr(x, "data_ptr"):
         return x.data_ptr()
     if isinstance(x, np.ndarray):
@@ -58,6 +67,9 @@ SIGNATURES = {
     "qlmx_render": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_step": (c_i, _STEP),
     "qlmx_servo": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_f, c_f, c_i, c_i, c_vp]),
+    "qlmx_moe_gemm_nn": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_moe_gemm_tn": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_moe_gemm_nt": (c_i, [c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
 }
 
 
@@ -105,6 +117,24 @@ class Qlmx:
 
     def servo(self, d, r, s, sp, nspan, group, dmax, f_hi, f_lo, packed, ngrp, stream=None):
         self.call("qlmx_servo", d, r, s, sp, nspan, group, dmax, f_hi, f_lo, packed, ngrp, stream)
+
+    @staticmethod
+    def problems(items):
+        """items: iterable of dicts/tuples (A, B, C, wq, wg, M, beta) with tensors or ints as pointers"""
+        arr = (GemmProb * max(1, len(items)))()
+        for i, (A, B, Cc, wq, wg, M, beta) in enumerate(items):
+            arr[i].A, arr[i].B, arr[i].C = _ptr(A), _ptr(B), _ptr(Cc)
+            arr[i].wq, arr[i].wg, arr[i].M, arr[i].beta = int(wq), int(wg), int(M), float(beta)
+        return arr
+
+    def gemm_nn(self, d, s, group, probs, nprob, K, N, act=ACT_F32, math=MATH_F32, stream=None):
+        self.call("qlmx_moe_gemm_nn", d, s, group, C.addressof(probs), nprob, K, N, act, math, stream)
+
+    def gemm_tn(self, d, s, group, probs, nprob, K, N, act=ACT_F32, math=MATH_F32, stream=None):
+        self.call("qlmx_moe_gemm_tn", d, s, group, C.addressof(probs), nprob, K, N, act, math, stream)
+
+    def gemm_nt(self, probs, nprob, K, N, act=ACT_F32, math=MATH_F32, stream=None):
+        self.call("qlmx_moe_gemm_nt", C.addressof(probs), nprob, K, N, act, math, stream)
 
     def sync(self, stream=None):
         self.call("qlmx_sync", stream)

@@ -1,0 +1,44 @@
+/* qlmx_gemm.h -- shared plumbing of the grouped expert GEMMs: the device problem record, the
+ * pinned upload ring (the counterpart of the reference's mg_h/mg_d ring, cudalm.cu:3220-3241) and
+ * the weight-tile readers. */
+#ifndef QLMX_GEMM_H
+#define QLMX_GEMM_H
+#include "qlmx_dev.h"
+
+enum { GEMM_NN = 0, GEMM_TN = 1, GEMM_NT = 2 };
+
+struct DevProb {
+    const void *A; const void *B; float *C;
+    unsigned long long wq, wg;
+    int M; float beta;
+    int tile0;              /* first tile of this problem in the flattened tile list */
+    int tiles_n;            /* tiles along the output's second dimension             */
+};
+
+/* Copies `nprob` problems into the next ring slot, fills tile0/tiles_n with the given tile shape
+ * over an output of rows_of(p) x ncols, uploads the slot asynchronously on `stream`, and returns
+ * the device pointer and the total tile count. Slots are guarded by events, so a slot is never
+ * rewritten while a kernel launched with it may still read it. */
+struct ProbUpload { const DevProb *dev; int ntiles; int nprob; };
+int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K, int N,
+                         int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot);
+int qlmx_upload_done(int slot, hipStream_t stream);
+
+/* locate the problem owning flattened tile t (tile0 ascending) */
+__device__ __forceinline__ int qx_find_problem(const DevProb *pr, int nprob, int t){
+    int lo = 0, hi = nprob - 1;
+    while(lo < hi){
+        int mid = (lo + hi + 1) >> 1;
+        if(pr[mid].tile0 <= t) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+
+__device__ __forceinline__ float qx_bf16_to_f32(unsigned short h){ return __uint_as_float((uint32_t)h << 16); }
+/* round to nearest even, as cudalm.cu:334-338 */
+__device__ __forceinline__ unsigned short qx_f32_to_bf16(float f){
+    uint32_t x = __float_as_uint(f);
+    return (unsigned short)((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16);
+}
+
+#endif

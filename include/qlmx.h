@@ -97,6 +97,47 @@ int qlmx_servo(signed char *d, signed char *r, float *s,
                const qlmx_span *sp, int nspan, int group, int dmax,
                float f_hi, float f_lo, int packed, int ngrp, void *stream);
 
+/* =====================================================================================
+ * Expert GEMMs with the dequantisation fused in
+ *
+ * The reference renders P = s*digit once per step and hands fp32 slices of P to its GEMM wrappers
+ * (row-major):  mg_ab   C[M,N]  = A[M,K] @ B[K,N]             cudalm.cu:3247-3249 (g_ab 3133)
+ *               mg_abt_b C[M,N] = A[M,K] @ B[N,K]^T + beta*C   cudalm.cu:3250-3253 (g_abt_b 3174)
+ *               mg_atb  C[K,N] += A[M,K]^T @ B[M,N]            cudalm.cu:3254-3256 (g_atb 3190)
+ * queued per expert and issued together by mg_flush (cudalm.cu:3230-3243). Here the weight operand
+ * is named by its position in the packed digits and scales instead of by a pointer into P, and one
+ * call takes the whole queue: an array of problems that share K and N. Results equal the
+ * reference's P = s*digit -> fp32 SGEMM semantics to rounding (fp32 math) or to bf16-MFMA
+ * accumulation order (MFMA math); C is always fp32.
+ * ===================================================================================== */
+#define QLMX_ACT_F32   0     /* activation operands are fp32                         */
+#define QLMX_ACT_BF16  1     /* activation operands are bf16 (high half of an fp32)  */
+#define QLMX_MATH_F32  0     /* fp32 FMA on the vector ALU                           */
+#define QLMX_MATH_MFMA 1     /* bf16 MFMA, fp32 accumulate                           */
+#define QLMX_MAX_PROBLEMS 1024   /* like MG_MAXP, cudalm.cu:3214 */
+
+typedef struct qlmx_gemm_prob {
+    const void *A;           /* device: nn/tn [M,K]; nt [M,K] (read transposed)                  */
+    const void *B;           /* device: nt only, [M,N] activation/gradient rows; else NULL      */
+    float      *C;           /* device: nn/tn [M,N]; nt [K,N]                                    */
+    unsigned long long wq;   /* nn/tn: element offset of the weight matrix in the digit array    */
+    unsigned long long wg;   /* nn/tn: index of the matrix's first scale group                   */
+    int   M;                 /* rows of A (0 is allowed and skipped)                             */
+    float beta;              /* tn: 0 or 1. nn is always beta=0, nt always accumulates           */
+} qlmx_gemm_prob;
+
+/* nn: weights [K,N] row-major, scale groups run along N (N % group == 0). */
+int qlmx_moe_gemm_nn(const signed char *d, const float *s, int group,
+                     const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
+                     int act_dtype, int math, void *stream);
+/* tn: weights [N,K] row-major, scale groups run along K (K % group == 0). */
+int qlmx_moe_gemm_tn(const signed char *d, const float *s, int group,
+                     const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
+                     int act_dtype, int math, void *stream);
+/* nt: no weight operand; both inputs are activations, C accumulates in fp32. */
+int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
+                     int act_dtype, int math, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,174 @@
+"""GPU parity of the grouped expert GEMMs with the dequantisation fused in, against the CPU oracle's
+P = s*digit -> fp32 GEMM on the same seeded inputs. Tolerance: 1e-3 relative L2 (the reference's
+relerr, cudalm.cu:9842) for the bf16-MFMA kernels, 1e-5 for the fp32 kernels."""
+import numpy as np
+import pytest
+
+from __graft_entry__ import load_package
+from oracle.binding import make_spans
+
+pkg = load_package()
+f32 = np.float32
+pytestmark = pytest.mark.gpu
+TOL_MFMA = 1e-3
+TOL_F32 = 1e-5
+
+
+@pytest.fixture(scope="module")
+def q():
+    return pkg.load()
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def to_bf16_bits(t):
+    """fp32 torch tensor holding bf16-representable values -> uint16 bit pattern tensor"""
+    import torch
+    return (t.view(torch.int32) >> 16).to(torch.int16)
+
+
+def make_weights(orc, seed, E, rows, cols, group=128):
+    """E expert matrices [rows, cols] encoded by the oracle; returns (d, s, rendered fp32 view)"""
+    n = E * rows * cols
+    tab, nq, ng = make_spans([n], group)
+    P = orc.normal(n, seed, 1, 0.02)
+    d = np.zeros(n // 2, np.int8); r = np.zeros(n, np.int8); s = np.zeros(ng, f32)
+    orc.encode(P, d, r, s, tab, group, 7, 1, ng)
+    orc.render(P, d, s, tab, group, 1, 0, ng)
+    return d, s, P
+
+
+def zipf_rows(total, E, seed):
+    rng = np.random.default_rng(seed)
+    p = (np.arange(E) + 1.0) ** -1.1
+    p /= p.sum()
+    cnt = rng.multinomial(total, p)
+    return [int(c) for c in cnt]
+
+
+def run_case(q, orc, mode, E, rowsM, K, N, act, math, seed=0, beta=0.0, group=128):
+    """One grouped call over E experts with the given row counts. Returns (got list, want list)."""
+    import torch
+    tot = sum(rowsM)
+    off = np.concatenate([[0], np.cumsum(rowsM)]).astype(int)
+    bf = act == pkg.ACT_BF16
+    if mode == "nt":
+        A = orc.normal(tot * K, seed, 10); B = orc.normal(tot * N, seed, 11)
+        if bf:
+            A = orc.bf16_round(A); B = orc.bf16_round(B)
+        C0 = orc.normal(E * K * N, seed, 12, 0.1)
+        dA, dB, dC = dev(A), dev(B), dev(C0.copy())
+        pa = to_bf16_bits(dA) if bf else dA
+        pb = to_bf16_bits(dB) if bf else dB
+        esz = 2 if bf else 4
+        items = [(pa.data_ptr() + off[e] * K * esz, pb.data_ptr() + off[e] * N * esz, dC.data_ptr() + e * K * N * 4, 0, 0, rowsM[e], 1.0)
+                 for e in range(E)]
+        pr = q.problems(items)
+        q.gemm_nt(pr, E, K, N, act, math)
+        torch.cuda.synchronize()
+        want = C0.copy()
+        for e in range(E):
+            if rowsM[e]:
+                orc.gemm_nt(A[off[e] * K:], B[off[e] * N:], want[e * K * N:(e + 1) * K * N], rowsM[e], K, N)
+        return dC.cpu().numpy(), want
+    wr, wc = (K, N) if mode == "nn" else (N, K)
+    d, s, P = make_weights(orc, seed, E, wr, wc, group)
+    A = orc.normal(tot * K, seed, 10)
+    if bf:
+        A = orc.bf16_round(A)
+    C0 = orc.normal(tot * N, seed, 12)
+    dA, dC, dd, ds = dev(A), dev(C0.copy()), dev(d), dev(s)
+    pa = to_bf16_bits(dA) if bf else dA
+    esz = 2 if bf else 4
+    items = [(pa.data_ptr() + off[e] * K * esz, None, dC.data_ptr() + off[e] * N * 4, e * wr * wc, e * wr * wc // group,
+              rowsM[e], beta) for e in range(E)]
+    pr = q.problems(items)
+    (q.gemm_nn if mode == "nn" else q.gemm_tn)(dd, ds, group, pr, E, K, N, act, math)
+    torch.cuda.synchronize()
+    want = C0.copy()
+    for e in range(E):
+        if not rowsM[e]:
+            continue
+        w = P[e * wr * wc:(e + 1) * wr * wc]
+        if mode == "nn":
+            orc.gemm_nn(A[off[e] * K:], w, want[off[e] * N:off[e + 1] * N], rowsM[e], K, N)
+        else:
+            orc.gemm_tn(A[off[e] * K:], w, want[off[e] * N:off[e + 1] * N], rowsM[e], K, N, beta)
+    return dC.cpu().numpy(), want
+
+
+# ------------------------------------------------------------------ fp32 vector-ALU kernels
+@pytest.mark.parametrize("mode", ["nn", "tn", "nt"])
+def test_f32_ragged_small(q, orc, mode):
+    """Ragged shapes incl. an empty expert and rows not a multiple of any tile (cudalm.cu:9919-9946 style)."""
+    K, N = (128, 256) if mode != "tn" else (256, 128)
+    got, want = run_case(q, orc, mode, 4, [67, 0, 5, 130], K, N, pkg.ACT_F32, pkg.MATH_F32, seed=3,
+                         beta=1.0 if mode == "tn" else 0.0)
+    assert orc.relerr(got, want) < TOL_F32
+
+
+def test_f32_c1_single_expert(q, orc):
+    """BASELINE config 1: X fp32 [1024,512], 512->1536 up and 1536->512 down; forward, dgrad, wgrad."""
+    for (K, N) in [(512, 1536), (1536, 512)]:
+        for mode in ["nn", "tn", "nt"]:
+            kk, nn = (K, N) if mode != "tn" else (N, K)
+            got, want = run_case(q, orc, mode, 1, [1024], kk, nn, pkg.ACT_F32, pkg.MATH_F32, seed=0)
+            assert orc.relerr(got, want) < TOL_F32, (mode, K, N)
+
+
+def test_f32_bf16_acts_and_group64(q, orc):
+    got, want = run_case(q, orc, "nn", 3, [40, 1, 77], 192, 128, pkg.ACT_BF16, pkg.MATH_F32, seed=5, group=64)
+    assert orc.relerr(got, want) < TOL_F32
+    got, want = run_case(q, orc, "tn", 3, [40, 1, 77], 128, 192, pkg.ACT_BF16, pkg.MATH_F32, seed=6, group=64)
+    assert orc.relerr(got, want) < TOL_F32
+
+
+# ------------------------------------------------------------------ bf16 MFMA kernels
+@pytest.mark.parametrize("mode", ["nn", "tn", "nt"])
+def test_mfma_grouped_zipf_small(q, orc, mode):
+    """8 experts, Zipf row counts incl. tiny and empty experts, D=256 F=384."""
+    rows = zipf_rows(1500, 8, 1)
+    rows[5] = 0
+    rows[6] = 1
+    K, N = {"nn": (256, 384), "tn": (384, 256), "nt": (256, 384)}[mode]
+    got, want = run_case(q, orc, mode, 8, rows, K, N, pkg.ACT_BF16, pkg.MATH_MFMA, seed=2,
+                         beta=1.0 if mode == "tn" else 0.0)
+    err = orc.relerr(got, want)
+    assert err < TOL_MFMA, err
+
+
+@pytest.mark.parametrize("mode,K,N", [("nn", 768, 2048), ("nn", 2048, 768), ("tn", 768, 2048), ("tn", 2048, 768),
+                                      ("nt", 768, 2048), ("nt", 2048, 768)])
+def test_mfma_layer_shapes(q, orc, mode, K, N):
+    """The 32-expert D=768 F=2048 layer's GEMM shapes on a 4-expert slice with Zipf rows (the CPU
+    oracle finishes these in seconds)."""
+    rows = zipf_rows(1100, 4, 7)
+    got, want = run_case(q, orc, mode, 4, rows, K, N, pkg.ACT_BF16, pkg.MATH_MFMA, seed=4)
+    err = orc.relerr(got, want)
+    assert err < TOL_MFMA, err
+
+
+def test_mfma_f32_acts_are_rounded_once(q, orc):
+    """fp32 activations on the MFMA path are rounded to bf16 on load: equal to feeding pre-rounded ones."""
+    import torch
+    got32, _ = run_case(q, orc, "tn", 2, [100, 200], 256, 128, pkg.ACT_F32, pkg.MATH_MFMA, seed=9)
+    # same inputs, rounded on the host first
+    E, K, N = 2, 256, 128
+    d, s, P = make_weights(orc, 9, E, N, K)
+    A = orc.bf16_round(orc.normal(300 * K, 9, 10))
+    want = np.zeros(300 * N, f32)
+    off = [0, 100, 300]
+    for e in range(E):
+        orc.gemm_tn(A[off[e] * K:], P[e * N * K:(e + 1) * N * K], want[off[e] * N:off[e + 1] * N], off[e + 1] - off[e], K, N, 0.0)
+    assert orc.relerr(got32, want) < TOL_MFMA
+
+
+def test_mfma_rejects_unsupported_shapes(q):
+    import torch
+    x = torch.zeros(4096, device="cuda")
+    pr = q.problems([(x, None, x, 0, 0, 4, 0.0)])
+    with pytest.raises(pkg.QlmxError, match="multiple"):
+        q.gemm_nn(x, x, 128, pr, 1, 32, 100, pkg.ACT_F32, pkg.MATH_MFMA)

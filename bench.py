@@ -58,6 +58,175 @@ def timed(torch, fn, steps, warmup):
     return {"wall_ms": wall, "event_ms_avg": sum(per) / len(per), "event_ms_med": per[len(per) // 2], "event_ms_min": per[0]}
 
 
+
+# --------------------------------------------------------------------------------------------- train
+def zipf_counts(E, tokens, topk, seed=0):
+    """Per-expert row counts when every token draws `topk` distinct experts with p_e ~ (e+1)^-1.1
+    (Gumbel top-k = sampling without replacement)."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    logp = -1.1 * np.log(np.arange(E) + 1.0)
+    keys = logp[None, :] + rng.gumbel(size=(tokens, E))
+    top = np.argsort(-keys, axis=1)[:, :topk]
+    return np.bincount(top.ravel(), minlength=E).astype(int)
+
+
+def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2):
+    from cudalm_c_amd.binding import ACT_BF16, MATH_MFMA
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev); g.manual_seed(0)
+    cnt = zipf_counts(E, tokens, topk)
+    rows = int(cnt.sum())
+    off = [0]
+    for c in cnt:
+        off.append(off[-1] + int(c))
+    group = 128
+    nw = E * D * F
+
+    def packed():
+        b = torch.randint(0, 256, (nw // 2,), dtype=torch.int16, device=dev, generator=g).to(torch.uint8)
+        lo = b & 15; hi = b >> 4
+        lo = torch.where(lo == 8, torch.zeros_like(lo), lo); hi = torch.where(hi == 8, torch.zeros_like(hi), hi)
+        return (lo | (hi << 4)).view(torch.int8)
+
+    # one digit array holding w1 | w3 | w2 back to back, like consecutive spans of a layer
+    d = torch.cat([packed(), packed(), packed()])
+    s = (0.02 * 3 / 7) * (0.5 + torch.rand(3 * nw // group, device=dev, generator=g))
+    o1, o3, o2 = 0, nw, 2 * nw
+
+    def bf16(n, scale=1.0):
+        return (scale * torch.randn(n, device=dev, generator=g)).to(torch.bfloat16)
+
+    Xp, ap, dyp = bf16(rows * D), bf16(rows * F), bf16(rows * D)
+    dgp, dup = bf16(rows * F), bf16(rows * F)
+    gp = torch.empty(rows * F, device=dev); up = torch.empty(rows * F, device=dev); yp = torch.empty(rows * D, device=dev)
+    dap = torch.empty(rows * F, device=dev); dXp = torch.empty(rows * D, device=dev)
+    G = torch.zeros(3 * nw, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def probs(A, a_w, B, b_w, Cm, c_w, wbase, per_expert_c=False):
+        items = []
+        for e in range(E):
+            m = int(cnt[e])
+            items.append((A.data_ptr() + off[e] * a_w * 2, (B.data_ptr() + off[e] * b_w * 2) if B is not None else None,
+                          (Cm.data_ptr() + (wbase + e * D * F) * 4) if per_expert_c else (Cm.data_ptr() + off[e] * c_w * 4),
+                          wbase + e * D * F, (wbase + e * D * F) // group, m, 0.0))
+        return items
+
+    P = q.problems
+    p_w13 = P(probs(Xp, D, None, 0, gp, F, o1) + probs(Xp, D, None, 0, up, F, o3))
+    p_w2 = P(probs(ap, F, None, 0, yp, D, o2))
+    p_d2 = P(probs(dyp, D, None, 0, dap, F, o2))
+    p_d1 = P(probs(dgp, F, None, 0, dXp, D, o1))
+    it3 = probs(dup, F, None, 0, dXp, D, o3)
+    p_d3 = P([(a, b, c, wq, wg, m, 1.0) for (a, b, c, wq, wg, m, _) in it3])
+    p_g2 = P(probs(ap, F, dyp, D, G, 0, o2, True))
+    p_g13 = P(probs(Xp, D, dgp, F, G, 0, o1, True) + probs(Xp, D, dup, F, G, 0, o3, True))
+    calls = [
+        ("fwd w1,w3 (nn)", lambda: q.gemm_nn(d, s, group, p_w13, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream), 2),
+        ("fwd w2 (nn)", lambda: q.gemm_nn(d, s, group, p_w2, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
+        ("dgrad w2 (tn)", lambda: q.gemm_tn(d, s, group, p_d2, E, D, F, ACT_BF16, MATH_MFMA, stream), 1),
+        ("dgrad w1 (tn)", lambda: q.gemm_tn(d, s, group, p_d1, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
+        ("dgrad w3 (tn,+=)", lambda: q.gemm_tn(d, s, group, p_d3, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
+        ("wgrad w2 (nt)", lambda: q.gemm_nt(p_g2, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
+        ("wgrad w1,w3 (nt)", lambda: q.gemm_nt(p_g13, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream), 2),
+    ]
+    unit = 2.0 * rows * D * F            # flops of one expert GEMM over all rows
+
+    def step():
+        for _, fn, _n in calls:
+            fn()
+
+    tm = timed(torch, step, args.steps, args.warmup)
+    per = {}
+    for name, fn, ng in calls:
+        t1 = timed(torch, fn, max(5, args.steps // 2), 2)
+        per[name] = {"ms": t1["event_ms_avg"], "tflops": ng * unit / (t1["event_ms_avg"] * 1e-3) / 1e12}
+    flops = 9 * unit
+    tf = flops / (tm["event_ms_avg"] * 1e-3) / 1e12
+    dom = max(per, key=lambda k: per[k]["ms"])
+    return {
+        "workload": "C3 train layer: E=%d top-%d D=%d F=%d, %d bf16 tokens -> %d expert rows, Zipf(1.1) load (max %d, min %d rows); "
+                    "fwd+dgrad+wgrad = 9 grouped GEMMs in 7 launches" % (E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min())),
+        "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tm["wall_ms"], "dtype": "bf16",
+        "kernel_ms": tm, "per_launch": per, "gflop_per_step": flops / 1e9,
+        "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": None, "kernel": "k_gemm_mfma<nn|tn|nt> (all 7 launches; slowest: %s)" % dom,
+                     "note": "algorithmic flops only; the forward issues two MFMAs per product (bf16 hi+lo weight split)"},
+    }
+
+
+# --------------------------------------------------------------------------------------------- decode
+def bench_decode(torch, q, args, E=32, D=768, F=2048, topk=2, layers=8):
+    """8 distinct layers (8 x 80 MB of packed weights > the 256 MB last-level cache) decoded back to
+    back for T = 1, 4, 16 tokens; bytes counted = digits + scales of the distinct experts hit."""
+    import numpy as np
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev); g.manual_seed(0)
+    group = 128
+    nw = E * D * F
+    per_expert = 3 * D * F // 2 + 3 * D * F // group * 4
+
+    def packed(n):
+        b = torch.randint(0, 256, (n // 2,), dtype=torch.int16, device=dev, generator=g).to(torch.uint8)
+        lo = b & 15; hi = b >> 4
+        lo = torch.where(lo == 8, torch.zeros_like(lo), lo); hi = torch.where(hi == 8, torch.zeros_like(hi), hi)
+        return (lo | (hi << 4)).view(torch.int8)
+
+    ds = [packed(3 * nw) for _ in range(layers)]
+    ss = [(0.02 * 3 / 7) * (0.5 + torch.rand(3 * nw // group, device=dev, generator=g)) for _ in range(layers)]
+    stream = torch.cuda.current_stream().cuda_stream
+    out_all = {}
+    for T in (1, 4, 16):
+        x = torch.randn(T * D, device=dev, generator=g)
+        asn, gates, hits = [], [], 0
+        for l in range(layers):
+            logits = torch.randn(T, E, device=dev, generator=g)
+            p = torch.softmax(logits, dim=1)
+            top = torch.topk(p, topk, dim=1)
+            a = top.indices.t().contiguous().to(torch.int32)          # pass-major [K][T]
+            asn.append(a.view(-1)); gates.append(top.values.t().contiguous().view(-1))
+            hits += int(torch.unique(a).numel())
+        out = torch.zeros(T * D, device=dev)
+
+        def step():
+            for l in range(layers):
+                q.decode_forward(x, asn[l], gates[l], out, ds[l], ss[l], group, 0, nw, 2 * nw, T, topk, E, D, F, stream)
+
+        tm = timed(torch, step, args.steps, args.warmup)
+        res = {"ms_8_layers": tm["event_ms_avg"], "distinct_expert_hits": hits, "bytes": hits * per_expert,
+               "gbs": hits * per_expert / (tm["event_ms_avg"] * 1e-3) / 1e9}
+        # the same 8-layer sequence replayed as one HIP graph (no launch gaps from the host)
+        try:
+            gr = torch.cuda.CUDAGraph()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                st2 = side.cuda_stream
+                for l in range(layers):
+                    q.decode_forward(x, asn[l], gates[l], out, ds[l], ss[l], group, 0, nw, 2 * nw, T, topk, E, D, F, st2)
+                side.synchronize()
+                with torch.cuda.graph(gr, stream=side):
+                    for l in range(layers):
+                        q.decode_forward(x, asn[l], gates[l], out, ds[l], ss[l], group, 0, nw, 2 * nw, T, topk, E, D, F, st2)
+            torch.cuda.current_stream().wait_stream(side)
+            tg = timed(torch, gr.replay, args.steps, args.warmup)
+            res["graph_ms_8_layers"] = tg["event_ms_avg"]
+            res["graph_gbs"] = hits * per_expert / (tg["event_ms_avg"] * 1e-3) / 1e9
+        except Exception as e:      # graph capture is an extra; the eager figure stands on its own
+            res["graph_error"] = str(e)[:200]
+        out_all["T%d" % T] = res
+    head = out_all["T16"]
+    gbs = max(head["gbs"], head.get("graph_gbs", 0.0))
+    return {
+        "workload": "C2 decode: %d layers x (E=%d top-%d D=%d F=%d), T=16 tokens per step (T=1,4 listed beside); fused group+w1|w3+SwiGLU, w2, combine"
+                    % (layers, E, topk, D, F),
+        "metric": "QLM expert dequant-GEMV GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": min(head["ms_8_layers"], head.get("graph_ms_8_layers", 1e9)),
+        "dtype": "u8+f32", "by_tokens": out_all, "bytes_per_expert_hit": per_expert,
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "k_qlmx_gemv<swiglu> + k_qlmx_gemv<store> (whole 8-layer sequence incl. group/combine kernels)"},
+    }
+
 # --------------------------------------------------------------------------------------------- adamw
 def bench_adamw(torch, q, args):
     import numpy as np
@@ -151,7 +320,7 @@ def main():
     q = pkg.load()           # raises if libqlmx.so is missing or no gfx950 device
     torch.cuda.set_device(0)
     want = ["train", "decode", "adamw"] if args.workload == "all" else [args.workload]
-    runners = {"adamw": bench_adamw}
+    runners = {"adamw": bench_adamw, "train": bench_train, "decode": bench_decode}
     results = {}
     for w in want:
         if w in runners:

@@ -70,6 +70,7 @@ SIGNATURES = {
     "qlmx_moe_gemm_nn": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_tn": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_nt": (c_i, [c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_moe_decode_forward": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
 }
 
 
@@ -135,6 +136,9 @@ class Qlmx:
 
     def gemm_nt(self, probs, nprob, K, N, act=ACT_F32, math=MATH_F32, stream=None):
         self.call("qlmx_moe_gemm_nt", C.addressof(probs), nprob, K, N, act, math, stream)
+
+    def decode_forward(self, x, assign, gate, out, d, s, group, w1q, w3q, w2q, T, K, E, D, F, stream=None):
+        self.call("qlmx_moe_decode_forward", x, assign, gate, out, d, s, group, w1q, w3q, w2q, T, K, E, D, F, stream)
 
     def sync(self, stream=None):
         self.call("qlmx_sync", stream)

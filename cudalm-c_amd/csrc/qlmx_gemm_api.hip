@@ -4,6 +4,8 @@
 
 int qlmx_gemm_f32_dispatch(int mode, const signed char *d, const float *s, int group,
                            const qlmx_gemm_prob *probs, int nprob, int K, int N, int act_dtype, hipStream_t st);
+int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob,
+                          int K, int N, hipStream_t st);
 int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int group,
                             const qlmx_gemm_prob *probs, int nprob, int K, int N, int act_dtype, hipStream_t st);
 
@@ -23,6 +25,12 @@ static int gemm_entry(const char *who, int mode, const signed char *d, const flo
     }
     if(math == QLMX_MATH_MFMA)
         return qlmx_gemm_mfma_dispatch(mode, d, s, group, probs, nprob, K, N, act_dtype, (hipStream_t)stream);
+    if(mode == GEMM_NN && act_dtype == QLMX_ACT_F32 && N % 32 == 0 && group % 32 == 0 && ((uintptr_t)d & 15) == 0){
+        /* every problem has a few rows only: stream the weights once (decode shape) */
+        bool small = nprob > 0;
+        for(int i = 0; i < nprob && small; i++) small = probs[i].M <= 4 && probs[i].wq % 32 == 0;
+        if(small) return qlmx_gemv_nn_dispatch(d, s, group, probs, nprob, K, N, (hipStream_t)stream);
+    }
     return qlmx_gemm_f32_dispatch(mode, d, s, group, probs, nprob, K, N, act_dtype, (hipStream_t)stream);
 }
 

@@ -138,6 +138,30 @@ int qlmx_moe_gemm_tn(const signed char *d, const float *s, int group,
 int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
                      int act_dtype, int math, void *stream);
 
+/* =====================================================================================
+ * Decode-shaped expert FFN (a few tokens per step)
+ *
+ * The reference's decoder runs the training forward on N = batch rows (dec_step, cudalm.cu:7163-7204
+ * -> moe_forward 7193), so each expert GEMM has 0..few rows and the work is reading the experts'
+ * packed weights once. qlmx_moe_gemm_nn with QLMX_MATH_F32 already takes a streaming GEMV path when
+ * every problem has at most 4 rows (the counterpart of the reference's R<=4 path, cpu_rt.h:233-258).
+ * qlmx_moe_decode_forward fuses the whole expert part of moe_forward for such batches: it groups
+ * the (pass, token) pairs by expert on the device (no host round trip, unlike cudalm.cu:3576-3602),
+ * streams w1|w3 with the SwiGLU applied on the fly, streams w2, and adds gate*y into `out` in pass
+ * order (cudalm.cu:4193-4228 semantics: out[n] += sum_k gate[k][n] * FFN_{assign[k][n]}(x[n])).
+ *   x      [T, D] fp32                    assign [K][T] int32 (pass-major)   gate [K][T] fp32
+ *   out    [T, D] fp32, accumulated into (the caller seeds it with the residual)
+ *   w1q/w3q/w2q: element offsets of expert 0's matrices in d; expert e adds e*D*F. All multiples of
+ *   `group`; w1, w3 are [D,F] row-major and w2 is [F,D] row-major (cudalm.cu:263-265). The scale of
+ *   element q is s[q / group] (every span a multiple of the group, true of all reference presets).
+ * Limits: K*T <= 64 pairs, D and F multiples of 32 and <= 8192. Uses a library-owned workspace that
+ * is (re)allocated on first use or growth; calls on different streams must not overlap.
+ * ===================================================================================== */
+int qlmx_moe_decode_forward(const float *x, const int *assign, const float *gate, float *out,
+                            const signed char *d, const float *s, int group,
+                            unsigned long long w1q, unsigned long long w3q, unsigned long long w2q,
+                            int T, int K, int E, int D, int F, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

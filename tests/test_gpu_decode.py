@@ -1,0 +1,122 @@
+"""GPU parity of the decode-shaped (few-token) expert path: the streaming GEMV behind
+qlmx_moe_gemm_nn and the fused qlmx_moe_decode_forward, against the CPU oracle's rendered-weights
+fp32 layer (moe_forward call order, cudalm.cu:4193-4228). fp32 math: tolerance 1e-3 relative L2 as
+stated for matmul outputs, observed ~1e-6; routing indices come from the oracle's router and are
+consumed as given."""
+import numpy as np
+import pytest
+
+from __graft_entry__ import load_package
+from oracle.binding import make_spans
+
+pkg = load_package()
+f32 = np.float32
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def q():
+    return pkg.load()
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def encode_layer(orc, seed, E, D, F, group=128):
+    """w1 | w3 | w2 back to back in one digit array (three consecutive spans)."""
+    n = E * D * F
+    tab, nq, ng = make_spans([n, n, n], group)
+    P = orc.normal(nq, seed, 1, 0.02)
+    d = np.zeros(nq // 2, np.int8); r = np.zeros(nq, np.int8); s = np.zeros(ng, f32)
+    orc.encode(P, d, r, s, tab, group, 7, 1, ng)
+    orc.render(P, d, s, tab, group, 1, 0, ng)
+    return d, s, P, n
+
+
+@pytest.mark.parametrize("K,N", [(768, 2048), (2048, 768), (512, 1536)])
+def test_gemv_small_rows_vs_oracle(q, orc, K, N):
+    """qlmx_moe_gemm_nn with 1..4 rows per expert takes the streaming path; an empty expert is skipped."""
+    import torch
+    E = 5
+    rows = [1, 4, 0, 2, 3]
+    n = E * K * N
+    tab, nq, ng = make_spans([n], 128)
+    P = orc.normal(n, 3, 1, 0.02)
+    d = np.zeros(n // 2, np.int8); r = np.zeros(n, np.int8); s = np.zeros(ng, f32)
+    orc.encode(P, d, r, s, tab, 128, 7, 1, ng)
+    orc.render(P, d, s, tab, 128, 1, 0, ng)
+    off = np.concatenate([[0], np.cumsum(rows)])
+    A = orc.normal(int(off[-1]) * K, 3, 2)
+    dA, dC, dd, ds = dev(A), torch.full((int(off[-1]) * N,), 7.0, device="cuda"), dev(d), dev(s)
+    items = [(dA.data_ptr() + int(off[e]) * K * 4, None, dC.data_ptr() + int(off[e]) * N * 4, e * K * N, e * K * N // 128, rows[e], 0.0)
+             for e in range(E)]
+    q.gemm_nn(dd, ds, 128, q.problems(items), E, K, N, pkg.ACT_F32, pkg.MATH_F32)
+    torch.cuda.synchronize()
+    want = np.zeros(int(off[-1]) * N, f32)
+    for e in range(E):
+        if rows[e]:
+            orc.gemm_nn(A[off[e] * K:], P[e * K * N:(e + 1) * K * N], want[off[e] * N:off[e + 1] * N], rows[e], K, N)
+    err = orc.relerr(dC.cpu().numpy(), want)
+    assert err < 1e-5, err
+    # a second call reuses the tickets and scratch: same answer
+    dC.fill_(0)
+    q.gemm_nn(dd, ds, 128, q.problems(items), E, K, N, pkg.ACT_F32, pkg.MATH_F32)
+    torch.cuda.synchronize()
+    assert orc.relerr(dC.cpu().numpy(), want) < 1e-5
+
+
+@pytest.mark.parametrize("T,E,D,F,K", [(1, 32, 768, 2048, 2), (4, 8, 768, 2048, 2), (16, 8, 768, 2048, 2),
+                                       (16, 4, 256, 384, 4), (5, 3, 128, 256, 1)])
+def test_decode_forward_vs_oracle_layer(q, orc, T, E, D, F, K):
+    import torch
+    d, s, P, n = encode_layer(orc, 11 + T, E, D, F)
+    x = orc.normal(T * D, 11, 2)
+    rt = orc.normal(T * E, 11, 3)
+    pr = np.zeros(T * E, f32); asn = np.zeros(K * T, np.int32); gate = np.zeros(K * T, f32)
+    orc.router_topk(rt, pr, asn, gate, T, E, K)
+    res = orc.normal(T * D, 11, 4)                      # residual the layer accumulates into
+    want = res.copy()
+    rc, ws = orc.moe_forward(x, P[:n], P[n:2 * n], P[2 * n:], asn, gate, want, T, D, F, E, K)
+    orc.moe_ws_free(ws)
+    assert rc == 0
+    out = dev(res)
+    dd, ds = dev(d), dev(s)
+    q.decode_forward(dev(x), dev(asn), dev(gate), out, dd, ds, 128, 0, n, 2 * n, T, K, E, D, F)
+    torch.cuda.synchronize()
+    err = orc.relerr(out.cpu().numpy() - res, want - res)
+    assert err < 1e-3, err
+    assert err < 2e-5, err          # fp32 math: only summation order and the libm exp differ
+    # run-to-run determinism: slice order, not arrival order, fixes the sums
+    out2 = dev(res)
+    q.decode_forward(dev(x), dev(asn), dev(gate), out2, dd, ds, 128, 0, n, 2 * n, T, K, E, D, F)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+
+
+def test_decode_all_tokens_one_expert(q, orc):
+    """Collision case: 16 tokens on the same two experts -> problems are cut into row pairs."""
+    import torch
+    T, E, D, F, K = 16, 4, 256, 512, 2
+    d, s, P, n = encode_layer(orc, 5, E, D, F)
+    x = orc.normal(T * D, 5, 2)
+    asn = np.concatenate([np.full(T, 2), np.full(T, 0)]).astype(np.int32)
+    gate = orc.uniform(K * T, 5, 3, 0.1, 0.6)
+    want = np.zeros(T * D, f32)
+    rc, ws = orc.moe_forward(x, P[:n], P[n:2 * n], P[2 * n:], asn, gate, want, T, D, F, E, K)
+    orc.moe_ws_free(ws)
+    out = torch.zeros(T * D, device="cuda")
+    q.decode_forward(dev(x), dev(asn), dev(gate), out, dev(d), dev(s), 128, 0, n, 2 * n, T, K, E, D, F)
+    torch.cuda.synchronize()
+    assert orc.relerr(out.cpu().numpy(), want) < 2e-5
+
+
+def test_decode_limits(q):
+    import torch
+    z = torch.zeros(65536, device="cuda")
+    zi = torch.zeros(256, dtype=torch.int32, device="cuda")
+    with pytest.raises(pkg.QlmxError, match="pairs"):
+        q.decode_forward(z, zi, z, z, z, z, 128, 0, 0, 0, 64, 2, 4, 128, 128)
+    with pytest.raises(pkg.QlmxError, match="multiples of 32"):
+        q.decode_forward(z, zi, z, z, z, z, 128, 0, 0, 0, 2, 2, 4, 100, 128)

@@ -54,6 +54,9 @@ def build_all(jobs=8):
     if os.path.exists(host_src):
         _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-I", os.path.join(HERE, "..", "include"),
               host_src, "-o", HOST_LIB, "-L", HERE, "-lqlmx", "-Wl,-rpath,$ORIGIN"])
+        _run(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-I", os.path.join(HERE, "..", "include"),
+              os.path.join(HERE, "host", "selftest.cpp"), "-o", os.path.join(HERE, "qlm_selftest"),
+              "-L", HERE, "-lqlmx_host", "-lqlmx", "-Wl,-rpath,$ORIGIN"])
     return LIB
 
 

@@ -1,0 +1,74 @@
+/* qlm_host.h -- C++ host mirror of the reference's QLM call surface on top of the C ABI (include/qlmx.h).
+ *
+ * Same names, argument order and error behaviour as the reference's host code so that cudalm.cu's
+ * call sites keep compiling against it: the Qlm / QSpanD types (qlm.cuh:30-58), qlm_add_span,
+ * qlm_gpu_init, qlm_gpu_render, qlm_render_layer, qlm_step_launch, qlm_gpu_update, qlm_save /
+ * qlm_load (qlm.cuh:448-541, 577-591, 377-397, 702-788; cudalm.cu:6082-6103) and the grouped expert
+ * GEMM queue mg_ab / mg_abt / mg_abt_b / mg_atb / mg_flush (cudalm.cu:3204-3256). Failures print
+ * and exit(1) like ck()/ckb() (cudalm.cu:147-152).
+ *
+ * What differs, because the weights are never rendered for the GEMMs:
+ *   - qlm_gpu_init takes the span list explicitly (the reference derives it from its Cfg/Off model
+ *     description, qlm.cuh:479-490, which is outside this path);
+ *   - the GEMM wrappers take the weight operand as a pointer INTO the fp32 view `P`, exactly as the
+ *     reference call sites pass it (P + offset), but only its offset is used: mg_bind() registers
+ *     the Qlm and the base of P, and the offset is mapped through the span table to digits + scales.
+ *     P itself may be unallocated (P rendering is optional, see qlm_gpu_update);
+ *   - the float spans' bf16 AdamW (k_adamw, cudalm.cu:6092-6096) is not part of this path; the
+ *     table of float gaps is still built so a caller can run its own update over them.
+ */
+#ifndef QLM_HOST_H
+#define QLM_HOST_H
+#include <stddef.h>
+#include <stdint.h>
+#include "../../include/qlmx.h"
+
+#define QLM_MAXSPAN 4096
+typedef qlmx_span QSpanD;
+typedef unsigned short bf16;
+
+typedef struct {
+    int on, adam, dmax, group, lrmode, servo_every, packed, v4;
+    float fstar, f_hi, f_lo;
+    int nspan;
+    QSpanD *spanH, *spanD;
+    unsigned long long nq, ngrp, np;
+    signed char *d, *r, *m8;
+    unsigned char *v8;
+    float *s, *m8s, *v8s;
+    unsigned long long fs_off[QLM_MAXSPAN], fs_n[QLM_MAXSPAN], fs_cs[QLM_MAXSPAN];
+    int nfs; unsigned long long nfloat;
+    bf16 *Mc, *Vc;                       /* owned by the caller's float-span optimizer; may be NULL */
+    long long *statD; long long statH[4];
+    int render_p;                        /* 1: the step keeps the fp32 view P up to date (reference behaviour) */
+} Qlm;
+
+typedef struct { unsigned long long pof, n; } QlmSpanDesc;
+
+void *dmalloc(size_t bytes);                                            /* cudalm.cu:153 */
+void  qlm_add_span(Qlm *q, unsigned long long pof, unsigned long long n);          /* qlm.cuh:448 */
+void  qlm_gpu_init(Qlm *q, const QlmSpanDesc *spans, int nspan, float *P, size_t np); /* qlm.cuh:458 */
+void  qlm_gpu_render(Qlm *q, float *P);                                 /* qlm.cuh:577 */
+void  qlm_render_spans(Qlm *q, float *P, int span0, int nspans);        /* qlm.cuh:586 (one layer = 7 spans) */
+void  qlm_step_launch(float *P, const float *G, signed char *d, signed char *r, float *s,
+                      signed char *m8, float *m8s, unsigned char *v8, float *v8s,
+                      const QSpanD *sp, int nspan, int group, int dmax,
+                      float lr, float b1, float b2, float wd, float gscale, const float *gsp,
+                      float inv_bc1, float inv_sqrt_bc2, int lrmode,
+                      unsigned long long t, int adam, long long *stat, int packed,
+                      int gi_base, int ng);                             /* qlm.cuh:377 */
+void  qlm_gpu_update(Qlm *q, float *P, float *G, float lr, float b1, float b2, float wd,
+                     float bc1, float bc2, int t, const float *gs);     /* cudalm.cu:6082 */
+double qlm_persist_bytes(const Qlm *q);                                 /* qlm.cuh:678 */
+int   qlm_save(const Qlm *q, const char *path, int iter, float prev_gn); /* qlm.cuh:702 */
+int   qlm_load(Qlm *q, const char *path, int *iter, float *prev_gn);    /* qlm.cuh:740 */
+void  qlm_free(Qlm *q);
+
+/* grouped expert GEMMs: row-major, B points into the (possibly virtual) fp32 view P */
+void mg_bind(const Qlm *q, const float *Pbase, int act_dtype, int math);
+void mg_ab(const void *A, const float *B, float *C, int M, int K, int N);                /* cudalm.cu:3247 */
+void mg_abt_b(const void *A, const float *B, float *C, int M, int K, int N, float beta); /* cudalm.cu:3250 */
+void mg_abt(const void *A, const float *B, float *C, int M, int K, int N);               /* cudalm.cu:3253 */
+void mg_atb(const void *A, const void *B, float *C, int M, int K, int N);                /* cudalm.cu:3254 */
+void mg_flush(void);                                                                      /* cudalm.cu:3243 */
+#endif

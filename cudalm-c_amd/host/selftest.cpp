@@ -1,0 +1,117 @@
+/* selftest.cpp -- the QLM section of the reference's in-binary selftest (cudalm.cu:10477-10649)
+ * rewritten against the host mirror: encode+render within half a quantisation step and at most
+ * 2*dmax+1 levels per group; one Integer AdamW step against a scalar host restatement that reuses
+ * the host helpers (digits/residuals must agree bit for bit here because both sides are compiled
+ * without FMA contraction); a save/load round trip; an expert FFN forward through the grouped GEMM
+ * queue against a host triple loop. Prints one line per check and exits 0 only if all pass. */
+#include "qlm_host.h"
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <vector>
+
+static uint64_t rng = 0x9E3779B97F4A7C15ULL;
+static float urand(){ rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17; return (float)((rng >> 40) * (1.0 / 16777216.0)); }
+static float nrand(){ float u1 = urand(); if(u1 < 1e-9f) u1 = 1e-9f; float u2 = urand(); return sqrtf(-2.0f * logf(u1)) * cosf(6.28318530718f * u2); }
+static int ok_all = 1;
+static void check(const char *name, double v, double tol){ printf("  %-34s %.3e  %s\n", name, v, v <= tol ? "OK" : "FAIL"); if(!(v <= tol)) ok_all = 0; }
+
+int main(){
+    if(qlmx_init(0) != QLMX_OK){ fprintf(stderr, "%s\n", qlmx_last_error()); return 2; }
+    printf("[selftest] %s\n", qlmx_device_name());
+    /* a toy layer: 16 floats of "norm", then w1, w3 [D,F] x E and w2 [F,D] x E */
+    const int E = 3, D = 128, F = 256, N = 40;
+    const size_t nw = (size_t)E * D * F, np = 16 + 3 * nw + 8;
+    QlmSpanDesc spans[3] = {{16, nw}, {16 + nw, nw}, {16 + 2 * nw, nw}};
+    std::vector<float> Ph(np), Gh(np);
+    for(size_t i = 0; i < np; i++){ Ph[i] = 0.02f * nrand(); Gh[i] = 0.01f * nrand(); }
+    float *Pd = (float *)dmalloc(np * 4), *Gd = (float *)dmalloc(np * 4);
+    qlmx_memcpy_h2d(Pd, Ph.data(), np * 4); qlmx_memcpy_h2d(Gd, Gh.data(), np * 4);
+    Qlm q; qlm_gpu_init(&q, spans, 3, Pd, np);
+    printf("[selftest] %d spans, %llu weights, %llu groups, %.2f B/param persistent\n", q.nspan, q.nq, q.ngrp, qlm_persist_bytes(&q) / (double)q.nq);
+
+    /* (a) encode + render */
+    std::vector<float> Pr(np), sh(q.ngrp);
+    qlmx_memcpy_d2h(Pr.data(), Pd, np * 4); qlmx_memcpy_d2h(sh.data(), q.s, q.ngrp * 4);
+    double worst = 0; int lvlmax = 0;
+    for(int si = 0; si < q.nspan; si++) for(int g = 0; g < q.spanH[si].ngrp; g++){
+        int gi = q.spanH[si].gi0 + g; std::vector<float> lv;
+        for(int j = 0; j < q.group; j++){
+            size_t k = q.spanH[si].pof + (size_t)g * q.group + j;
+            double e = fabs((double)Pr[k] - Ph[k]) / sh[gi]; if(e > worst) worst = e;
+            bool seen = false; for(float v : lv) if(v == Pr[k]) seen = true;
+            if(!seen) lv.push_back(Pr[k]);
+        }
+        if((int)lv.size() > lvlmax) lvlmax = (int)lv.size();
+    }
+    check("qlm encode err/step", worst, 0.51);
+    check("qlm distinct levels per group", lvlmax, 2 * q.dmax + 1);
+    for(size_t i = 0; i < 16; i++) if(Pr[i] != Ph[i]) ok_all = 0;        /* float span untouched */
+
+    /* (b) one step vs a scalar host restatement on the pre-step state */
+    const int T = 3; const float lr = 3e-4f, b1 = 0.9f, b2 = 0.95f, wd = 0.1f;
+    const float bc1 = 1.0f - powf(b1, (float)T), bc2 = 1.0f - powf(b2, (float)T);
+    unsigned long long nq = q.nq, ng = q.ngrp, nd = qlmx_qd_bytes(nq, q.packed);
+    std::vector<signed char> hd(nd), hr(nq), hm(nq), rd(nd), rr_(nq); std::vector<unsigned char> hv(nq);
+    std::vector<float> hs(ng), hms(ng), hvs(ng);
+    qlmx_memcpy_d2h(hd.data(), q.d, nd); qlmx_memcpy_d2h(hr.data(), q.r, nq); qlmx_memcpy_d2h(hm.data(), q.m8, nq);
+    qlmx_memcpy_d2h(hv.data(), q.v8, nq); qlmx_memcpy_d2h(hs.data(), q.s, ng * 4);
+    qlmx_memcpy_d2h(hms.data(), q.m8s, ng * 4); qlmx_memcpy_d2h(hvs.data(), q.v8s, ng * 4);
+    const float inv_bc1 = 1.0f / bc1, inv_sqrt_bc2 = 1.0f / sqrtf(bc2);
+    for(int si = 0; si < q.nspan; si++) for(int g = 0; g < q.spanH[si].ngrp; g++){
+        int gi = q.spanH[si].gi0 + g; unsigned long long j0 = (unsigned long long)g * q.group;
+        unsigned long long pof = q.spanH[si].pof + j0, qi0 = q.spanH[si].qi0 + j0;
+        float sg = hs[gi], L = lr * 128.0f / (q.lrmode ? sg : q.spanH[si].sref), dec = lr * wd * 128.0f;
+        float ms_old = hms[gi], vs_old = hvs[gi];
+        for(int j = 0; j < q.group; j++){
+            unsigned long long qi = qi0 + j; float gr = Gh[pof + j], mv = (float)hm[qi] * ms_old;
+            float sv = (float)hv[qi] * vs_old, vv = sv * sv, mn = b1 * mv + (1.0f - b1) * gr;
+            vv = b2 * vv + (1.0f - b2) * gr * gr; float rv = sqrtf(vv), veps = fmaxf(vs_old, 1e-8f);
+            float u = (mn * inv_bc1) / (rv * inv_sqrt_bc2 + veps); u = fmaxf(-8.0f, fminf(8.0f, u));
+            int dd = qlmx_qd_get(hd.data(), qi, q.packed), idl = qlmx_qsri(-(L * u + dec * (float)dd), qi, (unsigned long long)T);
+            int r2 = (int)hr[qi] + idl, c = (r2 > 64) ? (((r2 - 65) >> 7) + 1) : ((r2 < -64) ? -((((-r2) - 65) >> 7) + 1) : 0);
+            r2 -= c * 128; dd = qlmx_qclmp(dd + c, -q.dmax, q.dmax);
+            qlmx_qd_set_host(rd.data(), qi, dd, q.packed); rr_[qi] = (signed char)r2;
+        }
+    }
+    qlm_gpu_update(&q, Pd, Gd, lr, b1, b2, wd, bc1, bc2, T, NULL);
+    qlmx_sync(NULL);
+    std::vector<signed char> gd(nd), gr2(nq);
+    qlmx_memcpy_d2h(gd.data(), q.d, nd); qlmx_memcpy_d2h(gr2.data(), q.r, nq);
+    unsigned long long dmiss = 0, rmiss = 0;
+    for(unsigned long long i = 0; i < nq; i++){ if(qlmx_qd_get(gd.data(), i, q.packed) != qlmx_qd_get(rd.data(), i, q.packed)) dmiss++; if(gr2[i] != rr_[i]) rmiss++; }
+    check("qlm step digits differing", (double)dmiss, 0);
+    check("qlm step residuals differing", (double)rmiss, 0);
+
+    /* (c) checkpoint round trip */
+    const char *path = "/tmp/qlmx_selftest.opt.q";
+    int okio = qlm_save(&q, path, 77, 1.25f);
+    qlmx_memset(q.d, 0, nd, NULL); qlmx_memset(q.m8, 0, nq, NULL);
+    int iter = 0; float pg = 0; okio = okio && qlm_load(&q, path, &iter, &pg);
+    std::vector<signed char> gd2(nd); qlmx_memcpy_d2h(gd2.data(), q.d, nd);
+    check("qlm save/load round trip", (okio && iter == 77 && pg == 1.25f && !memcmp(gd.data(), gd2.data(), nd)) ? 0 : 1, 0);
+    remove(path);
+
+    /* (d) expert forward through the grouped queue, weights addressed as P + offset */
+    qlm_gpu_render(&q, Pd);                         /* host copy of what the digits mean */
+    qlmx_memcpy_d2h(Pr.data(), Pd, np * 4);
+    std::vector<float> X((size_t)N * D), Y((size_t)N * F, 0.f), Yref((size_t)N * F, 0.f);
+    for(auto &v : X) v = nrand();
+    float *Xd = (float *)dmalloc(X.size() * 4), *Yd = (float *)dmalloc(Y.size() * 4);
+    qlmx_memcpy_h2d(Xd, X.data(), X.size() * 4);
+    int off[4] = {0, 13, 13, 40};                   /* expert 1 gets no rows */
+    mg_bind(&q, Pd, QLMX_ACT_F32, QLMX_MATH_F32);
+    for(int e = 0; e < E; e++){ int ne = off[e + 1] - off[e]; if(!ne) continue;
+        mg_ab(Xd + (size_t)off[e] * D, Pd + 16 + (size_t)e * D * F, Yd + (size_t)off[e] * F, ne, D, F); }
+    mg_flush(); qlmx_sync(NULL);
+    qlmx_memcpy_d2h(Y.data(), Yd, Y.size() * 4);
+    for(int e = 0; e < E; e++) for(int m = off[e]; m < off[e + 1]; m++) for(int f = 0; f < F; f++){
+        double acc = 0; for(int k = 0; k < D; k++) acc += (double)X[(size_t)m * D + k] * Pr[16 + (size_t)e * D * F + (size_t)k * F + f];
+        Yref[(size_t)m * F + f] = (float)acc; }
+    double num = 0, den = 0; for(size_t i = 0; i < Y.size(); i++){ double dlt = (double)Y[i] - Yref[i]; num += dlt * dlt; den += (double)Yref[i] * Yref[i]; }
+    check("moe expert fwd (mg_ab) rel-err", sqrt(num / den), 1e-3);
+    qlm_free(&q);
+    printf(ok_all ? "[selftest] ALL PASS\n" : "[selftest] FAILED\n");
+    return ok_all ? 0 : 1;
+}

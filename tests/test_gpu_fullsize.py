@@ -1,0 +1,151 @@
+"""GPU checks at BASELINE.json's full sizes. Where the CPU oracle finishes in seconds the comparison
+is byte for byte (config 4: the whole 120*2^20-weight Integer AdamW sweep); for the training-size GEMMs
+(configs 3 and 5) the MFMA kernels are compared against the library's fp32 kernels at full size
+(those are themselves pinned to the oracle in test_gpu_gemm.py) and against the oracle on a sampled
+subset of experts, and through size-independent properties (linearity in the activations,
+wgrad == sum of per-row outer products in any row split)."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from __graft_entry__ import load_package, PKG_DIR
+from oracle.binding import make_spans
+
+pkg = load_package()
+f32 = np.float32
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def q():
+    return pkg.load()
+
+
+def dev(a):
+    import torch
+    if a.dtype.names:
+        a = a.view(np.uint8)
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def test_host_mirror_selftest_binary():
+    """The C++ host mirror (qlm_gpu_init / qlm_gpu_update / qlm_save / qlm_load / mg_ab + mg_flush)
+    run end to end by the compiled selftest, the counterpart of `cudalm selftest`'s QLM section."""
+    exe = os.path.join(PKG_DIR, "qlm_selftest")
+    assert os.path.exists(exe), "build with python cudalm-c_amd/build.py"
+    p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    print(p.stdout)
+    assert p.returncode == 0 and "ALL PASS" in p.stdout, p.stdout
+
+
+def test_c4_full_adamw_sweep_bit_exact(q, orc):
+    """Config 4: 120*2^20 weights, seeded random integer state, grads ~N(0,1e-3), lr 3e-4,
+    betas (0.9, 0.95), wd 0.1, t=1: d, r, m8, v8, m8s, v8s byte-identical to the CPU oracle."""
+    import torch
+    nq = 120 * 2 ** 20
+    group = 128
+    tab, _, ng = make_spans([nq], group)
+    hd = orc.digits(nq, 0, 20); hr = orc.int8(nq, 0, 21, -64, 64); hm8 = orc.int8(nq, 0, 22, -127, 127)
+    hv8 = orc.u8(nq, 0, 23, 0, 255)
+    hs = orc.uniform(ng, 0, 24, 0.5, 1.5) * f32(0.02 * 3 / 7)
+    hm8s = orc.uniform(ng, 0, 25, 0.5, 1.5) * f32(3e-3 / 127)
+    hv8s = orc.uniform(ng, 0, 26, 0.5, 1.5) * f32(3e-3 / 255)
+    tab["sref"] = f32(np.mean(hs.astype(np.float64)))
+    hG = orc.normal(nq, 0, 27, 1e-3)
+    d, r, m8, v8, s, m8s, v8s, G = (dev(x) for x in (hd, hr, hm8, hv8, hs, hm8s, hv8s, hG))
+    bc1 = f32(1) - f32(0.9); bc2 = f32(1) - f32(0.95)
+    hp = (3e-4, 0.9, 0.95, 0.1, 1.0, None, float(f32(1) / bc1), float(f32(1) / np.sqrt(bc2)), 0, 1, 1, None, 1, 0, ng)
+    q.step(None, G, d, r, s, m8, m8s, v8, v8s, dev(tab), 1, group, 7, *hp)
+    orc.step(None, hG, hd, hr, hs, hm8, hm8s, hv8, hv8s, tab, group, 7, *hp)
+    torch.cuda.synchronize()
+    for name, got, want in [("d", d, hd), ("r", r, hr), ("m8", m8, hm8), ("v8", v8, hv8), ("m8s", m8s, hm8s), ("v8s", v8s, hv8s)]:
+        g = got.cpu().numpy()
+        assert np.array_equal(g.view(np.uint8), want.view(np.uint8)), name
+    # the digits stayed inside [-7, 7] and the residuals inside [-64, 64]
+    u = d.view(torch.uint8)
+    assert int(((u & 15) == 8).sum()) == 0 and int(((u >> 4) == 8).sum()) == 0
+    assert int(r.min()) >= -64 and int(r.max()) <= 64
+
+
+def _packed_random(n, gen):
+    import torch
+    b = torch.randint(0, 256, (n // 2,), dtype=torch.int16, device="cuda", generator=gen).to(torch.uint8)
+    lo = b & 15; hi = b >> 4
+    lo = torch.where(lo == 8, torch.zeros_like(lo), lo); hi = torch.where(hi == 8, torch.zeros_like(hi), hi)
+    return (lo | (hi << 4)).view(torch.int8)
+
+
+@pytest.mark.parametrize("E,D,F,rows", [(32, 768, 2048, 16384), (8, 2048, 1408, 16384)])
+def test_train_size_mfma_vs_fp32_kernels_and_properties(q, orc, E, D, F, rows):
+    """Configs 3 and 5 (one layer's shapes; config 5 on 8 of its 64 experts): Zipf row counts, all three
+    orientations at full row count. MFMA vs the fp32 kernels <= 1e-3 relative L2; linearity of the
+    forward in the activations; the weight gradient of a row split sums to the unsplit one."""
+    import torch
+    gen = torch.Generator(device="cuda"); gen.manual_seed(1)
+    p = (np.arange(E) + 1.0) ** -1.1
+    cnt = np.random.default_rng(0).multinomial(rows, p / p.sum())
+    off = np.concatenate([[0], np.cumsum(cnt)]).astype(int)
+    nw = E * D * F
+    d = _packed_random(nw, gen)
+    s = (0.02 * 3 / 7) * (0.5 + torch.rand(nw // 128, device="cuda", generator=gen))
+    X = torch.randn(rows * D, device="cuda", generator=gen).to(torch.bfloat16)
+    dY = torch.randn(rows * F, device="cuda", generator=gen).to(torch.bfloat16)
+
+    def probs(A, aw, B, bw, C, cw, per_expert=False):
+        return q.problems([(A.data_ptr() + int(off[e]) * aw * 2, (B.data_ptr() + int(off[e]) * bw * 2) if B is not None else None,
+                            C.data_ptr() + (e * D * F * 4 if per_expert else int(off[e]) * cw * 4),
+                            e * D * F, e * D * F // 128, int(cnt[e]), 0.0) for e in range(E)])
+
+    def rel(a, b):
+        return float(((a - b).double().norm() / b.double().norm()).item())
+
+    # forward nn: [rows, D] @ W[D, F]
+    Y1 = torch.zeros(rows * F, device="cuda"); Y2 = torch.zeros(rows * F, device="cuda")
+    q.gemm_nn(d, s, 128, probs(X, D, None, 0, Y1, F), E, D, F, pkg.ACT_BF16, pkg.MATH_MFMA)
+    q.gemm_nn(d, s, 128, probs(X, D, None, 0, Y2, F), E, D, F, pkg.ACT_BF16, pkg.MATH_F32)
+    assert rel(Y1, Y2) < 1e-3
+    # linearity: f(-2x) == -2 f(x) up to the matrix core's internal summation rounding
+    X2 = (X.float() * -2).to(torch.bfloat16)
+    Y3 = torch.zeros(rows * F, device="cuda")
+    q.gemm_nn(d, s, 128, probs(X2, D, None, 0, Y3, F), E, D, F, pkg.ACT_BF16, pkg.MATH_MFMA)
+    assert rel(Y3, -2 * Y1) < 1e-6
+    # dgrad tn: [rows, F] @ W[D, F]^T -> [rows, D]
+    dX1 = torch.zeros(rows * D, device="cuda"); dX2 = torch.zeros(rows * D, device="cuda")
+    q.gemm_tn(d, s, 128, probs(dY, F, None, 0, dX1, D), E, F, D, pkg.ACT_BF16, pkg.MATH_MFMA)
+    q.gemm_tn(d, s, 128, probs(dY, F, None, 0, dX2, D), E, F, D, pkg.ACT_BF16, pkg.MATH_F32)
+    assert rel(dX1, dX2) < 1e-3
+    # wgrad nt: G[D, F] += X^T dY per expert
+    G1 = torch.zeros(nw, device="cuda"); G2 = torch.zeros(nw, device="cuda")
+    q.gemm_nt(probs(X, D, dY, F, G1, 0, True), E, D, F, pkg.ACT_BF16, pkg.MATH_MFMA)
+    q.gemm_nt(probs(X, D, dY, F, G2, 0, True), E, D, F, pkg.ACT_BF16, pkg.MATH_F32)
+    assert rel(G1, G2) < 1e-3
+    # splitting every expert's rows in two and accumulating (beta = 1 semantics) gives the same sum
+    half = [int(c) // 2 for c in cnt]
+    G3 = torch.zeros(nw, device="cuda")
+    pa = q.problems([(X.data_ptr() + int(off[e]) * D * 2, dY.data_ptr() + int(off[e]) * F * 2, G3.data_ptr() + e * D * F * 4, 0, 0, half[e], 1.0) for e in range(E)])
+    pb = q.problems([(X.data_ptr() + (int(off[e]) + half[e]) * D * 2, dY.data_ptr() + (int(off[e]) + half[e]) * F * 2, G3.data_ptr() + e * D * F * 4, 0, 0, int(cnt[e]) - half[e], 1.0) for e in range(E)])
+    q.gemm_nt(pa, E, D, F, pkg.ACT_BF16, pkg.MATH_MFMA)
+    q.gemm_nt(pb, E, D, F, pkg.ACT_BF16, pkg.MATH_MFMA)
+    assert rel(G3, G1) < 1e-5
+    # sampled experts against the CPU oracle (rendered weights, fp32 GEMM)
+    torch.cuda.synchronize()
+    hs = s.cpu().numpy(); hd = d.cpu().numpy()
+    for e in (0, E - 1):
+        m = min(int(cnt[e]), 256)
+        if m == 0:
+            continue
+        tab, _, ng = make_spans([D * F], 128)
+        P = np.zeros(D * F, f32)
+        orc.render(P, hd[e * D * F // 2:(e + 1) * D * F // 2].copy(), hs[e * D * F // 128:(e + 1) * D * F // 128].copy(), tab, 128, 1, 0, ng)
+        A = X[int(off[e]) * D:(int(off[e]) + m) * D].float().cpu().numpy()
+        want = np.zeros(m * F, f32)
+        orc.gemm_nn(A, P, want, m, D, F)
+        got = Y1[int(off[e]) * F:(int(off[e]) + m) * F].cpu().numpy()
+        assert orc.relerr(got, want) < 1e-3
+        B = dY[int(off[e]) * F:(int(off[e]) + m) * F].float().cpu().numpy()
+        want = np.zeros(m * D, f32)
+        orc.gemm_tn(B, P, want, m, F, D, 0.0)
+        got = dX1[int(off[e]) * D:(int(off[e]) + m) * D].cpu().numpy()
+        assert orc.relerr(got, want) < 1e-3

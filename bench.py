@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train"])
+    ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--adamw-weights", type=int, default=120 * 2 ** 20)
     ap.add_argument("--render-p", type=int, default=0, help="adamw: also write the fp32 view P (4 B/weight more)")
@@ -297,7 +297,7 @@ def cpu_adamw(args):
     P = np.zeros(nq, np.float32)
     reps, t_used = 0, 0.0
     lib.step(P, G, d, r, s, m8, m8s, v8, v8s, tab, 128, 7, 3e-4, 0.9, 0.95, 0.1, 1.0, None, 10.0, 4.47, 0, 1, 1, None, 1, 0, ng)
-    while t_used < 8.0 and reps < 50:
+    while t_used < 10.0 and reps < 5000:
         t0 = time.perf_counter()
         lib.step(P, G, d, r, s, m8, m8s, v8, v8s, tab, 128, 7, 3e-4, 0.9, 0.95, 0.1, 1.0, None, 10.0, 4.47, 0, 2 + reps, 1, None, 1, 0, ng)
         t_used += time.perf_counter() - t0
@@ -306,6 +306,52 @@ def cpu_adamw(args):
     return {"value": gbs, "unit": "GB/s", "cores": threads, "kind": kind,
             "sample": "Integer AdamW (P rendered, 15.16 B/weight) over %d weights x %d steps, %s" % (nq, reps, "cpu_kern.h cpu_qlm_step" if kind == "reference" else "oracle/qlm_oracle.c"),
             "weights_per_s": nq * reps / t_used}
+
+
+def bench_copy(torch, q, args):
+    """Plain 1 GiB device copy: the known-size kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
+    n = 2 ** 28
+    a = torch.randn(n, device="cuda:0"); b = torch.empty_like(a)
+    tm = timed(torch, lambda: b.copy_(a), args.steps, args.warmup)
+    gbs = 2 * n * 4 / (tm["event_ms_avg"] * 1e-3) / 1e9
+    return {"workload": "calibration: torch copy of 1 GiB (1 GiB read + 1 GiB written per launch)", "metric": "copy GB/s", "value": gbs,
+            "unit": "GB/s", "ms_per_step": tm["wall_ms"], "dtype": "f32",
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                         "kernel": "at::native elementwise copy"}}
+
+
+def cpu_gemm(args):
+    """Reference CPU expert GEMMs (cpu_rt.h packed SGEMM through g_ab / g_abt_b / g_atb on a rendered fp32
+    view) on a bounded sample: one expert's forward, input-gradient and weight-gradient GEMM at the layer's
+    D=768, F=2048 with 2048 rows, repeated for about 10 s."""
+    import numpy as np
+    from oracle.binding import Oracle, Ref, have_ref
+    orc = Oracle()
+    threads = min(16, os.cpu_count() or 1)
+    kind = "reference" if have_ref() else "port"
+    lib = Ref(threads=threads) if kind == "reference" else orc
+    orc.set_threads(threads)
+    M, D, F = 2048, 768, 2048
+    X = orc.normal(M * D, 0, 1); W = orc.normal(D * F, 0, 2, 0.02); dY = orc.normal(M * F, 0, 3)
+    Y = np.zeros(M * F, np.float32); dX = np.zeros(M * D, np.float32); G = np.zeros(D * F, np.float32)
+    lib.gemm_nn(X, W, Y, M, D, F)
+    reps, t_used = 0, 0.0
+    while t_used < 12.0 and reps < 5000:
+        t0 = time.perf_counter()
+        lib.gemm_nn(X, W, Y, M, D, F)
+        lib.gemm_tn(dY, W, dX, M, F, D, 0.0)
+        lib.gemm_nt(X, dY, G, M, D, F)
+        t_used += time.perf_counter() - t0
+        reps += 1
+    tf = 3 * 2.0 * M * D * F * reps / t_used / 1e12
+    return {"value": tf, "unit": "TFLOP/s", "cores": threads, "kind": kind,
+            "sample": "one expert, %d rows, D=%d F=%d: fwd + dgrad + wgrad fp32 SGEMM on the rendered view, %d repetitions (%s)"
+                      % (M, D, F, reps, "cpu_rt.h sg_core via g_ab/g_abt_b/g_atb" if kind == "reference" else "oracle/qlm_oracle.c")}
+
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the 1 GiB copy calibration);
+# the runs, counter values and scale factors are in profiles/*.txt. None where not measured.
+PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": None, "decode": None}
 
 
 def main():
@@ -320,12 +366,12 @@ def main():
     q = pkg.load()           # raises if libqlmx.so is missing or no gfx950 device
     torch.cuda.set_device(0)
     want = ["train", "decode", "adamw"] if args.workload == "all" else [args.workload]
-    runners = {"adamw": bench_adamw, "train": bench_train, "decode": bench_decode}
+    runners = {"adamw": bench_adamw, "train": bench_train, "decode": bench_decode, "copy": bench_copy}
     results = {}
     for w in want:
         if w in runners:
             results[w] = runners[w](torch, q, args)
-    first = next(results[w] for w in ["train", "decode", "adamw"] if w in results)
+    first = next(results[w] for w in ["train", "decode", "adamw", "copy"] if w in results)
     line = {
         "metric": "QLM expert dequant-GEMM TFLOP/s & GB/s (% roofline); int-AdamW GB/s",
         "value": first["value"], "unit": first["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -336,9 +382,16 @@ def main():
         "workloads": results,
         "device": q.call("qlmx_device_name").decode(),
     }
+    for w in results:
+        if results[w]["roofline"].get("traffic") is None and PROFILED_TRAFFIC.get(w) and not (w == "adamw" and args.render_p):
+            results[w]["roofline"]["traffic"] = PROFILED_TRAFFIC[w]
     if not args.no_cpu:
         if "adamw" in results:
-            line["cpu_baseline"] = cpu_adamw(args)
+            results["adamw"]["cpu_baseline"] = cpu_adamw(args)
+        if "train" in results:
+            line["cpu_baseline"] = cpu_gemm(args)
+        elif "adamw" in results:
+            line["cpu_baseline"] = results["adamw"]["cpu_baseline"]
     print(json.dumps(line))
 
 

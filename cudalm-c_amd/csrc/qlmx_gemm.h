@@ -34,6 +34,22 @@ __device__ __forceinline__ int qx_find_problem(const DevProb *pr, int nprob, int
     return lo;
 }
 
+/* Tile handled by workgroup b when workgroups go round-robin to 8 XCDs and the grid has been
+ * padded to a multiple of 8: XCD x gets the x-th contiguous eighth of the list. The caller drops
+ * results >= the real tile count. */
+__device__ __forceinline__ int qx_xcd_tile(int b, int grid){
+    const int per = grid >> 3;
+    return (b & 7) * per + (b >> 3);
+}
+
+/* The same for tiles of unequal cost (weight gradients: depth = the expert's row count): rows of
+ * `g` consecutive tiles (one output tile-row, sharing an operand block) are dealt round-robin to the
+ * XCDs, so a heavy expert's rows spread over all of them. grid = 8 * g * ceil(rows / 8). */
+__device__ __forceinline__ int qx_xcd_tile_rows(int b, int g){
+    const int x = b & 7, k = b >> 3;
+    return (x + 8 * (k / g)) * g + k % g;
+}
+
 __device__ __forceinline__ float qx_bf16_to_f32(unsigned short h){ return __uint_as_float((uint32_t)h << 16); }
 /* round to nearest even, as cudalm.cu:334-338 */
 __device__ __forceinline__ unsigned short qx_f32_to_bf16(float f){

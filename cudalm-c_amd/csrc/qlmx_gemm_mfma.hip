@@ -15,46 +15,61 @@
  *       running result. No weight rounding at all.
  *   nt (weight gradient): both operands are bf16 activations / gradients; fp32 accumulate into G.
  *
- * Tiling: 256 threads = 4 wavefronts per 128x128 output tile, each wave a 64x64 quadrant held as
- * 2x2 accumulators of 32x32 (64 accumulator registers). The contraction advances 32 at a time
- * through LDS tiles stored contraction-contiguous ([row][k], 80-byte pitch) so that a lane's MFMA
- * operand (8 consecutive k of one row) is a single 128-bit LDS read. Global loads for step t+1 are
- * issued before the MFMAs of step t. One launch covers every expert of the call through a
- * flattened (problem, row tile, column tile) list.
+ * Tiling: 256 threads = 4 wavefronts in a 2x2 arrangement; a wave owns (32*WM) x 64 of the output as
+ * WM x 2 accumulators of 32x32. nn and nt use WM = 4 (256x128 per workgroup, which halves the
+ * dequantisation work per flop); tn keeps a second set of accumulators for the per-group partial
+ * sums and uses WM = 2 (128x128). The contraction advances 32 at a time.
+ *
+ * LDS holds operands as 16-byte items of 8 consecutive contraction elements, item (ko, row) at
+ * index ko*ROWS + (row ^ swizzle), swizzle = ((row >> 4) ^ 4*ko) & 15 on the low four bits. A lane's
+ * MFMA operand is then one 128-bit read; the 128-bit writes of straight copies, the 32-bit writes of
+ * transposing stores and the operand reads each hit all 64 banks without (or with 2-way) conflicts,
+ * with no padding. Global loads walk the contiguous index fastest so every wave instruction covers
+ * 64-512 contiguous bytes per row. Two LDS buffers: the stores and loads for the next steps are
+ * issued around the MFMAs of the current one and a single barrier closes a step. One launch covers
+ * every expert of the call through a flattened (problem, row tile, column tile) list.
  */
 #include "qlmx_gemm.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float  f32x2  __attribute__((ext_vector_type(2)));
 typedef float  f32x16 __attribute__((ext_vector_type(16)));
 
-#define BM 128
 #define BN 128
 #define BK 32
-#define LDP 40              /* LDS row pitch in bf16 elements: 32 + 8 pad (80 bytes) */
+#define KO 4                 /* 16-byte items per row per step */
 
-struct MfmaArgs { const DevProb *pr; int nprob; const signed char *d; const float *s; int group; int K, N; };
+struct MfmaArgs { const DevProb *pr; int nprob, ntiles, tiles_n; const signed char *d; const float *s; int group, gshift; int K, N; };
 
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi){
-    return (uint32_t)qx_f32_to_bf16(lo) | ((uint32_t)qx_f32_to_bf16(hi) << 16);
+/* two floats -> packed bf16 pair, round to nearest even (one v_cvt_pk_bf16_f32) */
+__device__ __forceinline__ uint32_t pk_bf16(float lo, float hi){
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
-__device__ __forceinline__ bf16x8 lds_frag(const unsigned short *p){
-    const uint4 v = *(const uint4 *)p;
-    return __builtin_bit_cast(bf16x8, v);
+__device__ __forceinline__ uint4 pk8_bf16(const float *p){
+    const float4 a = *(const float4 *)p, b = *(const float4 *)(p + 4);
+    return make_uint4(pk_bf16(a.x, a.y), pk_bf16(a.z, a.w), pk_bf16(b.x, b.y), pk_bf16(b.z, b.w));
+}
+template<int ROWS> __device__ __forceinline__ int item_at(int ko, int row){
+    return ko * ROWS + (row ^ (((row >> 4) ^ (ko << 2)) & 15));
 }
 
-/* activation value as bf16 bits */
-template<bool BF16> __device__ __forceinline__ unsigned short act_bits(const void *p, size_t i){
-    if constexpr(BF16) return ((const unsigned short *)p)[i];
-    return qx_f32_to_bf16(((const float *)p)[i]);
-}
+template<int MODE, bool BF16, int WM, bool DEEP>
+__global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
+    constexpr int BM = 64 * WM;
+    constexpr int NB = MODE == GEMM_NN ? 2 : 1;                 /* B planes: hi (+ lo) */
+    constexpr int A_BYTES = KO * BM * 16, B_BYTES = KO * BN * 16;
+    /* one LDS block: [buffer 0: A | B hi | B lo][buffer 1: ...] */
+    constexpr int BUF_BYTES = A_BYTES + NB * B_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * BUF_BYTES];
 
-template<int MODE, bool BF16>
-__global__ void __launch_bounds__(256) k_gemm_mfma(MfmaArgs a){
-    /* As: rows of the output's first index; Bs: rows of the second. NN keeps two B tiles (hi, lo). */
-    __shared__ __attribute__((aligned(16))) unsigned short As[BM * LDP];
-    __shared__ __attribute__((aligned(16))) unsigned short Bs[(MODE == GEMM_NN ? 2 : 1) * BN * LDP];
-
-    const int t = blockIdx.x;
+    /* Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. nn/tn (tiles of equal
+     * cost): XCD x takes the x-th contiguous eighth of the tile list, so tiles sharing an expert's
+     * rows and weights meet in one L2. nt (cost = the expert's row count): whole output tile-rows are
+     * dealt round-robin instead, which keeps the XCDs balanced. */
+    const int t = MODE == GEMM_NT ? qx_xcd_tile_rows(blockIdx.x, a.tiles_n) : qx_xcd_tile(blockIdx.x, gridDim.x);
+    if(t >= a.ntiles) return;
     const DevProb P = a.pr[qx_find_problem(a.pr, a.nprob, t)];
     const int lt = t - P.tile0;
     const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
@@ -62,143 +77,198 @@ __global__ void __launch_bounds__(256) k_gemm_mfma(MfmaArgs a){
     const int rows  = MODE == GEMM_NT ? a.K : P.M;
     const int depth = MODE == GEMM_NT ? P.M : a.K;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;      /* quadrant of this wave */
+    const int wi = (wave >> 1) * (32 * WM), wj = (wave & 1) * 64;
+    const int fr = lane & 31, hf = lane >> 5;
 
-    f32x16 acc[2][2], part[2][2];
+    f32x16 acc[WM][2];
+    f32x16 part[MODE == GEMM_TN ? WM : 1][2];
 #pragma unroll
-    for(int i = 0; i < 2; i++)
+    for(int i = 0; i < WM; i++)
 #pragma unroll
-        for(int j = 0; j < 2; j++){ acc[i][j] = (f32x16)(0.0f); part[i][j] = (f32x16)(0.0f); }
+        for(int j = 0; j < 2; j++) acc[i][j] = (f32x16)(0.0f);
+    if constexpr(MODE == GEMM_TN){
+#pragma unroll
+        for(int i = 0; i < WM; i++)
+#pragma unroll
+            for(int j = 0; j < 2; j++) part[i][j] = (f32x16)(0.0f);
+    }
 
-    /* ---- per-thread staging registers for one 32-deep step ---- */
-    uint4 ra[2];            /* NN/TN: two 16-byte pieces of A rows. NT: two row-pairs x 8 k of A */
-    uint4 rb[2];            /* NT: two row-pairs x 8 n of B. */
-    uint32_t rw[2];         /* NN: digits of rows k,k+1 (8 n each). TN: two dwords (8 k each) */
-    float rs[2];            /* NN: scales of rows k, k+1 */
+    /* ---- everything that does not change from step to step is computed once: global pointers
+     * (advanced by a constant per step), LDS byte offsets of this thread's stores and of its MFMA
+     * operand reads. Rows past the end of a problem are clamped to its last row instead of being
+     * zero-filled when they only feed output rows that are never stored. ---- */
+    constexpr int NA = MODE == GEMM_NT ? 4 : WM;       /* 16-byte A-side loads per thread per step */
+    constexpr int ESZ = BF16 ? 2 : 4;
+    const char *pa[NA];                                /* A-side source pointers                    */
+    const char *pb[2];                                 /* nt: B-side source pointers                */
+    const signed char *pw0 = a.d, *pw1 = a.d;          /* nn: digit rows k, k+1; tn: row n          */
+    const float *ps0 = a.s, *ps1 = a.s;                /* nn: their scales                          */
+    int sa_off[MODE == GEMM_NT ? 2 : WM];              /* LDS store offsets, A side (nt: per task)  */
+    int sj_off[8];                                     /* transposing stores: the 8 row offsets     */
+    int sb_off = 0, sbj_off[8];                        /* B side                                    */
+    size_t astep, bstep = 0, wstep = 0, sstep = 0;     /* per-step advances in bytes / elements     */
 
-    auto load_step = [&](int p0){
-        if constexpr(MODE == GEMM_NT){
-            /* A^T tile: As[k][m], B^T tile: Bs[n][m]; thread takes the row pair (m, m+1) and 8
-             * consecutive k (resp. n): task = pair 0..15 x octet 0..15 */
-            const int pr_ = tid & 15, oc = tid >> 4;
+    if constexpr(MODE == GEMM_NT){
 #pragma unroll
-            for(int h = 0; h < 2; h++){
-                const int m = p0 + 2 * pr_ + h;
-                uint4 va = make_uint4(0, 0, 0, 0), vb = make_uint4(0, 0, 0, 0);
-                if(m < depth){
-                    if constexpr(BF16){
-                        va = *(const uint4 *)((const unsigned short *)P.A + (size_t)m * a.K + i0 + oc * 8);
-                        vb = *(const uint4 *)((const unsigned short *)P.B + (size_t)m * a.N + j0 + oc * 8);
-                    } else {
-                        const float *pa = (const float *)P.A + (size_t)m * a.K + i0 + oc * 8;
-                        const float *pb = (const float *)P.B + (size_t)m * a.N + j0 + oc * 8;
-                        va = make_uint4(pack_bf16(pa[0], pa[1]), pack_bf16(pa[2], pa[3]), pack_bf16(pa[4], pa[5]), pack_bf16(pa[6], pa[7]));
-                        vb = make_uint4(pack_bf16(pb[0], pb[1]), pack_bf16(pb[2], pb[3]), pack_bf16(pb[4], pb[5]), pack_bf16(pb[6], pb[7]));
-                    }
-                }
-                ra[h] = va; rb[h] = vb;
-            }
+        for(int h = 0; h < 2; h++){
+            const int id = tid + 256 * h, oc = id & 31, mp = id >> 5;
+            const int kk = (i0 + oc * 8 < a.K) ? i0 + oc * 8 : 0;          /* columns past K feed unstored rows */
+#pragma unroll
+            for(int e = 0; e < 2; e++) pa[2 * h + e] = (const char *)P.A + ((size_t)(2 * mp + e) * a.K + kk) * ESZ;
+            sa_off[h] = (mp >> 2) * BM * 16 + (mp & 3) * 4;
+        }
+        { const int oc = (tid & 31), ko = (tid >> 5) >> 2;                 /* task 1 has ko + 2: its swizzle differs in bit 3 */
+          const int sw = ((oc >> 1) ^ (ko << 2)) & 15;
+#pragma unroll
+          for(int j = 0; j < 8; j++) sj_off[j] = ((oc * 8 + j) ^ sw) * 16; }
+        { const int oc = tid & 15, mp = tid >> 4, ko = mp >> 2;
+#pragma unroll
+          for(int e = 0; e < 2; e++) pb[e] = (const char *)P.B + ((size_t)(2 * mp + e) * a.N + j0 + oc * 8) * ESZ;
+          sb_off = A_BYTES + ko * BN * 16 + (mp & 3) * 4;
+          const int sw = ((oc >> 1) ^ (ko << 2)) & 15;
+#pragma unroll
+          for(int j = 0; j < 8; j++) sbj_off[j] = ((oc * 8 + j) ^ sw) * 16; }
+        astep = (size_t)BK * a.K * ESZ; bstep = (size_t)BK * a.N * ESZ;
+    } else {
+#pragma unroll
+        for(int h = 0; h < WM; h++){
+            const int id = tid + 256 * h, kq = id & 3, r = id >> 2;
+            const int rr = (i0 + r < rows) ? i0 + r : rows - 1;            /* clamp: feeds unstored rows only */
+            pa[h] = (const char *)P.A + ((size_t)rr * a.K + kq * 8) * ESZ;
+            sa_off[h] = item_at<BM>(kq, r) * 16;
+        }
+        astep = (size_t)BK * ESZ;
+        if constexpr(MODE == GEMM_NN){
+            const int oc = tid & 15, kp = tid >> 4, ko = kp >> 2;
+            const size_t e0 = (size_t)(2 * kp) * a.N + j0 + oc * 8;
+            pw0 = a.d + ((P.wq + e0) >> 1); pw1 = pw0 + (a.N >> 1);
+            ps0 = a.s + P.wg + (e0 >> a.gshift); ps1 = a.s + P.wg + ((e0 + a.N) >> a.gshift);
+            wstep = (size_t)BK * a.N >> 1; sstep = (size_t)BK * a.N >> a.gshift;
+            sb_off = A_BYTES + ko * BN * 16 + (kp & 3) * 4;
+            const int sw = ((oc >> 1) ^ (ko << 2)) & 15;
+#pragma unroll
+            for(int j = 0; j < 8; j++) sbj_off[j] = ((oc * 8 + j) ^ sw) * 16;
         } else {
-            /* A tile 128 rows x 32 k: 512 pieces of 8 k, two per thread */
+            const int n = tid & (BN - 1);
+            pw0 = a.d + ((P.wq + (size_t)(j0 + n) * a.K) >> 1);
+            wstep = BK >> 1;
+#pragma unroll
+            for(int ko = 0; ko < KO; ko++) sbj_off[ko] = A_BYTES + item_at<BN>(ko, n) * 16;
+        }
+    }
+    /* MFMA operand read offsets: [k16 half][tile] */
+    int ra_off[2][WM], rb_off[2][2];
+#pragma unroll
+    for(int ks = 0; ks < 2; ks++){
+#pragma unroll
+        for(int i = 0; i < WM; i++) ra_off[ks][i] = item_at<BM>(ks * 2 + hf, wi + i * 32 + fr) * 16;
+#pragma unroll
+        for(int j = 0; j < 2; j++) rb_off[ks][j] = A_BYTES + item_at<BN>(ks * 2 + hf, wj + j * 32 + fr) * 16;
+    }
+
+    struct Stage {
+        uint4 ra[NA];
+        uint4 rb[2];
+        uint4 rw;                                      /* nn: .x,.y digits of rows k,k+1; tn: 32 digits of one n row */
+        float rs0, rs1;
+    };
+    Stage S0, S1;
+    S0.rw = make_uint4(0, 0, 0, 0); S1.rw = S0.rw; S0.rs0 = S0.rs1 = S1.rs0 = S1.rs1 = 0.0f;
+
+    auto ld16 = [&](const char *p) -> uint4 {
+        if constexpr(BF16) return *(const uint4 *)p;
+        else return pk8_bf16((const float *)p);
+    };
+    /* loads the tile of the next step in program order (pointers advance as a side effect) */
+    auto load_step = [&](Stage &G, int p0){
+        if constexpr(MODE == GEMM_NT){
 #pragma unroll
             for(int h = 0; h < 2; h++){
-                const int piece = tid + 256 * h, r = piece >> 2, kq = piece & 3;
-                uint4 v = make_uint4(0, 0, 0, 0);
-                if(i0 + r < rows){
-                    if constexpr(BF16) v = *(const uint4 *)((const unsigned short *)P.A + (size_t)(i0 + r) * a.K + p0 + kq * 8);
-                    else {
-                        const float *pa = (const float *)P.A + (size_t)(i0 + r) * a.K + p0 + kq * 8;
-                        v = make_uint4(pack_bf16(pa[0], pa[1]), pack_bf16(pa[2], pa[3]), pack_bf16(pa[4], pa[5]), pack_bf16(pa[6], pa[7]));
-                    }
+                const int mp = (tid + 256 * h) >> 5;
+#pragma unroll
+                for(int e = 0; e < 2; e++){
+                    G.ra[2 * h + e] = (p0 + 2 * mp + e < depth) ? ld16(pa[2 * h + e]) : make_uint4(0, 0, 0, 0);
+                    pa[2 * h + e] += astep;
                 }
-                ra[h] = v;
             }
+            { const int mp = tid >> 4;
+#pragma unroll
+              for(int e = 0; e < 2; e++){
+                  G.rb[e] = (p0 + 2 * mp + e < depth) ? ld16(pb[e]) : make_uint4(0, 0, 0, 0);
+                  pb[e] += bstep;
+              } }
+        } else {
+#pragma unroll
+            for(int h = 0; h < WM; h++){ G.ra[h] = ld16(pa[h]); pa[h] += astep; }
             if constexpr(MODE == GEMM_NN){
-                /* W[k, n]: thread = (k pair 0..15, n octet 0..15) */
-                const int kp = tid & 15, oc = tid >> 4;
-#pragma unroll
-                for(int h = 0; h < 2; h++){
-                    const size_t e = (size_t)(p0 + 2 * kp + h) * a.N + j0 + oc * 8;
-                    rw[h] = *(const uint32_t *)(a.d + ((P.wq + e) >> 1));
-                    rs[h] = a.s[P.wg + e / (size_t)a.group];
-                }
+                G.rw.x = *(const uint32_t *)pw0; G.rw.y = *(const uint32_t *)pw1;
+                G.rs0 = *ps0; G.rs1 = *ps1;
+                pw0 += wstep; pw1 += wstep; ps0 += sstep; ps1 += sstep;
             } else {
-                /* W[n, k]: 128 rows x 4 k-octets = 512 dwords, two per thread */
-#pragma unroll
-                for(int h = 0; h < 2; h++){
-                    const int piece = tid + 256 * h, r = piece >> 2, kq = piece & 3;
-                    const size_t e = (size_t)(j0 + r) * a.K + p0 + kq * 8;
-                    rw[h] = *(const uint32_t *)(a.d + ((P.wq + e) >> 1));
-                }
+                if(tid < BN) G.rw = *(const uint4 *)pw0;
+                pw0 += wstep;
             }
         }
     };
 
-    auto store_step = [&](){
+    auto store_step = [&](const Stage &G, int nb){
+        unsigned char *L = lds + nb * BUF_BYTES;
         if constexpr(MODE == GEMM_NT){
-            const int pr_ = tid & 15, oc = tid >> 4;
-            const uint32_t a0[4] = {ra[0].x, ra[0].y, ra[0].z, ra[0].w}, a1[4] = {ra[1].x, ra[1].y, ra[1].z, ra[1].w};
-            const uint32_t b0[4] = {rb[0].x, rb[0].y, rb[0].z, rb[0].w}, b1[4] = {rb[1].x, rb[1].y, rb[1].z, rb[1].w};
-#pragma unroll
-            for(int j = 0; j < 8; j++){
-                const int w = j >> 1, sh = (j & 1) * 16;
-                const uint32_t pa = ((a0[w] >> sh) & 0xFFFFu) | (((a1[w] >> sh) & 0xFFFFu) << 16);
-                const uint32_t pb = ((b0[w] >> sh) & 0xFFFFu) | (((b1[w] >> sh) & 0xFFFFu) << 16);
-                *(uint32_t *)&As[(oc * 8 + j) * LDP + 2 * pr_] = pa;
-                *(uint32_t *)&Bs[(oc * 8 + j) * LDP + 2 * pr_] = pb;
-            }
-        } else {
 #pragma unroll
             for(int h = 0; h < 2; h++){
-                const int piece = tid + 256 * h, r = piece >> 2, kq = piece & 3;
-                *(uint4 *)&As[r * LDP + kq * 8] = ra[h];
+                const uint32_t x0[4] = {G.ra[2 * h].x, G.ra[2 * h].y, G.ra[2 * h].z, G.ra[2 * h].w};
+                const uint32_t x1[4] = {G.ra[2 * h + 1].x, G.ra[2 * h + 1].y, G.ra[2 * h + 1].z, G.ra[2 * h + 1].w};
+#pragma unroll
+                for(int j = 0; j < 8; j++)
+                    *(uint32_t *)(L + sa_off[h] + (sj_off[j] ^ (h * 128))) = __builtin_amdgcn_perm(x1[j >> 1], x0[j >> 1], (j & 1) ? 0x07060302u : 0x05040100u);
             }
+            { const uint32_t y0[4] = {G.rb[0].x, G.rb[0].y, G.rb[0].z, G.rb[0].w}, y1[4] = {G.rb[1].x, G.rb[1].y, G.rb[1].z, G.rb[1].w};
+#pragma unroll
+              for(int j = 0; j < 8; j++)
+                  *(uint32_t *)(L + sb_off + sbj_off[j]) = __builtin_amdgcn_perm(y1[j >> 1], y0[j >> 1], (j & 1) ? 0x07060302u : 0x05040100u); }
+        } else {
+#pragma unroll
+            for(int h = 0; h < WM; h++) *(uint4 *)(L + sa_off[h]) = G.ra[h];
             if constexpr(MODE == GEMM_NN){
-                const int kp = tid & 15, oc = tid >> 4;
 #pragma unroll
                 for(int j = 0; j < 8; j++){
-                    const float w0 = rs[0] * (float)qx_nib(rw[0], j), w1 = rs[1] * (float)qx_nib(rw[1], j);
-                    const unsigned short h0 = qx_f32_to_bf16(w0), h1 = qx_f32_to_bf16(w1);
-                    const float l0 = w0 - qx_bf16_to_f32(h0), l1 = w1 - qx_bf16_to_f32(h1);
-                    *(uint32_t *)&Bs[(oc * 8 + j) * LDP + 2 * kp] = (uint32_t)h0 | ((uint32_t)h1 << 16);
-                    *(uint32_t *)&Bs[BN * LDP + (oc * 8 + j) * LDP + 2 * kp] = pack_bf16(l0, l1);
+                    const float w0 = G.rs0 * (float)qx_nib(G.rw.x, j), w1 = G.rs1 * (float)qx_nib(G.rw.y, j);
+                    const uint32_t hi = pk_bf16(w0, w1);
+                    const float l0 = w0 - __uint_as_float(hi << 16), l1 = w1 - __uint_as_float(hi & 0xFFFF0000u);
+                    *(uint32_t *)(L + sb_off + sbj_off[j]) = hi;
+                    *(uint32_t *)(L + sb_off + B_BYTES + sbj_off[j]) = pk_bf16(l0, l1);
                 }
             } else {
+                if(tid < BN){
+                    const uint32_t wd[4] = {G.rw.x, G.rw.y, G.rw.z, G.rw.w};
 #pragma unroll
-                for(int h = 0; h < 2; h++){
-                    const int piece = tid + 256 * h, r = piece >> 2, kq = piece & 3;
-                    uint4 v;
-                    v.x = pack_bf16((float)qx_nib(rw[h], 0), (float)qx_nib(rw[h], 1));
-                    v.y = pack_bf16((float)qx_nib(rw[h], 2), (float)qx_nib(rw[h], 3));
-                    v.z = pack_bf16((float)qx_nib(rw[h], 4), (float)qx_nib(rw[h], 5));
-                    v.w = pack_bf16((float)qx_nib(rw[h], 6), (float)qx_nib(rw[h], 7));
-                    *(uint4 *)&Bs[r * LDP + kq * 8] = v;
+                    for(int ko = 0; ko < KO; ko++){
+                        uint4 v;
+                        v.x = pk_bf16((float)qx_nib(wd[ko], 0), (float)qx_nib(wd[ko], 1));
+                        v.y = pk_bf16((float)qx_nib(wd[ko], 2), (float)qx_nib(wd[ko], 3));
+                        v.z = pk_bf16((float)qx_nib(wd[ko], 4), (float)qx_nib(wd[ko], 5));
+                        v.w = pk_bf16((float)qx_nib(wd[ko], 6), (float)qx_nib(wd[ko], 7));
+                        *(uint4 *)(L + sbj_off[ko]) = v;
+                    }
                 }
             }
         }
     };
 
-    const int fr = lane & 31, fk = (lane >> 5) * 8;       /* operand row and k-offset of this lane */
-    const int steps = (depth + BK - 1) / BK;
-    const int steps_per_group = MODE == GEMM_TN ? a.group / BK : 0;
-
-    load_step(0);
-    for(int st = 0; st < steps; st++){
-        store_step();
-        __syncthreads();
-        if(st + 1 < steps) load_step((st + 1) * BK);
+    auto compute = [&](int cb){
+        const unsigned char *L = lds + cb * BUF_BYTES;
 #pragma unroll
-        for(int ks = 0; ks < BK; ks += 16){
-            bf16x8 fa[2], fb[2], fl[2];
+        for(int ks = 0; ks < 2; ks++){
+            bf16x8 fa[WM], fb[2], fl[2];
 #pragma unroll
-            for(int i = 0; i < 2; i++) fa[i] = lds_frag(&As[(wi + i * 32 + fr) * LDP + ks + fk]);
+            for(int i = 0; i < WM; i++) fa[i] = __builtin_bit_cast(bf16x8, *(const uint4 *)(L + ra_off[ks][i]));
 #pragma unroll
             for(int j = 0; j < 2; j++){
-                fb[j] = lds_frag(&Bs[(wj + j * 32 + fr) * LDP + ks + fk]);
-                if constexpr(MODE == GEMM_NN) fl[j] = lds_frag(&Bs[BN * LDP + (wj + j * 32 + fr) * LDP + ks + fk]);
+                fb[j] = __builtin_bit_cast(bf16x8, *(const uint4 *)(L + rb_off[ks][j]));
+                if constexpr(MODE == GEMM_NN) fl[j] = __builtin_bit_cast(bf16x8, *(const uint4 *)(L + rb_off[ks][j] + B_BYTES));
             }
 #pragma unroll
-            for(int i = 0; i < 2; i++)
+            for(int i = 0; i < WM; i++)
 #pragma unroll
                 for(int j = 0; j < 2; j++){
                     if constexpr(MODE == GEMM_TN){
@@ -210,33 +280,80 @@ __global__ void __launch_bounds__(256) k_gemm_mfma(MfmaArgs a){
                     }
                 }
         }
-        if(MODE == GEMM_TN && ((st + 1) % steps_per_group == 0)){
-            /* one scale group of the contraction is complete: fold it in with its fp32 scale */
-            const int chunk = (st * BK) / a.group;
+    };
+
+    const int steps = (depth + BK - 1) / BK;
+    const int steps_per_group = MODE == GEMM_TN ? (1 << a.gshift) / BK : 1;
+    const float *pfold[2] = {a.s, a.s};                /* tn: scale of (this lane's column, current group) */
+    if constexpr(MODE == GEMM_TN){
 #pragma unroll
-            for(int j = 0; j < 2; j++){
-                const int n = j0 + wj + j * 32 + fr;              /* this lane's output column */
-                const float sc = a.s[P.wg + (size_t)n * (a.K / a.group) + chunk];
+        for(int j = 0; j < 2; j++) pfold[j] = a.s + P.wg + (size_t)(j0 + wj + j * 32 + fr) * (a.K >> a.gshift);
+    }
+
+    auto fold_group = [&](int st){
+        if constexpr(MODE == GEMM_TN){
+            if((st + 1) % steps_per_group == 0){
+                /* one scale group of the contraction is complete: fold it in with its fp32 scale */
 #pragma unroll
-                for(int i = 0; i < 2; i++){
+                for(int j = 0; j < 2; j++){
+                    const float sc = *pfold[j]; pfold[j] += 1;
 #pragma unroll
-                    for(int v = 0; v < 16; v++) acc[i][j][v] = fmaf(sc, part[i][j][v], acc[i][j][v]);
-                    part[i][j] = (f32x16)(0.0f);
+                    for(int i = 0; i < WM; i++){
+#pragma unroll
+                        for(int v = 0; v < 16; v++) acc[i][j][v] = fmaf(sc, part[i][j][v], acc[i][j][v]);
+                        part[i][j] = (f32x16)(0.0f);
+                    }
                 }
             }
         }
+    };
+
+    /* step st computes from LDS buffer st&1. While it computes, the tile of step st+1 is written to
+     * the other buffer and the tile of a later step is requested from global memory (two steps ahead
+     * with DEEP, which keeps two sets of staging registers; one otherwise). */
+    if constexpr(DEEP){
+        load_step(S0, 0);
+        if(steps > 1) load_step(S1, BK);
+        store_step(S0, 0);
+        if(steps > 2) load_step(S0, 2 * BK);
         __syncthreads();
+        for(int st = 0; st < steps; st += 2){
+            compute(0);
+            if(st + 1 < steps) store_step(S1, 1);
+            if(st + 3 < steps) load_step(S1, (st + 3) * BK);
+            fold_group(st);
+            __syncthreads();
+            if(st + 1 < steps){
+                compute(1);
+                if(st + 2 < steps) store_step(S0, 0);
+                if(st + 4 < steps) load_step(S0, (st + 4) * BK);
+                fold_group(st + 1);
+                __syncthreads();
+            }
+        }
+    } else {
+        load_step(S0, 0);
+        store_step(S0, 0);
+        if(steps > 1) load_step(S0, BK);
+        __syncthreads();
+        for(int st = 0; st < steps; st++){
+            compute(st & 1);
+            if(st + 1 < steps) store_step(S0, (st + 1) & 1);
+            if(st + 2 < steps) load_step(S0, (st + 2) * BK);
+            fold_group(st);
+            __syncthreads();
+        }
     }
 
     /* ---- epilogue: lane holds column fr of each 32x32 tile, rows (v/4)*8 + (lane/32)*4 + v%4 ---- */
 #pragma unroll
-    for(int i = 0; i < 2; i++)
+    for(int i = 0; i < WM; i++)
 #pragma unroll
         for(int j = 0; j < 2; j++){
             const int c = j0 + wj + j * 32 + fr;
 #pragma unroll
             for(int v = 0; v < 16; v++){
-                const int r = i0 + wi + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                const int r = i0 + wi + i * 32 + (v >> 2) * 8 + hf * 4 + (v & 3);
                 if(r < rows){
                     float *o = P.C + (size_t)r * a.N + c;
                     *o = P.beta != 0.0f ? *o + acc[i][j][v] : acc[i][j][v];
@@ -245,15 +362,17 @@ __global__ void __launch_bounds__(256) k_gemm_mfma(MfmaArgs a){
         }
 }
 
-template<int MODE>
+template<int MODE, int WM, bool DEEP>
 static int launch_mfma(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob,
                        int K, int N, int act_dtype, hipStream_t st){
     ProbUpload up; int slot;
-    int rc = qlmx_upload_problems(probs, nprob, MODE, K, N, BM, BN, st, &up, &slot); if(rc) return rc;
+    int rc = qlmx_upload_problems(probs, nprob, MODE, K, N, 64 * WM, BN, st, &up, &slot); if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;
-    MfmaArgs a; a.pr = up.dev; a.nprob = up.nprob; a.d = d; a.s = s; a.group = group; a.K = K; a.N = N;
-    if(act_dtype == QLMX_ACT_BF16) hipLaunchKernelGGL((k_gemm_mfma<MODE, true>),  dim3(up.ntiles), dim3(256), 0, st, a);
-    else                           hipLaunchKernelGGL((k_gemm_mfma<MODE, false>), dim3(up.ntiles), dim3(256), 0, st, a);
+    MfmaArgs a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.tiles_n = N / BN; a.d = d; a.s = s; a.group = group; a.gshift = 0; while((1 << a.gshift) < group) a.gshift++; a.K = K; a.N = N;
+    int grid = (up.ntiles + 7) / 8 * 8;
+    if(MODE == GEMM_NT){ const int trows = up.ntiles / a.tiles_n; grid = 8 * a.tiles_n * ((trows + 7) / 8); }
+    if(act_dtype == QLMX_ACT_BF16) hipLaunchKernelGGL((k_gemm_mfma<MODE, true, WM, DEEP>),  dim3(grid), dim3(256), 0, st, a);
+    else                           hipLaunchKernelGGL((k_gemm_mfma<MODE, false, WM, DEEP>), dim3(grid), dim3(256), 0, st, a);
     QLMX_LAUNCH_CHECK("grouped gemm (mfma) launch");
     return qlmx_upload_done(slot, st);
 }
@@ -262,18 +381,16 @@ int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int 
                             const qlmx_gemm_prob *probs, int nprob, int K, int N, int act_dtype, hipStream_t st){
     /* shapes the tiling assumes; anything else must use QLMX_MATH_F32 */
     QLMX_REQUIRE(N % BN == 0, "mfma gemm: N=%d is not a multiple of %d (use QLMX_MATH_F32)", N, BN);
-    if(mode == GEMM_NT) QLMX_REQUIRE(K % BM == 0, "mfma gemm nt: K=%d is not a multiple of %d (use QLMX_MATH_F32)", K, BM);
+    if(mode == GEMM_NT) QLMX_REQUIRE(K % 8 == 0, "mfma gemm nt: K=%d is not a multiple of 8 (use QLMX_MATH_F32)", K);
     else                QLMX_REQUIRE(K % BK == 0, "mfma gemm: K=%d is not a multiple of %d (use QLMX_MATH_F32)", K, BK);
-    if(mode != GEMM_NT) QLMX_REQUIRE(group % BK == 0, "mfma gemm: group %d is not a multiple of %d", group, BK);
+    if(mode != GEMM_NT) QLMX_REQUIRE(group >= BK && (group & (group - 1)) == 0, "mfma gemm: group %d must be a power of two >= %d (use QLMX_MATH_F32)", group, BK);
     for(int i = 0; i < nprob; i++){
-        const int al = act_dtype == QLMX_ACT_BF16 ? 15 : 3;
-        QLMX_REQUIRE(((uintptr_t)probs[i].A & al) == 0 && (mode != GEMM_NT || ((uintptr_t)probs[i].B & al) == 0),
+        QLMX_REQUIRE(((uintptr_t)probs[i].A & 15) == 0 && (mode != GEMM_NT || ((uintptr_t)probs[i].B & 15) == 0),
                      "mfma gemm: problem %d operand is not 16-byte aligned", i);
-        QLMX_REQUIRE(mode == GEMM_NT || (probs[i].wq & 7ULL) == 0, "mfma gemm: problem %d weight offset not a multiple of 8", i);
+        QLMX_REQUIRE(mode == GEMM_NT || (probs[i].wq & 31ULL) == 0, "mfma gemm: problem %d weight offset not a multiple of 32", i);
     }
-    QLMX_REQUIRE(((uintptr_t)d & 3) == 0, "mfma gemm: digit array is not 4-byte aligned");
-    QLMX_REQUIRE(act_dtype != QLMX_ACT_BF16 || (K % 8 == 0 && N % 8 == 0), "mfma gemm: bf16 rows must be multiples of 8 elements");
-    if(mode == GEMM_NN) return launch_mfma<GEMM_NN>(d, s, group, probs, nprob, K, N, act_dtype, st);
-    if(mode == GEMM_TN) return launch_mfma<GEMM_TN>(d, s, group, probs, nprob, K, N, act_dtype, st);
-    return launch_mfma<GEMM_NT>(d, s, group, probs, nprob, K, N, act_dtype, st);
+    QLMX_REQUIRE(mode == GEMM_NT || ((uintptr_t)d & 15) == 0, "mfma gemm: digit array is not 16-byte aligned");
+    if(mode == GEMM_NN) return launch_mfma<GEMM_NN, 4, true>(d, s, group, probs, nprob, K, N, act_dtype, st);
+    if(mode == GEMM_TN) return launch_mfma<GEMM_TN, 2, false>(d, s, group, probs, nprob, K, N, act_dtype, st);
+    return launch_mfma<GEMM_NT, 4, false>(d, s, group, probs, nprob, K, N, act_dtype, st);
 }

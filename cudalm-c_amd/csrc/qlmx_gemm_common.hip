@@ -40,11 +40,11 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
         if(p.M == 0) continue;
         QLMX_REQUIRE(p.A && p.C, "grouped gemm: problem %d has a NULL operand", i);
         QLMX_REQUIRE(mode != GEMM_NT || p.B, "grouped gemm nt: problem %d has no B operand", i);
-        QLMX_REQUIRE(mode != GEMM_TN || p.beta == 0.0f || p.beta == 1.0f, "grouped gemm tn: beta must be 0 or 1");
+        QLMX_REQUIRE(p.beta == 0.0f || p.beta == 1.0f, "grouped gemm: beta must be 0 or 1");
         const int rows = mode == GEMM_NT ? K : p.M;
         DevProb &q = h[n++];
         q.A = p.A; q.B = p.B; q.C = p.C; q.wq = p.wq; q.wg = p.wg; q.M = p.M;
-        q.beta = mode == GEMM_TN ? p.beta : (mode == GEMM_NT ? 1.0f : 0.0f);
+        q.beta = mode == GEMM_NN ? 0.0f : p.beta;
         q.tile0 = (int)tiles; q.tiles_n = tiles_n;
         tiles += (long long)((rows + tile_rows - 1) / tile_rows) * tiles_n;
         QLMX_REQUIRE(tiles < (1LL << 30), "grouped gemm: too many tiles");

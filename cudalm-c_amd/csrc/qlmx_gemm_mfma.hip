@@ -182,21 +182,27 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
     /* loads the tile of the next step in program order (pointers advance as a side effect) */
     auto load_step = [&](Stage &G, int p0){
         if constexpr(MODE == GEMM_NT){
+            /* Rows past the end of the expert exist only in its last step. They are loaded from row 0
+             * (always valid) and zeroed when the tile is written to LDS: a load inside a branch would
+             * make every one of the six loads wait for the previous one. */
 #pragma unroll
             for(int h = 0; h < 2; h++){
                 const int mp = (tid + 256 * h) >> 5;
 #pragma unroll
                 for(int e = 0; e < 2; e++){
-                    G.ra[2 * h + e] = (p0 + 2 * mp + e < depth) ? ld16(pa[2 * h + e]) : make_uint4(0, 0, 0, 0);
+                    const char *q = (p0 + 2 * mp + e < depth) ? pa[2 * h + e] : (const char *)P.A;
+                    G.ra[2 * h + e] = ld16(q);
                     pa[2 * h + e] += astep;
                 }
             }
             { const int mp = tid >> 4;
 #pragma unroll
               for(int e = 0; e < 2; e++){
-                  G.rb[e] = (p0 + 2 * mp + e < depth) ? ld16(pb[e]) : make_uint4(0, 0, 0, 0);
+                  const char *q = (p0 + 2 * mp + e < depth) ? pb[e] : (const char *)P.B;
+                  G.rb[e] = ld16(q);
                   pb[e] += bstep;
               } }
+            G.rw.x = (uint32_t)p0;                     /* remembered for the zeroing at store time */
         } else {
 #pragma unroll
             for(int h = 0; h < WM; h++){ G.ra[h] = ld16(pa[h]); pa[h] += astep; }
@@ -214,15 +220,20 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
     auto store_step = [&](const Stage &G, int nb){
         unsigned char *L = lds + nb * BUF_BYTES;
         if constexpr(MODE == GEMM_NT){
+            const int p0 = (int)G.rw.x;
 #pragma unroll
             for(int h = 0; h < 2; h++){
-                const uint32_t x0[4] = {G.ra[2 * h].x, G.ra[2 * h].y, G.ra[2 * h].z, G.ra[2 * h].w};
-                const uint32_t x1[4] = {G.ra[2 * h + 1].x, G.ra[2 * h + 1].y, G.ra[2 * h + 1].z, G.ra[2 * h + 1].w};
+                const int m0 = p0 + 2 * ((tid + 256 * h) >> 5);
+                const uint32_t k0 = m0 < depth ? 0xFFFFFFFFu : 0u, k1 = m0 + 1 < depth ? 0xFFFFFFFFu : 0u;
+                const uint32_t x0[4] = {G.ra[2 * h].x & k0, G.ra[2 * h].y & k0, G.ra[2 * h].z & k0, G.ra[2 * h].w & k0};
+                const uint32_t x1[4] = {G.ra[2 * h + 1].x & k1, G.ra[2 * h + 1].y & k1, G.ra[2 * h + 1].z & k1, G.ra[2 * h + 1].w & k1};
 #pragma unroll
                 for(int j = 0; j < 8; j++)
                     *(uint32_t *)(L + sa_off[h] + (sj_off[j] ^ (h * 128))) = __builtin_amdgcn_perm(x1[j >> 1], x0[j >> 1], (j & 1) ? 0x07060302u : 0x05040100u);
             }
-            { const uint32_t y0[4] = {G.rb[0].x, G.rb[0].y, G.rb[0].z, G.rb[0].w}, y1[4] = {G.rb[1].x, G.rb[1].y, G.rb[1].z, G.rb[1].w};
+            { const int m0 = p0 + 2 * (tid >> 4);
+              const uint32_t k0 = m0 < depth ? 0xFFFFFFFFu : 0u, k1 = m0 + 1 < depth ? 0xFFFFFFFFu : 0u;
+              const uint32_t y0[4] = {G.rb[0].x & k0, G.rb[0].y & k0, G.rb[0].z & k0, G.rb[0].w & k0}, y1[4] = {G.rb[1].x & k1, G.rb[1].y & k1, G.rb[1].z & k1, G.rb[1].w & k1};
 #pragma unroll
               for(int j = 0; j < 8; j++)
                   *(uint32_t *)(L + sb_off + sbj_off[j]) = __builtin_amdgcn_perm(y1[j >> 1], y0[j >> 1], (j & 1) ? 0x07060302u : 0x05040100u); }
@@ -345,19 +356,31 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
         }
     }
 
-    /* ---- epilogue: lane holds column fr of each 32x32 tile, rows (v/4)*8 + (lane/32)*4 + v%4 ---- */
+    /* ---- epilogue: lane holds column fr of each 32x32 tile, rows (v/4)*8 + (lane/32)*4 + v%4.
+     * When accumulating, the 16 old values of a tile are all requested before the first store: a
+     * load-add-store chain per element would cost one memory round trip each. ---- */
+    const bool accumulate = P.beta != 0.0f;
 #pragma unroll
     for(int i = 0; i < WM; i++)
 #pragma unroll
         for(int j = 0; j < 2; j++){
-            const int c = j0 + wj + j * 32 + fr;
+            float *col = P.C + (size_t)(i0 + wi + i * 32 + hf * 4) * a.N + (j0 + wj + j * 32 + fr);
+            const int rbase = i0 + wi + i * 32 + hf * 4;
+            float old[16];
+            if(accumulate){
+#pragma unroll
+                for(int v = 0; v < 16; v++){
+                    const int ro = (v >> 2) * 8 + (v & 3);
+                    old[v] = (rbase + ro < rows) ? col[(size_t)ro * a.N] : 0.0f;
+                }
+            } else {
+#pragma unroll
+                for(int v = 0; v < 16; v++) old[v] = 0.0f;
+            }
 #pragma unroll
             for(int v = 0; v < 16; v++){
-                const int r = i0 + wi + i * 32 + (v >> 2) * 8 + hf * 4 + (v & 3);
-                if(r < rows){
-                    float *o = P.C + (size_t)r * a.N + c;
-                    *o = P.beta != 0.0f ? *o + acc[i][j][v] : acc[i][j][v];
-                }
+                const int ro = (v >> 2) * 8 + (v & 3);
+                if(rbase + ro < rows) col[(size_t)ro * a.N] = old[v] + acc[i][j][v];
             }
         }
 }

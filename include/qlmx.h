@@ -123,7 +123,8 @@ typedef struct qlmx_gemm_prob {
     unsigned long long wq;   /* nn/tn: element offset of the weight matrix in the digit array    */
     unsigned long long wg;   /* nn/tn: index of the matrix's first scale group                   */
     int   M;                 /* rows of A (0 is allowed and skipped)                             */
-    float beta;              /* tn: 0 or 1. nn is always beta=0, nt always accumulates           */
+    float beta;              /* tn, nt: 0 (overwrite C) or 1 (accumulate, the reference's mg_atb and
+                              * the second mg_abt_b of a pair). nn always overwrites.              */
 } qlmx_gemm_prob;
 
 /* nn: weights [K,N] row-major, scale groups run along N (N % group == 0). */
@@ -134,7 +135,8 @@ int qlmx_moe_gemm_nn(const signed char *d, const float *s, int group,
 int qlmx_moe_gemm_tn(const signed char *d, const float *s, int group,
                      const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
                      int act_dtype, int math, void *stream);
-/* nt: no weight operand; both inputs are activations, C accumulates in fp32. */
+/* nt: no weight operand; both inputs are activations, fp32 result. beta = 1 reproduces the
+ * reference's accumulation into a zeroed G; beta = 0 saves the read when G is known to be fresh. */
 int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
                      int act_dtype, int math, void *stream);
 

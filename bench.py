@@ -219,12 +219,12 @@ def bench_decode(torch, q, args, E=32, D=768, F=2048, topk=2, layers=8):
     head = out_all["T16"]
     gbs = max(head["gbs"], head.get("graph_gbs", 0.0))
     return {
-        "workload": "C2 decode: %d layers x (E=%d top-%d D=%d F=%d), T=16 tokens per step (T=1,4 listed beside); fused group+w1|w3+SwiGLU, w2, combine"
+        "workload": "C2 decode: %d layers x (E=%d top-%d D=%d F=%d), T=16 tokens per step (T=1,4 listed beside); one launch per layer: grouping, w1|w3, SwiGLU, w2, gated combine"
                     % (layers, E, topk, D, F),
         "metric": "QLM expert dequant-GEMV GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": min(head["ms_8_layers"], head.get("graph_ms_8_layers", 1e9)),
         "dtype": "u8+f32", "by_tokens": out_all, "bytes_per_expert_hit": per_expert,
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "k_qlmx_gemv<swiglu> + k_qlmx_gemv<store> (whole 8-layer sequence incl. group/combine kernels)"},
+                     "kernel": "k_decode_fused (one launch per layer; figure is the whole 8-layer sequence)"},
     }
 
 # --------------------------------------------------------------------------------------------- adamw

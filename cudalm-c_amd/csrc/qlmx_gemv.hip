@@ -2,21 +2,21 @@
  *
  * Serves the reference's decode step, where moe_forward runs on N = batch rows (dec_step,
  * cudalm.cu:7163-7204) and each expert GEMM of cudalm.cu:4211-4225 has at most a few rows: the
- * work is one pass over the hit experts' digits and scales. Also the small-row path of
- * qlmx_moe_gemm_nn (the reference's CPU SGEMM has the same split at R<=4, cpu_rt.h:233-258).
+ * work is one pass over the hit experts' digits and scales. Two parts: the small-row path of
+ * qlmx_moe_gemm_nn (the reference's CPU SGEMM has the same split at R<=4, cpu_rt.h:233-258), and
+ * further down the whole decode layer fused into one launch.
  *
  * y[m, n] = sum_k x[m, k] * s[k, n/group] * digit[k, n], W row-major [K, N].
  *
- * Mapping. A thread owns one 16-byte chunk column (32 consecutive n) and walks down the rows of
+ * Mapping of the small-row GEMV. A thread owns one 16-byte chunk column (32 consecutive n) and walks down the rows of
  * its workgroup's K-slice; consecutive threads own consecutive chunks, and when a row is narrower
  * than the workgroup the next threads continue on the following rows, so every load instruction
  * of a wave covers one contiguous 1 KiB of the weight matrix. Per chunk: xor 0x88888888 turns the
  * two's-complement nibbles into offset-8 bytes, two masks split even and odd nibbles, the
  * byte-to-float converts feed fp32 FMAs against x*s, and the offset (8 * sum of x*s) is taken out
  * once per row. The K dimension is split over workgroups for parallelism; slices leave partial sums
- * in a scratch buffer and whoever consumes them (the next stage's prologue, the combine kernel or
- * the finishing kernel) adds them in slice order, so results do not depend on scheduling and no
- * workgroup ever waits for another.
+ * in a scratch buffer and the finishing kernel adds them in slice order, so results do not depend on
+ * scheduling and no workgroup ever waits for another.
  *
  * Algorithmic HBM bytes per expert hit: K*N/2 digits + K*N/group*4 scales per matrix
  * (D=768, F=2048, three matrices: 2,506,752 B).
@@ -30,10 +30,9 @@
 #define GV_MAXSLICE 512       /* K rows per workgroup slice held in LDS */
 #define GV_BATCH 4            /* rows a thread has in flight */
 
-enum { PRO_ROWS = 0, PRO_SWIGLU = 1 };   /* where a problem's input rows come from */
 
 struct GvProb {               /* 64 bytes */
-    const float *x[GV_MAXROWS];   /* PRO_ROWS: the input rows (each K floats) */
+    const float *x[GV_MAXROWS];   /* the input rows (each K floats)           */
     float *out;                   /* finish kernel: [M, N] rows, pitch N      */
     unsigned long long wq, wg;
     int M, pad;
@@ -45,7 +44,6 @@ struct GvArgs {
     int nmat; unsigned long long mat_dq, mat_dg;     /* second matrix of a pair: +mat_dq elements, +mat_dg groups */
     int S, rps;                                      /* K slices, rows per slice */
     float *part;                                     /* out: [task][slice][MR][N] partial sums */
-    const float *prev; int prevS;                    /* PRO_SWIGLU: partial sums of the gate|up stage (its N == this K) */
 };
 
 __device__ __forceinline__ float ub(uint32_t w, int k){ return (float)((w >> (8 * k)) & 0xFFu); }
@@ -65,7 +63,7 @@ __device__ __forceinline__ float sum_slices(const float *src, size_t stride, int
     return v;
 }
 
-template<int PRO, int MR>
+template<int MR>
 __global__ void __launch_bounds__(GV_THREADS) k_qlmx_gemv(GvArgs a){
     __shared__ float xs[MR][GV_MAXSLICE];
     __shared__ float red[GV_THREADS * 33];
@@ -87,18 +85,7 @@ __global__ void __launch_bounds__(GV_THREADS) k_qlmx_gemv(GvArgs a){
     for(int i = tid; i < MR * a.rps; i += GV_THREADS){
         const int m = i / a.rps, r = i - m * a.rps;
         float v = 0.0f;
-        if(m < PM && kb0 + r < kb1){
-            if(PRO == PRO_ROWS) v = Pp->x[m][kb0 + r];
-            else {
-                /* x = silu(gate) * up, both summed over the previous stage's slices in slice order
-                 * (k_swiglu, cudalm.cu:2430-2432) */
-                const int ix = part_index(kb0 + r, a.K);
-                const float *g0 = a.prev + (((size_t)(2 * p) * a.prevS) * MR + m) * a.K + ix;
-                const float *u0 = a.prev + (((size_t)(2 * p + 1) * a.prevS) * MR + m) * a.K + ix;
-                const float g = sum_slices(g0, (size_t)MR * a.K, a.prevS), u = sum_slices(u0, (size_t)MR * a.K, a.prevS);
-                v = (g / (1.0f + expf(-g))) * u;
-            }
-        }
+        if(m < PM && kb0 + r < kb1) v = Pp->x[m][kb0 + r];
         xs[m][r] = v;
     }
     __syncthreads();
@@ -208,18 +195,10 @@ __global__ void __launch_bounds__(256) k_qlmx_gemv_finish(const GvProb *pr, cons
  * Workspace owned by the library (grow-only): partial sums, device problem tables and the row maps
  * of the fused decode layer.
  * ---------------------------------------------------------------------------------------- */
-struct GvWorkspace {
-    float *part[2] = {nullptr, nullptr}; size_t part_floats[2] = {0, 0};
-    GvProb *prob = nullptr;                 /* device problem table of the decode path: 2 x 64 */
-    int *meta = nullptr;
-};
+struct GvWorkspace { float *part[1] = {nullptr}; size_t part_floats[1] = {0}; };
 static GvWorkspace g_ws;
 
 static int ws_reserve(int which, size_t floats, hipStream_t st){
-    if(!g_ws.prob){
-        QLMX_HIP(hipMalloc((void **)&g_ws.prob, 2 * 64 * sizeof(GvProb)), "gemv problem table");
-        QLMX_HIP(hipMalloc((void **)&g_ws.meta, 512 * sizeof(int)), "gemv meta");
-    }
     if(floats > g_ws.part_floats[which]){
         QLMX_HIP(hipStreamSynchronize(st), "gemv workspace sync");
         if(g_ws.part[which]) QLMX_HIP(hipFree(g_ws.part[which]), "gemv workspace free");
@@ -243,9 +222,9 @@ static void choose_split(int K, int N, int ntask, int *S, int *rps){
     *S = s; *rps = r;
 }
 
-template<int PRO, int MR>
+template<int MR>
 static int launch_gemv(GvArgs &a, int ntask_max, hipStream_t st){
-    hipLaunchKernelGGL((k_qlmx_gemv<PRO, MR>), dim3(a.S, ntask_max), dim3(GV_THREADS), 0, st, a);
+    hipLaunchKernelGGL((k_qlmx_gemv<MR>), dim3(a.S, ntask_max), dim3(GV_THREADS), 0, st, a);
     QLMX_LAUNCH_CHECK("gemv launch");
     return QLMX_OK;
 }
@@ -272,12 +251,12 @@ int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const
     }
     if(n == 0) return QLMX_OK;
     GvArgs a; a.pr = d_tab; a.nprob_dev = nullptr; a.nprob = n; a.d = d; a.s = s; a.group = group; a.K = K; a.N = N;
-    a.nmat = 1; a.mat_dq = 0; a.mat_dg = 0; a.prev = nullptr; a.prevS = 0;
+    a.nmat = 1; a.mat_dq = 0; a.mat_dg = 0;
     choose_split(K, N, n, &a.S, &a.rps);
     int rc = ws_reserve(0, (size_t)n * a.S * GV_MAXROWS * N, st); if(rc) return rc;
     a.part = g_ws.part[0];
     QLMX_HIP(hipMemcpyAsync(d_tab, h_tab, (size_t)n * sizeof(GvProb), hipMemcpyHostToDevice, st), "gemv table h2d");
-    rc = launch_gemv<PRO_ROWS, GV_MAXROWS>(a, n, st); if(rc) return rc;
+    rc = launch_gemv<GV_MAXROWS>(a, n, st); if(rc) return rc;
     hipLaunchKernelGGL(k_qlmx_gemv_finish<GV_MAXROWS>, dim3((N + 255) / 256, n), dim3(256), 0, st, d_tab, g_ws.part[0], a.S, N);
     QLMX_LAUNCH_CHECK("gemv finish launch");
     QLMX_HIP(hipEventRecord(ev, st), "gemv table record"); used = true;
@@ -285,82 +264,452 @@ int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const
 }
 
 /* ------------------------------------------------------------------------------------------
- * Fused decode layer
+ * Fused decode layer: one launch for grouping, gate|up GEMV, SwiGLU, down GEMV and the gated
+ * combine (moe_forward on decode rows, cudalm.cu:4189-4228).
+ *
+ * At decode sizes a layer moves a few tens of MB, i.e. a handful of microseconds of HBM time, so a
+ * chain of launches costs more than the data. The layer therefore runs as one grid of resident
+ * workgroups that walk three task lists in order:
+ *   1. gate|up tasks  (problem, matrix w1|w3, 256-column chunk of F, K slice of D)  -> part1
+ *   2. down tasks     (problem, 256-column chunk of D, K slice of F)                -> part2
+ *      input rows h = silu(g) * u come from part1
+ *   3. combine tasks  (token, 256-column chunk of D): out += gate * y from part2, passes in order.
+ * Hand-over between lists: every partial sum is stored as one 8-byte word {value, epoch of this
+ * call}; a consumer re-reads a word until it carries the current epoch. There are no flags to set,
+ * clear or fence, and a consumer pays one memory round trip when its producer is already done.
+ * Every workgroup finishes all of its tasks of one list before it starts the next, tasks of list 1
+ * never wait, and the grid is sized to be co-resident, so the waits cannot deadlock; they are also
+ * bounded (DF_SPIN_LIMIT polls) and report through a status word in pinned host memory if ever
+ * exceeded. Partial sums are added in slice order by their consumer, so results do not depend on
+ * timing. The 8-byte words are written and read with device-scope atomic accesses, which go to the
+ * point where all XCDs (each has its own L2) agree, so no cache-wide write-back or invalidate is
+ * needed around them.
+ *
+ * A "problem" is up to DF_MB (pass, token) pairs that hit the same expert; every workgroup derives
+ * the same problem table from `assign` in LDS (stable counting sort by expert, the order of the
+ * reference's host permutation, cudalm.cu:3586-3599).
+ *
+ * Task kernel: 256 threads cover 16 rows x 256 columns per step (a lane owns 16 columns = 8 bytes of
+ * digits of one row; 16 lanes cover the 128 contiguous bytes of a row's chunk), two batches of
+ * DF_BATCH steps in flight (the next batch is requested before the current one is consumed). The
+ * input rows are staged in LDS already multiplied by the row's group scales, so the inner loop
+ * loads digits only. Tasks of one (problem, matrix) are given to workgroups of one XCD so that the
+ * 64-byte scale sectors shared by neighbouring chunks are fetched into one L2 only.
  * ---------------------------------------------------------------------------------------- */
 #define DEC_MAXPAIR 64
-/* meta layout (ints): [0] nprob, [1] invalid-expert flag, [8 + j] row of pair j,
- * [8 + 64 + r] pair of row r, [8 + 128 + r] problem*GV_MAXROWS + row-in-problem of row r */
+#define DF_THREADS 256
+#define DF_MB 4               /* pairs per problem */
+#define DF_CW 256             /* columns per task */
+#define DF_NG 2               /* scale groups per task row: group 128, or one when the group is a multiple of 256 */
+#define DF_RMAX 256           /* rows per task at most */
+#define DF_BATCH 8            /* steps (of 16 rows) per half task: a task is two halves of at most 128 rows */
+#define DF_SPIN_LIMIT (1 << 17)
+typedef unsigned long long u64;
 
-/* Groups the (pass, token) pairs by expert: a stable counting sort over j = k*T + n, i.e. rows are
- * ordered by (expert, pass, token), the order of the reference's host permutation
- * (cudalm.cu:3586-3599) applied to the merged passes. Experts with more than MR rows are cut into
- * several problems. One wavefront, lane j owns pair j; ranks come from 64 lane broadcasts, so no
- * serial chain of global-memory round trips sits in front of the first GEMV. */
-template<int MR>
-__global__ void __launch_bounds__(64) k_decode_group(const int *assign, int npair, int T, int E, int D, int F,
-                               const float *x, unsigned long long w1q, unsigned long long w2q, int group,
-                               GvProb *prob1, GvProb *prob2, int *meta){
-    __shared__ int rowpair[DEC_MAXPAIR], isstart[DEC_MAXPAIR];
-    const int j = threadIdx.x;
-    const bool live = j < npair;
-    int e = live ? assign[j] : 0x7FFFFFFF;
-    const bool bad = live && (unsigned)e >= (unsigned)E;
-    if(bad) e = 0x7FFFFFFE;                               /* sorts after every valid expert */
-    int rank = 0, pos = 0, cnt = 0;
-    for(int i = 0; i < DEC_MAXPAIR; i++){
-        const int ei = __shfl(e, i, 64);
-        rank += (ei < e) || (ei == e && i < j);
-        pos  += (ei == e && i < j);
-        cnt  += (ei == e);
-    }
-    isstart[j] = 0;
-    __syncthreads();
-    const bool start = live && !bad && (pos % MR == 0);
-    if(live && !bad){ rowpair[rank] = j; isstart[rank] = start ? 1 : 0; meta[8 + j] = rank; meta[8 + DEC_MAXPAIR + rank] = j; }
-    if(bad) meta[8 + j] = -1;
-    __syncthreads();
-    if(live && !bad){
-        const int first = rank - (pos % MR);              /* row of the problem's first pair */
-        int np = 0;
-        for(int r = 0; r < first; r++) np += isstart[r];
-        meta[8 + 2 * DEC_MAXPAIR + rank] = np * GV_MAXROWS + (pos % MR);
-        if(start){
-            const int M = min(MR, cnt - pos);
-            GvProb g1, g2;
-#pragma unroll
-            for(int m = 0; m < GV_MAXROWS; m++){
-                g1.x[m] = nullptr; g2.x[m] = nullptr;
-                if(m < M) g1.x[m] = x + (size_t)(rowpair[rank + m] % T) * D;
-            }
-            const unsigned long long eo = (unsigned long long)e * D * F;
-            g1.out = nullptr; g1.wq = w1q + eo; g1.wg = (w1q + eo) / group; g1.M = M; g1.pad = 0;
-            g2.out = nullptr; g2.wq = w2q + eo; g2.wg = (w2q + eo) / group; g2.M = M; g2.pad = 0;
-            prob1[np] = g1; prob2[np] = g2;
-        }
-    }
-    const unsigned long long sm = __ballot(start), bm = __ballot(bad);
-    if(j == 0){ meta[0] = __popcll(sm); meta[1] = bm ? 1 : 0; }
+struct DfArgs {
+    const float *x; const int *assign; const float *gate; float *out;
+    const signed char *d; const float *s;
+    u64 w1q, w3q, w2q; int group;
+    int T, K, E, D, F;
+    int R1, S1, NC1, R2, S2, NC2;
+    u64 *part1, *part2; unsigned epoch; unsigned *status;
+};
+
+struct DfMeta {
+    int nprob;
+    int p_e[DEC_MAXPAIR], p_M[DEC_MAXPAIR], p_row0[DEC_MAXPAIR];
+    int rowpair[DEC_MAXPAIR], pair_prob[DEC_MAXPAIR], pair_m[DEC_MAXPAIR];
+    int se[DEC_MAXPAIR], sj[DEC_MAXPAIR], ein[DEC_MAXPAIR], rk[4][DEC_MAXPAIR];
+};
+
+__device__ __forceinline__ void df_st(u64 *p, float v, unsigned epoch){
+    __hip_atomic_store(p, ((u64)epoch << 32) | (u64)__float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-/* out[n,:] += gate[k][n] * y[row(k,n),:], passes in order (cudalm.cu:4227); y is summed here from
- * the down-projection's slices in slice order. A pair whose expert index was out of range adds
- * nothing (the reference aborts the run in that case, cudalm.cu:3476-3478). */
-template<int MR>
-__global__ void __launch_bounds__(256) k_decode_combine(const float *part, int S, const float *gate, const int *meta,
-                                                        float *out, int T, int K, int D){
-    const int n = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
-    if(c >= D) return;
-    const int ix = part_index(c, D);
-    float o = out[(size_t)n * D + c];
-    for(int k = 0; k < K; k++){
-        const int j = k * T + n, row = meta[8 + j];
-        if(row < 0) continue;
-        const int pm = meta[8 + 2 * DEC_MAXPAIR + row], p = pm / GV_MAXROWS, m = pm - p * GV_MAXROWS;
-        const float *src = part + (((size_t)p * S) * MR + m) * D + ix;
-        const float y = sum_slices(src, (size_t)MR * D, S);
-        o = o + gate[j] * y;
+/* Sums of S tagged partial sums `stride` words apart from each of NSRC sources, in slice order;
+ * re-reads until every word carries `epoch`. All loads of a pass are issued before the first is
+ * looked at. */
+#define DF_SLICE_STEP 4
+template<int NSRC>
+__device__ __forceinline__ void df_sum_wait(const u64 *const (&src)[NSRC], size_t stride, int S, unsigned epoch,
+                                            volatile int *giveup, unsigned *status, float (&v)[NSRC]){
+    int spins = 0;
+    for(;;){
+        bool ok = true;
+#pragma unroll
+        for(int q = 0; q < NSRC; q++) v[q] = 0.0f;
+        for(int b = 0; b < S; b += DF_SLICE_STEP){
+            u64 t[NSRC][DF_SLICE_STEP];
+#pragma unroll
+            for(int q = 0; q < NSRC; q++)
+#pragma unroll
+                for(int u = 0; u < DF_SLICE_STEP; u++)
+                    t[q][u] = __hip_atomic_load(src[q] + (size_t)min(b + u, S - 1) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for(int q = 0; q < NSRC; q++)
+#pragma unroll
+                for(int u = 0; u < DF_SLICE_STEP; u++){
+                    ok = ok && (unsigned)(t[q][u] >> 32) == epoch;
+                    if(b + u < S) v[q] += __uint_as_float((unsigned)t[q][u]);
+                }
+        }
+        if(ok) break;
+        if(++spins > DF_SPIN_LIMIT || *giveup){ *(volatile unsigned *)status = 1u; *giveup = 1; break; }
+        __builtin_amdgcn_s_sleep(2);
     }
-    out[(size_t)n * D + c] = o;
+}
+
+/* Cheap wait in front of the tagged reads: thread i < n polls one word of producer i until it carries
+ * the epoch, then the workgroup meets. A producer's words become visible within a short time of each
+ * other, so the full read that follows rarely has to repeat, and while a producer is still busy only
+ * n threads per workgroup poll instead of all of them. */
+template<class ADDR>
+__device__ __forceinline__ void df_wait_first(int n, unsigned epoch, volatile int *giveup, unsigned *status, ADDR addr){
+    for(int i = threadIdx.x; i < n; i += DF_THREADS){
+        const u64 *p = addr(i);
+        if(!p) continue;
+        int spins = 0;
+        while((unsigned)(__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) != epoch){
+            if(++spins > DF_SPIN_LIMIT || *giveup){ *(volatile unsigned *)status = 1u; *giveup = 1; break; }
+            __builtin_amdgcn_s_sleep(4);
+        }
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ uint32_t df_and(uint32_t v){
+    uint32_t r; asm("v_and_b32 %0, %1, %2" : "=v"(r) : "s"(0x0F0F0F0Fu), "v"(v)); return r;
+}
+
+/* One task: which slice of which matrix, for which problem. list 0 = none. */
+struct DfT { u64 wq; int list, N, k0, rows, chunk, M, prob, mat, sl; };
+
+/* first DF_BATCH steps of a task's digits into W (the caller keeps them in flight across the end of
+ * the previous task) */
+__device__ __forceinline__ const signed char *df_digits(const DfArgs &a, const DfT &t){
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int cl = lane & 15, rp = wave * 4 + (lane >> 4);
+    const int col0 = t.chunk * DF_CW + cl * 16;
+    return a.d + ((t.wq + (size_t)(t.k0 + rp) * t.N + (col0 < t.N ? col0 : 0)) >> 1);
+}
+/* rows is a multiple of 16, so a step is live or not for the whole workgroup. Every load is issued
+ * unconditionally (a dead step re-reads step 0): loads under a branch make the compiler wait for
+ * each one where the branches join, which turns a batch into a chain of memory round trips. */
+#define DF_LOAD(W, dp, rowb, rows, hsteps, h)                                      \
+    _Pragma("unroll")                                                              \
+    for(int b = 0; b < DF_BATCH; b++){                                             \
+        const int st_ = (h) * (hsteps) + b;                                        \
+        const int sc_ = (b < (hsteps) && st_ * 16 < (rows)) ? st_ : 0;             \
+        W[b] = *(const uint2 *)((dp) + (size_t)sc_ * 16 * (rowb));                 \
+    }
+
+/* dst[m*mstride + chunk*256 + c] = sum_{r<rows} x[m][r] * s * digit(k0+r, chunk*256+c), m < M, stored
+ * tagged. w0, w1 hold the digits of the task's two halves, requested earlier. `prep` fills
+ * xs[m][g][r] = x[m][r] * scale(k0+r, column group g) and ends with a workgroup barrier. `next0`
+ * and `next1` request the following task's halves into w0 and w1 as soon as this task has consumed
+ * them, so the reduction, the stores and the next task's staging overlap that trip from HBM. */
+template<int MT, class PREP, class NEXT0, class NEXT1>
+__device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w0)[DF_BATCH], uint2 (&w1)[DF_BATCH], int hsteps,
+                                        const float (*xs)[DF_RMAX][DF_MB], float *red, u64 *dst, size_t mstride,
+                                        PREP prep, NEXT0 next0, NEXT1 next1){
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cl = lane & 15, rp = wave * 4 + (lane >> 4);
+    const int N = t.N, rows = t.rows, M = t.M, chunk = t.chunk;
+    const int gl = a.group >= DF_CW ? 0 : (cl >> 3);          /* this lane's scale group inside the chunk */
+    float acc[MT][16], corr[MT];
+#pragma unroll
+    for(int m = 0; m < MT; m++){ corr[m] = 0.0f;
+#pragma unroll
+        for(int j = 0; j < 16; j++) acc[m][j] = 0.0f; }
+    /* The nibble masks go through df_and so that the byte-to-float converts (one instruction per
+     * digit, v_cvt_f32_ubyteN) survive: seen through, the compiler rewrites mask + byte select into a
+     * bit-field extract per digit and doubles the instruction count. The four input values of a row
+     * sit side by side in LDS and come in with one 16-byte read. */
+#define DF_COMPUTE(W, h)                                                          \
+    _Pragma("unroll")                                                              \
+    for(int b = 0; b < DF_BATCH; b++){                                             \
+        if(b < hsteps && ((h) * hsteps + b) * 16 < rows){                          \
+            const int r = ((h) * hsteps + b) * 16 + rp;                            \
+            const float4 x4 = *(const float4 *)&xs[gl][r][0];                      \
+            const float xm[DF_MB] = {x4.x, x4.y, x4.z, x4.w};                      \
+            float f[16];                                                           \
+            const uint32_t u0 = W[b].x ^ 0x88888888u, u1 = W[b].y ^ 0x88888888u;   \
+            const uint32_t l0 = df_and(u0), h0 = df_and(u0 >> 4);                  \
+            const uint32_t l1 = df_and(u1), h1 = df_and(u1 >> 4);                  \
+            _Pragma("unroll")                                                      \
+            for(int k = 0; k < 4; k++){ f[2 * k] = ub(l0, k); f[2 * k + 1] = ub(h0, k); f[8 + 2 * k] = ub(l1, k); f[9 + 2 * k] = ub(h1, k); } \
+            _Pragma("unroll")                                                      \
+            for(int m = 0; m < MT; m++){                                           \
+                const float xv = xm[m];                                            \
+                corr[m] += xv;                                                     \
+                _Pragma("unroll")                                                  \
+                for(int j = 0; j < 16; j++) acc[m][j] = fmaf(xv, f[j], acc[m][j]); \
+            }                                                                      \
+        }                                                                          \
+    }
+    prep();
+    DF_COMPUTE(w0, 0)
+    next0();
+    DF_COMPUTE(w1, 1)
+    next1();
+#undef DF_COMPUTE
+    /* four row phases of a wave: reduce-scatter over lane bits 5 and 4, then the four waves via LDS */
+    const bool hi32 = lane & 32, hi16 = lane & 16;
+    __syncthreads();
+#pragma unroll
+    for(int m = 0; m < MT; m++){
+        if(m < M){
+            float k8[8], k4[4];
+            const float off = 8.0f * corr[m];
+#pragma unroll
+            for(int j = 0; j < 8; j++){
+                const float lo = acc[m][j] - off, hi = acc[m][8 + j] - off;
+                const float mine = hi32 ? hi : lo, send = hi32 ? lo : hi;
+                k8[j] = mine + __shfl_xor(send, 32, 64);
+            }
+#pragma unroll
+            for(int j = 0; j < 4; j++){
+                const float mine = hi16 ? k8[4 + j] : k8[j], send = hi16 ? k8[j] : k8[4 + j];
+                k4[j] = mine + __shfl_xor(send, 16, 64);
+            }
+            *(float4 *)&red[(wave * DF_MB + m) * DF_CW + cl * 16 + (hi32 ? 8 : 0) + (hi16 ? 4 : 0)] = make_float4(k4[0], k4[1], k4[2], k4[3]);
+        }
+    }
+    __syncthreads();
+    const int col = chunk * DF_CW + tid;
+    if(col < N){
+        for(int m = 0; m < M; m++){
+            const float v = ((red[(0 * DF_MB + m) * DF_CW + tid] + red[(1 * DF_MB + m) * DF_CW + tid])
+                           + red[(2 * DF_MB + m) * DF_CW + tid]) + red[(3 * DF_MB + m) * DF_CW + tid];
+            df_st(dst + (size_t)m * mstride + col, v, a.epoch);
+        }
+    }
+}
+
+/* scale of row r of the slice, column group g of the chunk; srow0 points at the slice's first row,
+ * chunk's first group */
+__device__ __forceinline__ float df_scale(const DfArgs &a, const float *srow0, int gpr, int N, int r, int chunk, int g){
+    if(chunk * DF_CW + g * a.group >= N) return 0.0f;
+    return srow0[(size_t)r * gpr + g];
+}
+
+__global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
+    __shared__ DfMeta mt;
+    __shared__ __align__(16) float xs[DF_NG][DF_RMAX][DF_MB];   /* x[m][r] * scale(r, g), the four m side by side */
+    __shared__ float red[4 * DF_MB * DF_CW];
+    __shared__ int giveup;
+    const int tid = threadIdx.x;
+    if(tid == 0) giveup = 0;
+    const int npair = a.T * a.K;
+    const int ng = a.group >= DF_CW ? 1 : DF_CW / a.group;
+
+    /* ---- problem table (identical in every workgroup): rank of pair j among (expert, j) ---- */
+    if(tid < DEC_MAXPAIR){
+        int e = 0x7FFFFFFF;
+        if(tid < npair){ e = a.assign[tid]; if((unsigned)e >= (unsigned)a.E) e = 0x7FFFFFFE; }   /* invalid: sorts after every valid expert */
+        mt.ein[tid] = e;
+    }
+    __syncthreads();
+    {
+        const int j = tid & 63, part = tid >> 6, e = mt.ein[j];
+        int rank = 0;
+        for(int i = part * 16; i < min(npair, part * 16 + 16); i++){
+            const int ei = mt.ein[i];
+            rank += (ei < e) || (ei == e && i < j);
+        }
+        mt.rk[part][j] = rank;
+    }
+    __syncthreads();
+    if(tid < 64){
+        const bool live = tid < npair;
+        const int e = mt.ein[tid];
+        const bool bad = live && e == 0x7FFFFFFE;
+        const int rank = mt.rk[0][tid] + mt.rk[1][tid] + mt.rk[2][tid] + mt.rk[3][tid];
+        if(live){ mt.se[rank] = e; mt.sj[rank] = tid; }
+        if(bad){ mt.pair_prob[tid] = -1; mt.pair_m[tid] = 0; }
+    }
+    __syncthreads();
+    if(tid < 64){
+        const bool live = tid < npair;
+        const int nvalid = __popcll(__ballot(live && mt.ein[tid] != 0x7FFFFFFE));
+        const int r = tid; const bool valid = r < nvalid;
+        const int er = valid ? mt.se[r] : -1;
+        const bool head = valid && (r == 0 || mt.se[r - 1] != er);
+        const u64 upto = r == 63 ? ~0ull : ((2ull << r) - 1ull);
+        const u64 hm = __ballot(head);
+        const int hidx = 63 - __clzll((long long)((hm & upto) | 1ull));
+        const u64 after = hm & ~upto;
+        const int nidx = after ? __ffsll((long long)after) - 1 : nvalid;
+        const int pos = r - hidx, cnt = nidx - hidx;
+        const bool start = valid && (pos % DF_MB == 0);
+        const u64 sm = __ballot(start);
+        const int prob = __popcll(sm & upto) - 1;
+        if(valid){
+            const int j = mt.sj[r];
+            mt.rowpair[r] = j; mt.pair_prob[j] = prob; mt.pair_m[j] = pos % DF_MB;
+            if(start){ mt.p_e[prob] = er; mt.p_M[prob] = min(DF_MB, cnt - pos); mt.p_row0[prob] = r; }
+        }
+        if(tid == 0) mt.nprob = __popcll(sm);
+    }
+    __syncthreads();
+    const int nprob = mt.nprob;
+    const int G = gridDim.x, xcd = blockIdx.x & 7, slot0 = blockIdx.x >> 3, nslot = G >> 3;
+    const u64 DF = (u64)a.D * a.F;
+
+    /* ---- this workgroup's tasks, list 1 (gate|up) then list 2 (down), in one stream so that the
+     * first digits of a task are already on their way while the task before it finishes ---- */
+    const int tpg1 = a.NC1 * a.S1, ngrp1 = 2 * nprob, lim1 = ((ngrp1 + 7) >> 3) * tpg1;
+    const int tpg2 = a.NC2 * a.S2, lim2 = ((nprob + 7) >> 3) * tpg2;
+    int list = 1, q = slot0;
+    auto fetch = [&]() -> DfT {
+        DfT t; t.list = 0; t.wq = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = 0;
+        for(;;){
+            if(list == 1){
+                if(q >= lim1){ list = 2; q = slot0; continue; }
+                const int g = (q / tpg1) * 8 + xcd, sub = q % tpg1; q += nslot;
+                if(g >= ngrp1) continue;
+                t.list = 1; t.prob = g >> 1; t.mat = g & 1; t.chunk = sub / a.S1; t.sl = sub - t.chunk * a.S1;
+                t.N = a.F; t.k0 = t.sl * a.R1; t.rows = min(a.R1, a.D - t.k0); t.M = mt.p_M[t.prob];
+                t.wq = (t.mat ? a.w3q : a.w1q) + (u64)mt.p_e[t.prob] * DF;
+                return t;
+            }
+            if(list == 2){
+                if(q >= lim2){ list = 3; return t; }
+                const int prob = (q / tpg2) * 8 + xcd, sub = q % tpg2; q += nslot;
+                if(prob >= nprob) continue;
+                t.list = 2; t.prob = prob; t.mat = 0; t.chunk = sub / a.S2; t.sl = sub - t.chunk * a.S2;
+                t.N = a.D; t.k0 = t.sl * a.R2; t.rows = min(a.R2, a.F - t.k0); t.M = mt.p_M[prob];
+                t.wq = a.w2q + (u64)mt.p_e[prob] * DF;
+                return t;
+            }
+            return t;
+        }
+    };
+    uint2 w0[DF_BATCH], w1[DF_BATCH];
+    const int hs1 = a.R1 >> 5, hs2 = a.R2 >> 5;               /* steps per half task */
+    DfT cur = fetch();
+    if(cur.list){
+        const signed char *dp = df_digits(a, cur); const int hs = cur.list == 1 ? hs1 : hs2;
+        DF_LOAD(w0, dp, (size_t)cur.N >> 1, cur.rows, hs, 0)
+        DF_LOAD(w1, dp, (size_t)cur.N >> 1, cur.rows, hs, 1)
+    }
+    while(cur.list){
+        const DfT nxt = fetch();
+        /* after the last task the same loads go to the current task's digits again and are dropped */
+        const DfT &pre = nxt.list ? nxt : cur;
+        const signed char *ndp = df_digits(a, pre); const int nhs = pre.list == 1 ? hs1 : hs2;
+        auto next0 = [&](){ DF_LOAD(w0, ndp, (size_t)pre.N >> 1, pre.rows, nhs, 0) };
+        auto next1 = [&](){ DF_LOAD(w1, ndp, (size_t)pre.N >> 1, pre.rows, nhs, 1) };
+        const int hs = cur.list == 1 ? hs1 : hs2;
+        const int prob = cur.prob, chunk = cur.chunk, k0 = cur.k0, rows = cur.rows, M = cur.M;
+        const int gpr = cur.N / a.group;
+        const float *srow0 = a.s + cur.wq / (u64)a.group + (size_t)k0 * gpr + (chunk * DF_CW) / a.group;
+        u64 *dst; size_t mstride;
+        if(cur.list == 1){ dst = a.part1 + ((((size_t)prob * 2 + cur.mat) * a.S1 + cur.sl) * DF_MB) * a.F; mstride = (size_t)a.F; }
+        else             { dst = a.part2 + (((size_t)prob * a.S2 + cur.sl) * DF_MB) * a.D;                  mstride = (size_t)a.D; }
+        auto prep = [&](){
+            if(cur.list == 1){
+                __syncthreads();                             /* the previous task is done with xs */
+                if(tid < rows){
+                    float sc[DF_NG], xv[DF_MB];
+#pragma unroll
+                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = gg < ng ? df_scale(a, srow0, gpr, a.F, tid, chunk, gg) : 0.0f;
+#pragma unroll
+                    for(int m = 0; m < DF_MB; m++)
+                        xv[m] = m < M ? a.x[(size_t)(mt.rowpair[mt.p_row0[prob] + m] % a.T) * a.D + k0 + tid] : 0.0f;
+#pragma unroll
+                    for(int gg = 0; gg < DF_NG; gg++)
+                        *(float4 *)&xs[gg][tid][0] = make_float4(xv[0] * sc[gg], xv[1] * sc[gg], xv[2] * sc[gg], xv[3] * sc[gg]);
+                }
+                __syncthreads();
+            } else {
+                const u64 *p1 = a.part1 + (((size_t)prob * 2) * a.S1 * DF_MB) * a.F + k0;
+                const size_t sstride = (size_t)DF_MB * a.F;
+                df_wait_first(2 * a.S1, a.epoch, &giveup, a.status, [=](int i){ return p1 + (size_t)i * sstride; });
+                if(tid < rows){
+                    float sc[DF_NG];
+#pragma unroll
+                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = gg < ng ? df_scale(a, srow0, gpr, a.D, tid, chunk, gg) : 0.0f;
+                    float hv[DF_MB];
+#pragma unroll
+                    for(int m = 0; m < DF_MB; m++){
+                        hv[m] = 0.0f;
+                        if(m < M){
+                            /* h = silu(gate) * up (k_swiglu, cudalm.cu:2430-2432), both summed over the K slices in order */
+                            const u64 *const src[2] = { p1 + (size_t)m * a.F + tid, p1 + (size_t)a.S1 * sstride + (size_t)m * a.F + tid };
+                            float gu[2];
+                            df_sum_wait<2>(src, sstride, a.S1, a.epoch, &giveup, a.status, gu);
+                            hv[m] = (gu[0] / (1.0f + expf(-gu[0]))) * gu[1];
+                        }
+                    }
+#pragma unroll
+                    for(int gg = 0; gg < DF_NG; gg++)
+                        *(float4 *)&xs[gg][tid][0] = make_float4(hv[0] * sc[gg], hv[1] * sc[gg], hv[2] * sc[gg], hv[3] * sc[gg]);
+                }
+                __syncthreads();
+            }
+        };
+        /* the inner loop is compiled for 1, 2 and 4 input rows (3 runs as 4 with a zero row) */
+        if(M == 1)      df_task<1>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1);
+        else if(M == 2) df_task<2>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1);
+        else            df_task<4>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1);
+        cur = nxt;
+    }
+    /* ---- 3. out[n,:] += gate[k][n] * y[row(k,n),:], passes in order (cudalm.cu:4227). A pair whose
+     * expert index was out of range adds nothing (the reference aborts the run, cudalm.cu:3476-3478). ---- */
+    {
+        const int ntask = a.T * a.NC2;
+        for(int q3 = blockIdx.x; q3 < ntask; q3 += G){
+            const int n = q3 / a.NC2, chunk = q3 - n * a.NC2;
+            const int col = chunk * DF_CW + tid;
+            {
+                const int S2 = a.S2, T = a.T, Dd = a.D; const int *pp = mt.pair_prob, *pm = mt.pair_m; const u64 *p2 = a.part2;
+                df_wait_first(a.K * S2, a.epoch, &giveup, a.status, [=](int i) -> const u64 * {
+                    const int j = (i / S2) * T + n, prob = pp[j];
+                    if(prob < 0) return nullptr;
+                    return p2 + (((size_t)prob * S2 + i % S2) * DF_MB + pm[j]) * Dd + chunk * DF_CW; });
+            }
+            if(col < a.D){
+                float o = a.out[(size_t)n * a.D + col];
+                for(int k = 0; k < a.K; k++){
+                    const int j = k * a.T + n, prob = mt.pair_prob[j];
+                    if(prob < 0) continue;
+                    const u64 *const src[1] = { a.part2 + (((size_t)prob * a.S2) * DF_MB + mt.pair_m[j]) * a.D + col };
+                    float y[1];
+                    df_sum_wait<1>(src, (size_t)DF_MB * a.D, a.S2, a.epoch, &giveup, a.status, y);
+                    o = o + a.gate[j] * y[0];
+                }
+                a.out[(size_t)n * a.D + col] = o;
+            }
+        }
+    }
+}
+#undef DF_LOAD
+
+struct DfWorkspace { u64 *part[2] = {nullptr, nullptr}; size_t words[2] = {0, 0}; unsigned *status = nullptr; unsigned epoch = 0; int grid = 0; };
+static DfWorkspace g_df;
+
+/* tagged partial sums: grow-only, cleared when (re)allocated so that no word carries a live epoch */
+static int df_reserve(int which, size_t words, hipStream_t st){
+    if(words <= g_df.words[which]) return QLMX_OK;
+    QLMX_HIP(hipStreamSynchronize(st), "decode workspace sync");
+    if(g_df.part[which]) QLMX_HIP(hipFree(g_df.part[which]), "decode workspace free");
+    g_df.part[which] = nullptr; g_df.words[which] = 0;
+    QLMX_HIP(hipMalloc((void **)&g_df.part[which], words * sizeof(u64)), "decode partial sums");
+    QLMX_HIP(hipMemset(g_df.part[which], 0, words * sizeof(u64)), "decode partial sums clear");
+    g_df.words[which] = words;
+    return QLMX_OK;
+}
+
+/* rows per task: 256 keeps the per-task fixed cost (staging, reduction, hand-over) small against
+ * the streaming part; only when even that leaves most of the grid without a gate|up task (a single
+ * token) are the slices halved. The number of problems is only known on the device; the host uses
+ * the expected number of distinct experts hit by `npair` uniform picks out of E. */
+static int df_rows(int Kdim, double tasks_per_slice, int grid){
+    int R = DF_RMAX;
+    while(R > 64 && tasks_per_slice * ((Kdim + R - 1) / R) < 0.25 * grid) R >>= 1;
+    while((Kdim + R - 1) / R > 32 && R < DF_RMAX) R <<= 1;
+    return R;
 }
 
 extern "C" int qlmx_moe_decode_forward(const float *x, const int *assign, const float *gate, float *out,
@@ -370,38 +719,45 @@ extern "C" int qlmx_moe_decode_forward(const float *x, const int *assign, const 
     int rc = qlmx_check_ready(); if(rc) return rc;
     hipStream_t st = (hipStream_t)stream;
     QLMX_REQUIRE(x && assign && gate && out && d && s, "qlmx_moe_decode_forward: NULL buffer");
-    QLMX_REQUIRE(T > 0 && K > 0 && E > 0 && E <= 256, "qlmx_moe_decode_forward: T=%d K=%d E=%d", T, K, E);
+    QLMX_REQUIRE(T > 0 && K > 0 && E > 0, "qlmx_moe_decode_forward: T=%d K=%d E=%d", T, K, E);
     if(T * K > DEC_MAXPAIR){ qlmx_set_error("qlmx_moe_decode_forward: %d (pass, token) pairs exceed the limit of %d", T * K, DEC_MAXPAIR); return QLMX_E_LIMIT; }
     QLMX_REQUIRE(D % 32 == 0 && F % 32 == 0 && D <= 8192 && F <= 8192, "qlmx_moe_decode_forward: D=%d F=%d must be multiples of 32, at most 8192", D, F);
-    QLMX_REQUIRE(group % 32 == 0 && F % group == 0 && D % group == 0, "qlmx_moe_decode_forward: group %d must divide D and F", group);
-    QLMX_REQUIRE(w1q % 32 == 0 && w3q % 32 == 0 && w2q % 32 == 0 && ((uintptr_t)d & 15) == 0, "qlmx_moe_decode_forward: weight offsets must be multiples of 32 elements");
-    QLMX_REQUIRE(w3q >= w1q, "qlmx_moe_decode_forward: w3 must follow w1 in the digit array");
-    const int npair = T * K;
-    const int MR = T == 1 ? 1 : 2;
-    GvArgs a1, a2;
-    a1.nmat = 2; a2.nmat = 1;
-    choose_split(D, F, 2 * npair, &a1.S, &a1.rps);
-    choose_split(F, D, npair, &a2.S, &a2.rps);
-    rc = ws_reserve(0, (size_t)npair * 2 * a1.S * MR * F, st); if(rc) return rc;
-    rc = ws_reserve(1, (size_t)npair * a2.S * MR * D, st); if(rc) return rc;
-    GvProb *p1 = g_ws.prob, *p2 = g_ws.prob + 64;
-    if(MR == 1) hipLaunchKernelGGL(k_decode_group<1>, dim3(1), dim3(64), 0, st, assign, npair, T, E, D, F, x, w1q, w2q, group, p1, p2, g_ws.meta);
-    else        hipLaunchKernelGGL(k_decode_group<2>, dim3(1), dim3(64), 0, st, assign, npair, T, E, D, F, x, w1q, w2q, group, p1, p2, g_ws.meta);
-    QLMX_LAUNCH_CHECK("decode group launch");
-    a1.pr = p1; a1.nprob_dev = g_ws.meta; a1.nprob = npair; a1.d = d; a1.s = s; a1.group = group; a1.K = D; a1.N = F;
-    a1.mat_dq = w3q - w1q; a1.mat_dg = (w3q - w1q) / group; a1.part = g_ws.part[0]; a1.prev = nullptr; a1.prevS = 0;
-    a2.pr = p2; a2.nprob_dev = g_ws.meta; a2.nprob = npair; a2.d = d; a2.s = s; a2.group = group; a2.K = F; a2.N = D;
-    a2.mat_dq = 0; a2.mat_dg = 0; a2.part = g_ws.part[1]; a2.prev = g_ws.part[0]; a2.prevS = a1.S;
-    const dim3 cg((D + 255) / 256, T);
-    if(MR == 1){
-        rc = launch_gemv<PRO_ROWS, 1>(a1, 2 * npair, st); if(rc) return rc;
-        rc = launch_gemv<PRO_SWIGLU, 1>(a2, npair, st); if(rc) return rc;
-        hipLaunchKernelGGL(k_decode_combine<1>, cg, dim3(256), 0, st, g_ws.part[1], a2.S, gate, g_ws.meta, out, T, K, D);
-    } else {
-        rc = launch_gemv<PRO_ROWS, 2>(a1, 2 * npair, st); if(rc) return rc;
-        rc = launch_gemv<PRO_SWIGLU, 2>(a2, npair, st); if(rc) return rc;
-        hipLaunchKernelGGL(k_decode_combine<2>, cg, dim3(256), 0, st, g_ws.part[1], a2.S, gate, g_ws.meta, out, T, K, D);
+    QLMX_REQUIRE(group == 128 || (group > 0 && group % DF_CW == 0), "qlmx_moe_decode_forward: group %d is not supported (128 or a multiple of 256)", group);
+    QLMX_REQUIRE(F % group == 0 && D % group == 0, "qlmx_moe_decode_forward: group %d must divide D and F", group);
+    QLMX_REQUIRE(w1q % group == 0 && w3q % group == 0 && w2q % group == 0 && ((uintptr_t)d & 15) == 0,
+                 "qlmx_moe_decode_forward: weight offsets must be multiples of the group and the digit array 16-byte aligned");
+    if(!g_df.status){
+        QLMX_HIP(hipHostMalloc((void **)&g_df.status, 64, hipHostMallocDefault), "decode status word");
+        *g_df.status = 0;
+        int nb = 0, dev = 0; hipDeviceProp_t pr;
+        QLMX_HIP(hipGetDevice(&dev), "decode device");
+        QLMX_HIP(hipGetDeviceProperties(&pr, dev), "decode device properties");
+        QLMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, k_decode_fused, DF_THREADS, 0), "decode occupancy");
+        if(nb > 3) nb = 3;
+        g_df.grid = (nb * pr.multiProcessorCount) & ~7;
+        QLMX_REQUIRE(g_df.grid >= 8, "qlmx_moe_decode_forward: device too small (%d resident workgroups)", g_df.grid);
     }
-    QLMX_LAUNCH_CHECK("decode combine launch");
+    if(*(volatile unsigned *)g_df.status){
+        *g_df.status = 0;
+        qlmx_set_error("qlmx_moe_decode_forward: an earlier call gave up waiting for a task of its own grid; its output is invalid");
+        return QLMX_E_HIP;
+    }
+    const int npair = T * K;
+    DfArgs a;
+    a.x = x; a.assign = assign; a.gate = gate; a.out = out; a.d = d; a.s = s; a.w1q = w1q; a.w3q = w3q; a.w2q = w2q; a.group = group;
+    a.T = T; a.K = K; a.E = E; a.D = D; a.F = F;
+    a.NC1 = (F + DF_CW - 1) / DF_CW; a.NC2 = (D + DF_CW - 1) / DF_CW;
+    const double hits = E * (1.0 - pow(1.0 - 1.0 / E, (double)npair));
+    a.R1 = df_rows(D, 2.0 * hits * a.NC1, g_df.grid); a.S1 = (D + a.R1 - 1) / a.R1;
+    a.R2 = DF_RMAX;                                     a.S2 = (F + a.R2 - 1) / a.R2;
+    rc = df_reserve(0, (size_t)npair * 2 * a.S1 * DF_MB * F, st); if(rc) return rc;
+    rc = df_reserve(1, (size_t)npair * a.S2 * DF_MB * D, st); if(rc) return rc;
+    a.part1 = g_df.part[0]; a.part2 = g_df.part[1]; a.status = g_df.status;
+    a.epoch = ++g_df.epoch;
+    if(a.epoch == 0) a.epoch = ++g_df.epoch;          /* 0 is the cleared state */
+    const long long most = (long long)2 * npair * a.NC1 * a.S1;
+    const int grid = (int)std::min<long long>(g_df.grid, (most + 7) & ~7LL);
+    hipLaunchKernelGGL(k_decode_fused, dim3(grid), dim3(DF_THREADS), 0, st, a);
+    QLMX_LAUNCH_CHECK("decode launch");
     return QLMX_OK;
 }

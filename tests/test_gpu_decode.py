@@ -112,6 +112,77 @@ def test_decode_all_tokens_one_expert(q, orc):
     assert orc.relerr(out.cpu().numpy(), want) < 2e-5
 
 
+def test_decode_group_256_and_rejected_groups(q, orc):
+    """Scale groups of 256 (one per task row) go through the same kernel; 64 and 96 are refused."""
+    import torch
+    T, E, D, F, K = 4, 4, 512, 768, 2
+    d, s, P, n = encode_layer(orc, 21, E, D, F, group=256)
+    x = orc.normal(T * D, 21, 2)
+    rt = orc.normal(T * E, 21, 3)
+    pr = np.zeros(T * E, f32); asn = np.zeros(K * T, np.int32); gate = np.zeros(K * T, f32)
+    orc.router_topk(rt, pr, asn, gate, T, E, K)
+    want = np.zeros(T * D, f32)
+    rc, ws = orc.moe_forward(x, P[:n], P[n:2 * n], P[2 * n:], asn, gate, want, T, D, F, E, K)
+    orc.moe_ws_free(ws)
+    out = torch.zeros(T * D, device="cuda")
+    q.decode_forward(dev(x), dev(asn), dev(gate), out, dev(d), dev(s), 256, 0, n, 2 * n, T, K, E, D, F)
+    torch.cuda.synchronize()
+    assert orc.relerr(out.cpu().numpy(), want) < 2e-5
+    for g in (64, 96):
+        with pytest.raises(pkg.QlmxError, match="group"):
+            q.decode_forward(dev(x), dev(asn), dev(gate), out, dev(d), dev(s), g, 0, n, 2 * n, T, K, E, D, F)
+
+
+def test_decode_invalid_expert_is_skipped(q, orc):
+    """A pair with an out-of-range expert adds nothing; the other pairs are unaffected."""
+    import torch
+    T, E, D, F, K = 3, 4, 256, 512, 2
+    d, s, P, n = encode_layer(orc, 9, E, D, F)
+    x = orc.normal(T * D, 9, 2)
+    asn = np.array([1, 3, 0, 2, 1, 3], np.int32)          # [k][t]
+    gate = orc.uniform(K * T, 9, 3, 0.1, 0.6)
+    bad = asn.copy(); bad[4] = 7                          # pass 1, token 1 -> expert 7 of 4
+    gate_ref = gate.copy(); gate_ref[4] = 0.0             # the reference result with that pair's weight zeroed
+    want = np.zeros(T * D, f32)
+    rc, ws = orc.moe_forward(x, P[:n], P[n:2 * n], P[2 * n:], asn, gate_ref, want, T, D, F, E, K)
+    orc.moe_ws_free(ws)
+    out = torch.zeros(T * D, device="cuda")
+    q.decode_forward(dev(x), dev(bad), dev(gate), out, dev(d), dev(s), 128, 0, n, 2 * n, T, K, E, D, F)
+    torch.cuda.synchronize()
+    assert orc.relerr(out.cpu().numpy(), want) < 2e-5
+    allbad = np.full(K * T, -1, np.int32)
+    out.zero_()
+    q.decode_forward(dev(x), dev(allbad), dev(gate), out, dev(d), dev(s), 128, 0, n, 2 * n, T, K, E, D, F)
+    torch.cuda.synchronize()
+    assert float(out.abs().max()) == 0.0
+
+
+def test_decode_repeated_calls_alternating_shapes(q, orc):
+    """The hand-over words carry the call's epoch: stale partial sums of earlier calls, of other
+    shapes and token counts, must never be taken for current ones."""
+    import torch
+    cases = []
+    for (T, E, D, F, K, seed) in [(16, 8, 256, 512, 2, 31), (1, 8, 256, 512, 2, 32), (5, 4, 512, 256, 3, 33)]:
+        d, s, P, n = encode_layer(orc, seed, E, D, F)
+        x = orc.normal(T * D, seed, 2)
+        rt = orc.normal(T * E, seed, 3)
+        pr = np.zeros(T * E, f32); asn = np.zeros(K * T, np.int32); gate = np.zeros(K * T, f32)
+        orc.router_topk(rt, pr, asn, gate, T, E, K)
+        want = np.zeros(T * D, f32)
+        rc, ws = orc.moe_forward(x, P[:n], P[n:2 * n], P[2 * n:], asn, gate, want, T, D, F, E, K)
+        orc.moe_ws_free(ws)
+        cases.append((T, E, D, F, K, n, dev(x), dev(asn), dev(gate), dev(d), dev(s), want))
+    outs = []
+    for rep in range(12):
+        T, E, D, F, K, n, x, asn, gate, d, s, want = cases[rep % 3]
+        out = torch.zeros(T * D, device="cuda")
+        q.decode_forward(x, asn, gate, out, d, s, 128, 0, n, 2 * n, T, K, E, D, F)
+        outs.append((out, want))
+    torch.cuda.synchronize()
+    for out, want in outs:
+        assert orc.relerr(out.cpu().numpy(), want) < 2e-5
+
+
 def test_decode_limits(q):
     import torch
     z = torch.zeros(65536, device="cuda")

@@ -1,6 +1,7 @@
 /* qlmx_gemm_common.hip -- problem-table upload ring and argument checks of the grouped GEMMs. */
 #include "qlmx_gemm.h"
 #include <string.h>
+#include <algorithm>
 
 #define RING_SLOTS 64
 static DevProb   *g_ring_h = nullptr, *g_ring_d = nullptr;
@@ -34,7 +35,24 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
     DevProb *dv = g_ring_d + (size_t)slot * QLMX_MAX_PROBLEMS;
     const int tiles_n = (N + tile_cols - 1) / tile_cols;
     long long tiles = 0; int n = 0;
-    for(int i = 0; i < nprob; i++){
+    /* Weight gradients: every problem has the same number of tiles but a cost proportional to its
+     * row count, and the kernel gives table slot p to XCD p % 8 so that all tiles of an expert share
+     * one L2. The slots are therefore filled heaviest first, dealt to the XCDs back and forth. */
+    static int order[QLMX_MAX_PROBLEMS];
+    int live = 0;
+    for(int i = 0; i < nprob; i++) if(probs[i].M != 0) order[live++] = i;
+    if(mode == GEMM_NT && live > 8){
+        static int sorted[QLMX_MAX_PROBLEMS];
+        memcpy(sorted, order, (size_t)live * sizeof(int));
+        std::stable_sort(sorted, sorted + live, [&](int x, int y){ return probs[x].M > probs[y].M; });
+        for(int i = 0; i < live; i++){
+            const int grp = i >> 3, pos = i & 7, cnt = std::min(8, live - grp * 8);
+            const int x = (cnt == 8 && (grp & 1)) ? 7 - pos : pos;
+            order[grp * 8 + x] = sorted[i];
+        }
+    }
+    for(int oi = 0; oi < live; oi++){
+        const int i = order[oi];
         const qlmx_gemm_prob &p = probs[i];
         QLMX_REQUIRE(p.M >= 0, "grouped gemm: problem %d has M=%d", i, p.M);
         if(p.M == 0) continue;

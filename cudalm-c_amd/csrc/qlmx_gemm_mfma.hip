@@ -40,7 +40,7 @@ typedef float  f32x16 __attribute__((ext_vector_type(16)));
 #define BK 32
 #define KO 4                 /* 16-byte items per row per step */
 
-struct MfmaArgs { const DevProb *pr; int nprob, ntiles, tiles_n; const signed char *d; const float *s; int group, gshift; int K, N; };
+struct MfmaArgs { const DevProb *pr; int nprob, ntiles, tiles_n, rows_p; const signed char *d; const float *s; int group, gshift; int K, N; };
 
 /* two floats -> packed bf16 pair, round to nearest even (one v_cvt_pk_bf16_f32) */
 __device__ __forceinline__ uint32_t pk_bf16(float lo, float hi){
@@ -66,9 +66,10 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
 
     /* Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. nn/tn (tiles of equal
      * cost): XCD x takes the x-th contiguous eighth of the tile list, so tiles sharing an expert's
-     * rows and weights meet in one L2. nt (cost = the expert's row count): whole output tile-rows are
-     * dealt round-robin instead, which keeps the XCDs balanced. */
-    const int t = MODE == GEMM_NT ? qx_xcd_tile_rows(blockIdx.x, a.tiles_n) : qx_xcd_tile(blockIdx.x, gridDim.x);
+     * rows and weights meet in one L2. nt (cost = the expert's row count): whole problems per XCD, or
+     * output tile-rows dealt round-robin when their number per problem is a multiple of 8. */
+    const int t = MODE != GEMM_NT ? qx_xcd_tile(blockIdx.x, gridDim.x)
+                : (a.rows_p & 7) ? qx_xcd_tile_probs(blockIdx.x, a.tiles_n, a.rows_p) : qx_xcd_tile_rows(blockIdx.x, a.tiles_n);
     if(t >= a.ntiles) return;
     const DevProb P = a.pr[qx_find_problem(a.pr, a.nprob, t)];
     const int lt = t - P.tile0;
@@ -393,7 +394,12 @@ static int launch_mfma(const signed char *d, const float *s, int group, const ql
     if(up.ntiles == 0) return QLMX_OK;
     MfmaArgs a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.tiles_n = N / BN; a.d = d; a.s = s; a.group = group; a.gshift = 0; while((1 << a.gshift) < group) a.gshift++; a.K = K; a.N = N;
     int grid = (up.ntiles + 7) / 8 * 8;
-    if(MODE == GEMM_NT){ const int trows = up.ntiles / a.tiles_n; grid = 8 * a.tiles_n * ((trows + 7) / 8); }
+    a.rows_p = 1;
+    if(MODE == GEMM_NT){
+        a.rows_p = up.ntiles / (a.tiles_n * up.nprob);
+        if(a.rows_p & 7) grid = 8 * a.tiles_n * a.rows_p * ((up.nprob + 7) / 8);
+        else             grid = 8 * a.tiles_n * ((up.ntiles / a.tiles_n + 7) / 8);
+    }
     if(act_dtype == QLMX_ACT_BF16) hipLaunchKernelGGL((k_gemm_mfma<MODE, true, WM, DEEP>),  dim3(grid), dim3(256), 0, st, a);
     else                           hipLaunchKernelGGL((k_gemm_mfma<MODE, false, WM, DEEP>), dim3(grid), dim3(256), 0, st, a);
     QLMX_LAUNCH_CHECK("grouped gemm (mfma) launch");

@@ -71,6 +71,16 @@ SIGNATURES = {
     "qlmx_moe_gemm_tn": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_nt": (c_i, [c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_decode_forward": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_router_topk": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_vp, c_i, c_vp]),
+    "qlmx_moe_perm_workspace": (c_sz, [c_i, c_i, c_i]),
+    "qlmx_moe_perm": (c_i, [c_vp, c_i, c_i, c_i, c_vp, c_vp, c_vp, c_vp]),
+    "qlmx_moe_perm_status": (c_i, [c_vp, c_i, c_i, c_i, c_vp]),
+    "qlmx_moe_gather": (c_i, [c_vp, c_vp, c_vp, c_i, c_i, c_i, c_vp]),
+    "qlmx_moe_scatter_gate": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_vp]),
+    "qlmx_moe_scatter_add": (c_i, [c_vp, c_vp, c_vp, c_i, c_i, c_vp]),
+    "qlmx_moe_dgate": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_vp]),
+    "qlmx_swiglu": (c_i, [c_vp, c_vp, c_vp, c_sz, c_i, c_vp]),
+    "qlmx_swiglu_bwd": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_i, c_vp]),
 }
 
 
@@ -139,6 +149,37 @@ class Qlmx:
 
     def decode_forward(self, x, assign, gate, out, d, s, group, w1q, w3q, w2q, T, K, E, D, F, stream=None):
         self.call("qlmx_moe_decode_forward", x, assign, gate, out, d, s, group, w1q, w3q, w2q, T, K, E, D, F, stream)
+
+    # MoE glue (argument order of the reference kernels)
+    def router_topk(self, rt, rprobs, assign, gate, N, E, K, bias=None, bs=0, stream=None):
+        self.call("qlmx_router_topk", rt, rprobs, assign, gate, N, E, K, bias, bs, stream)
+
+    def moe_perm_workspace(self, N, E, K):
+        return int(self.lib.qlmx_moe_perm_workspace(N, E, K))
+
+    def moe_perm(self, assign, N, E, K, perm, off, workspace, stream=None):
+        self.call("qlmx_moe_perm", assign, N, E, K, perm, off, workspace, stream)
+
+    def moe_perm_status(self, workspace, N, E, K, stream=None):
+        self.call("qlmx_moe_perm_status", workspace, N, E, K, stream)
+
+    def moe_gather(self, src, perm, Xp, N, D, out_dtype=ACT_F32, stream=None):
+        self.call("qlmx_moe_gather", src, perm, Xp, N, D, out_dtype, stream)
+
+    def moe_scatter_gate(self, yp, perm, gate, out, N, D, stream=None):
+        self.call("qlmx_moe_scatter_gate", yp, perm, gate, out, N, D, stream)
+
+    def moe_scatter_add(self, dXp, perm, dst, N, D, stream=None):
+        self.call("qlmx_moe_scatter_add", dXp, perm, dst, N, D, stream)
+
+    def moe_dgate(self, dout, yp, perm, gate, d_gate, dyp, N, D, out_dtype=ACT_F32, stream=None):
+        self.call("qlmx_moe_dgate", dout, yp, perm, gate, d_gate, dyp, N, D, out_dtype, stream)
+
+    def swiglu(self, G, U, O, n, out_dtype=ACT_F32, stream=None):
+        self.call("qlmx_swiglu", G, U, O, n, out_dtype, stream)
+
+    def swiglu_bwd(self, Gg, U, dact, dg, du, n, out_dtype=ACT_F32, stream=None):
+        self.call("qlmx_swiglu_bwd", Gg, U, dact, dg, du, n, out_dtype, stream)
 
     def sync(self, stream=None):
         self.call("qlmx_sync", stream)

@@ -164,6 +164,44 @@ int qlmx_moe_decode_forward(const float *x, const int *assign, const float *gate
                             unsigned long long w1q, unsigned long long w3q, unsigned long long w2q,
                             int T, int K, int E, int D, int F, void *stream);
 
+/* =====================================================================================
+ * MoE layer glue around the expert GEMMs (training shape). Indices and gate probabilities are
+ * bit-exact against the reference's CPU build; float outputs follow its operation order.
+ * `out_dtype` (QLMX_ACT_F32 / QLMX_ACT_BF16) selects the type of a buffer that feeds a GEMM next,
+ * so the bf16 MFMA path needs no separate cast pass (bf16 = round to nearest even, cudalm.cu:334-338).
+ * Row buffers must be 16-byte aligned and D a multiple of 4.
+ * ===================================================================================== */
+
+/* k_router_topk (cudalm.cu:2515-2534; cpu_kern.h:413-425): softmax over E per token with the CPU
+ * build's polynomial exp (cpu_kern.h:29-34), then K greedy picks on prob + bias[k*bs + e] with a
+ * strict >, lowest index winning ties. rt, rprobs [N,E]; assign, gate pass-major [K][N]; gate is the
+ * raw softmax probability; bias may be NULL. K <= 8. */
+int qlmx_router_topk(const float *rt, float *rprobs, int *assign, float *gate, int N, int E, int K,
+                     const float *bias, int bs, void *stream);
+
+/* k_gp_hist / k_gp_scan / k_gp_scatter (cudalm.cu:3504-3530), equal to the host permutation of
+ * cudalm.cu:3586-3599: for each pass k a stable counting sort of the tokens by expert.
+ * perm [K][N]: perm[k][j] = token in row j of pass k; off [K][E+1]: first row of each expert.
+ * `workspace` = qlmx_moe_perm_workspace(N,E,K) bytes of device memory. Asynchronous; an expert index
+ * out of range is reported by qlmx_moe_perm_status (the reference aborts, cudalm.cu:3476-3478). */
+size_t qlmx_moe_perm_workspace(int N, int E, int K);
+int qlmx_moe_perm(const int *assign, int N, int E, int K, int *perm, int *off, void *workspace, void *stream);
+int qlmx_moe_perm_status(const void *workspace, int N, int E, int K, void *stream);
+
+/* k_gather / k_gather4 (cudalm.cu:2536-2539, 2558-2563): Xp[j,:] = src[perm[j],:], zeros where perm[j] < 0 */
+int qlmx_moe_gather(const float *src, const int *perm, void *Xp, int N, int D, int out_dtype, void *stream);
+/* k_scatter_gate (cudalm.cu:2541-2545): out[perm[j],:] += gate[perm[j]] * yp[j,:] */
+int qlmx_moe_scatter_gate(const float *yp, const int *perm, const float *gate, float *out, int N, int D, void *stream);
+/* k_scatter_add4 (cudalm.cu:2564-2567; cpu_kern.h:445-450): dst[perm[j],:] += dXp[j,:] */
+int qlmx_moe_scatter_add(const float *dXp, const int *perm, float *dst, int N, int D, void *stream);
+/* k_moe_dgate (cudalm.cu:2591; cpu_kern.h:454-468): d_gate[n] = dout[n,:] . yp[j,:], dyp[j,:] = gate[n] * dout[n,:], n = perm[j] */
+int qlmx_moe_dgate(const float *dout, const float *yp, const int *perm, const float *gate,
+                   float *d_gate, void *dyp, int N, int D, int out_dtype, void *stream);
+/* k_swiglu / k_swiglu_bwd (cudalm.cu:2430-2453; cpu_kern.h:376-394): O = g*sigmoid(g)*u and its
+ * gradient (dg, du) from dact, with the CPU build's polynomial sigmoid. n % 4 == 0. */
+int qlmx_swiglu(const float *G, const float *U, void *O, size_t n, int out_dtype, void *stream);
+int qlmx_swiglu_bwd(const float *Gg, const float *U, const float *dact, void *dg, void *du, size_t n, int out_dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

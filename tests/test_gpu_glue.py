@@ -1,0 +1,292 @@
+"""GPU parity of the MoE glue (router, grouping permutation, gather / scatter, gate gradient, SwiGLU)
+and of a whole expert-FFN layer -- forward and backward -- put together from the library's entry
+points, against the CPU oracle (orc_moe_forward / orc_moe_backward follow cudalm.cu:4193-4228 and
+4299-4371) and the fixtures written by the compiled reference.
+
+Bars: indices (assign, perm, off), gate probabilities and every pure data move are bit-exact; SwiGLU
+and the dot product of the gate gradient follow the oracle to 1e-6 relative L2; layer outputs to 1e-5
+with the fp32 GEMMs. With the bf16 MFMA GEMMs each GEMM meets 1e-3 on equal inputs (tested with the
+GEMMs); the whole layer, whose intermediates are then stored as bf16, is held to 4e-3 here."""
+import numpy as np
+import pytest
+
+from __graft_entry__ import load_package
+from oracle.binding import make_spans
+
+pkg = load_package()
+f32 = np.float32
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def q():
+    return pkg.load()
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def zeros(n, dtype=None):
+    import torch
+    return torch.zeros(n, dtype=dtype or torch.float32, device="cuda")
+
+
+def bf16_to_f32(t):
+    """int16 tensor of bf16 bit patterns -> fp32 numpy"""
+    import torch
+    return (t.to(torch.int32) << 16).view(torch.float32).cpu().numpy()
+
+
+# ------------------------------------------------------------------ router
+@pytest.mark.parametrize("tag", ["a", "b", "c"])
+def test_router_vs_reference_fixture(q, golden, tag):
+    import torch
+    g = golden("router")
+    N, E, K = (int(v) for v in g["dims_" + tag])
+    pr, asn, gate = zeros(N * E), zeros(K * N, torch.int32), zeros(K * N)
+    q.router_topk(dev(g["rt_" + tag]), pr, asn, gate, N, E, K)
+    torch.cuda.synchronize()
+    assert np.array_equal(asn.cpu().numpy(), g["asn_" + tag])
+    assert np.array_equal(gate.cpu().numpy().view(np.uint32), g["gate_" + tag].view(np.uint32))
+    assert np.array_equal(pr.cpu().numpy().view(np.uint32), g["pr_" + tag].view(np.uint32))
+
+
+def test_router_bias_vs_reference_fixture(q, golden):
+    import torch
+    g = golden("router")
+    N, E, K = (int(v) for v in g["dims_a"])
+    pr, asn, gate = zeros(N * E), zeros(K * N, torch.int32), zeros(K * N)
+    q.router_topk(dev(g["rt_a"]), pr, asn, gate, N, E, K, dev(g["bias"]), E)
+    torch.cuda.synchronize()
+    assert np.array_equal(asn.cpu().numpy(), g["asn_bias"])
+    assert np.array_equal(gate.cpu().numpy().view(np.uint32), g["gate_bias"].view(np.uint32))
+
+
+def test_router_training_size_vs_oracle(q, orc):
+    """8192 tokens x 32 experts, logits quantised to 1/8 so that many exact ties occur."""
+    import torch
+    N, E, K = 8192, 32, 2
+    rt = np.round(orc.normal(N * E, 3, 1, 2.0) * 8).astype(f32) / 8
+    want_pr = np.zeros(N * E, f32); want_asn = np.zeros(K * N, np.int32); want_gate = np.zeros(K * N, f32)
+    orc.router_topk(rt, want_pr, want_asn, want_gate, N, E, K)
+    pr, asn, gate = zeros(N * E), zeros(K * N, torch.int32), zeros(K * N)
+    q.router_topk(dev(rt), pr, asn, gate, N, E, K)
+    torch.cuda.synchronize()
+    assert np.array_equal(asn.cpu().numpy(), want_asn)
+    assert np.array_equal(gate.cpu().numpy().view(np.uint32), want_gate.view(np.uint32))
+    assert np.array_equal(pr.cpu().numpy().view(np.uint32), want_pr.view(np.uint32))
+
+
+def test_router_limits(q):
+    z = zeros(64)
+    with pytest.raises(pkg.QlmxError, match="K"):
+        q.router_topk(z, z, z, z, 4, 4, 9)
+
+
+# ------------------------------------------------------------------ permutation
+def gpu_perm(q, asn, N, E, K):
+    import torch
+    ws = torch.zeros(q.moe_perm_workspace(N, E, K), dtype=torch.uint8, device="cuda")
+    perm, off = zeros(K * N, torch.int32), zeros(K * (E + 1), torch.int32)
+    q.moe_perm(dev(asn), N, E, K, perm, off, ws)
+    q.moe_perm_status(ws, N, E, K)
+    return perm.cpu().numpy(), off.cpu().numpy(), ws
+
+
+@pytest.mark.parametrize("N,E,K", [(1, 1, 1), (50, 3, 2), (256, 8, 1), (257, 8, 3), (1000, 64, 4), (8192, 32, 2), (5000, 300, 2)])
+def test_perm_vs_oracle(q, orc, N, E, K):
+    rng = np.random.default_rng(N * 31 + E)
+    p = (np.arange(E) + 1.0) ** -1.1; p /= p.sum()
+    asn = rng.choice(E, size=K * N, p=p).astype(np.int32)
+    if E > 2:
+        asn[asn == 1] = 0                                # an expert nobody picks
+    perm, off, _ = gpu_perm(q, asn, N, E, K)
+    for k in range(K):
+        wp = np.zeros(N, np.int32); wo = np.zeros(E + 1, np.int32)
+        assert orc.moe_perm(asn[k * N:(k + 1) * N], N, E, wp, wo) == 0
+        assert np.array_equal(off[k * (E + 1):(k + 1) * (E + 1)], wo)
+        assert np.array_equal(perm[k * N:(k + 1) * N], wp)
+
+
+def test_perm_reports_bad_expert(q):
+    asn = np.array([0, 1, 9, 2], np.int32)
+    with pytest.raises(pkg.QlmxError, match="out of range"):
+        gpu_perm(q, asn, 4, 4, 1)
+
+
+# ------------------------------------------------------------------ row movers, dgate, swiglu
+def test_glue_vs_reference_fixture(q, golden):
+    import torch
+    g = golden("glue")
+    N, D = (int(v) for v in g["dims"])
+    perm, gate = dev(g["perm"]), dev(g["gate"])
+    Xp = zeros(N * D)
+    q.moe_gather(dev(g["src"]), perm, Xp, N, D)
+    sg = dev(g["out0"].copy()); q.moe_scatter_gate(Xp, perm, gate, sg, N, D)
+    sa = dev(g["out0"].copy()); q.moe_scatter_add(Xp, perm, sa, N, D)
+    dgate, dyp = zeros(N), zeros(N * D)
+    q.moe_dgate(dev(g["dout"]), Xp, perm, gate, dgate, dyp, N, D)
+    n = (g["G"].size // 4) * 4
+    O, dg, du = zeros(n), zeros(n), zeros(n)
+    G, U, dA = dev(g["G"][:n]), dev(g["U"][:n]), dev(g["dA"][:n])
+    q.swiglu(G, U, O, n)
+    q.swiglu_bwd(G, U, dA, dg, du, n)
+    torch.cuda.synchronize()
+    bits = lambda a: np.ascontiguousarray(a).view(np.uint32)
+    assert np.array_equal(bits(Xp.cpu().numpy()), bits(g["Xp"]))
+    assert np.array_equal(bits(sg.cpu().numpy()), bits(g["sg"]))
+    assert np.array_equal(bits(sa.cpu().numpy()), bits(g["sa"]))
+    assert np.array_equal(bits(dyp.cpu().numpy()), bits(g["dyp"]))
+    rel = lambda a, b: float(np.linalg.norm(a.astype(np.float64) - b) / max(np.linalg.norm(b.astype(np.float64)), 1e-30))
+    assert rel(dgate.cpu().numpy(), g["dgate"]) < 1e-6
+    # the reference's CPU sigmoid uses explicit FMA intrinsics (cpu_kern.h:37-50): tolerance, not bits
+    assert rel(O.cpu().numpy(), g["O"][:n]) < 1e-6
+    assert rel(dg.cpu().numpy(), g["dg"][:n]) < 1e-6
+    assert rel(du.cpu().numpy(), g["du"][:n]) < 1e-6
+
+
+def test_glue_negative_perm_and_bf16_outputs(q, orc):
+    import torch
+    N, D = 37, 64
+    src = orc.normal(N * D, 2, 1)
+    perm = np.arange(N, dtype=np.int32)[::-1].copy(); perm[5] = -1; perm[20] = -1
+    want = np.zeros(N * D, f32); orc.gather(src, perm, want, N, D)
+    Xp = zeros(N * D); q.moe_gather(dev(src), dev(perm), Xp, N, D)
+    Xb = zeros(N * D, torch.int16); q.moe_gather(dev(src), dev(perm), Xb, N, D, pkg.ACT_BF16)
+    torch.cuda.synchronize()
+    assert np.array_equal(Xp.cpu().numpy(), want)
+    assert np.array_equal(bf16_to_f32(Xb), orc.bf16_round(want))
+    n = 4096
+    G, U = orc.normal(n, 2, 2, 2.0), orc.normal(n, 2, 3)
+    wantO = np.zeros(n, f32); orc.swiglu(G, U, wantO)
+    Ob = zeros(n, torch.int16); q.swiglu(dev(G), dev(U), Ob, n, pkg.ACT_BF16)
+    Of = zeros(n); q.swiglu(dev(G), dev(U), Of, n)
+    torch.cuda.synchronize()
+    assert np.array_equal(Of.cpu().numpy().view(np.uint32), wantO.view(np.uint32))      # same operations as the oracle
+    assert np.array_equal(bf16_to_f32(Ob), orc.bf16_round(wantO))
+
+
+# ------------------------------------------------------------------ a whole layer from the entry points
+def encode_layer(orc, seed, E, D, F, group=128):
+    n = E * D * F
+    tab, nq, ng = make_spans([n, n, n], group)
+    P = np.concatenate([orc.normal(n, seed, 1, 0.02), orc.normal(n, seed, 2, 0.02), orc.normal(n, seed, 3, 0.02)])
+    d = np.zeros(nq // 2, np.int8); r = np.zeros(nq, np.int8); s = np.zeros(ng, f32)
+    orc.encode(P, d, r, s, tab, group, 7, 1, ng)
+    orc.render(P, d, s, tab, group, 1, 0, ng)
+    return d, s, P, n
+
+
+class GpuLayer:
+    """moe_forward / moe_backward (cudalm.cu:4193-4228, 4299-4371, stash off) on the library's entry
+    points; the only host step is reading the expert row counts to size the grouped GEMM calls, which
+    the reference does as well (cudalm.cu:3576-3602)."""
+
+    def __init__(self, q, dd, ds, n, N, D, F, E, K, math, group=128):
+        import torch
+        self.q, self.dd, self.ds, self.n, self.N, self.D, self.F, self.E, self.K, self.math, self.group = q, dd, ds, n, N, D, F, E, K, math, group
+        self.act = pkg.ACT_BF16 if math == pkg.MATH_MFMA else pkg.ACT_F32
+        self.esz = 2 if math == pkg.MATH_MFMA else 4
+        adt = torch.int16 if math == pkg.MATH_MFMA else torch.float32
+        self.ws = torch.zeros(q.moe_perm_workspace(N, E, K), dtype=torch.uint8, device="cuda")
+        self.perm, self.off = zeros(K * N, torch.int32), zeros(K * (E + 1), torch.int32)
+        self.Xp, self.ap = zeros(N * D, adt), zeros(N * F, adt)
+        self.gp, self.up, self.yp = zeros(N * F), zeros(N * F), zeros(N * D)
+        self.dyp, self.dgp, self.dup = zeros(N * D, adt), zeros(N * F, adt), zeros(N * F, adt)
+        self.dap, self.dXp = zeros(N * F), zeros(N * D)
+
+    def group_tokens(self, assign):
+        q = self.q
+        q.moe_perm(assign, self.N, self.E, self.K, self.perm, self.off, self.ws)
+        q.moe_perm_status(self.ws, self.N, self.E, self.K)
+        self.offh = self.off.cpu().numpy().reshape(self.K, self.E + 1)
+
+    def probs(self, k, A, a_cols, a_esz, C, c_cols, wbase, B=None, b_cols=0, b_esz=0, beta=0.0, out_expert=False):
+        off = self.offh[k]; DF = self.D * self.F
+        items = []
+        for e in range(self.E):
+            ne = int(off[e + 1] - off[e])
+            a = A.data_ptr() + int(off[e]) * a_cols * a_esz
+            b = None if B is None else B.data_ptr() + int(off[e]) * b_cols * b_esz
+            c = C.data_ptr() + (e * DF * 4 if out_expert else int(off[e]) * c_cols * 4)
+            wq = wbase + e * DF
+            items.append((a, b, c, wq, wq // self.group, ne, beta))
+        return self.q.problems(items)
+
+    def experts_fwd(self, k):
+        q, D, F, E, n = self.q, self.D, self.F, self.E, self.n
+        q.gemm_nn(self.dd, self.ds, self.group, self.probs(k, self.Xp, D, self.esz, self.gp, F, 0), E, D, F, self.act, self.math)
+        q.gemm_nn(self.dd, self.ds, self.group, self.probs(k, self.Xp, D, self.esz, self.up, F, n), E, D, F, self.act, self.math)
+        q.swiglu(self.gp, self.up, self.ap, self.N * F, self.act)
+        q.gemm_nn(self.dd, self.ds, self.group, self.probs(k, self.ap, F, self.esz, self.yp, D, 2 * n), E, F, D, self.act, self.math)
+
+    def forward(self, x, assign, gate, out):
+        q, N, D = self.q, self.N, self.D
+        self.group_tokens(assign)
+        for k in range(self.K):
+            prm = self.perm[k * N:(k + 1) * N]
+            q.moe_gather(x, prm, self.Xp, N, D, self.act)
+            self.experts_fwd(k)
+            q.moe_scatter_gate(self.yp, prm, gate[k * N:(k + 1) * N], out, N, D)
+
+    def backward(self, x, gate, dout, dx, dgate, Gw1, Gw3, Gw2):
+        q, N, D, F, E, n = self.q, self.N, self.D, self.F, self.E, self.n
+        dx.zero_()
+        for k in range(self.K):
+            prm = self.perm[k * N:(k + 1) * N]
+            q.moe_gather(x, prm, self.Xp, N, D, self.act)
+            self.experts_fwd(k)
+            q.moe_dgate(dout, self.yp, prm, gate[k * N:(k + 1) * N], dgate[k * N:(k + 1) * N], self.dyp, N, D, self.act)
+            q.gemm_nt(self.probs(k, self.ap, F, self.esz, Gw2, 0, 0, B=self.dyp, b_cols=D, b_esz=self.esz, beta=1.0, out_expert=True), E, F, D, self.act, self.math)
+            q.gemm_tn(self.dd, self.ds, self.group, self.probs(k, self.dyp, D, self.esz, self.dap, F, 2 * n), E, D, F, self.act, self.math)
+            q.swiglu_bwd(self.gp, self.up, self.dap, self.dgp, self.dup, N * F, self.act)
+            q.gemm_nt(self.probs(k, self.Xp, D, self.esz, Gw1, 0, 0, B=self.dgp, b_cols=F, b_esz=self.esz, beta=1.0, out_expert=True), E, D, F, self.act, self.math)
+            q.gemm_nt(self.probs(k, self.Xp, D, self.esz, Gw3, 0, 0, B=self.dup, b_cols=F, b_esz=self.esz, beta=1.0, out_expert=True), E, D, F, self.act, self.math)
+            q.gemm_tn(self.dd, self.ds, self.group, self.probs(k, self.dgp, F, self.esz, self.dXp, D, 0), E, F, D, self.act, self.math)
+            q.gemm_tn(self.dd, self.ds, self.group, self.probs(k, self.dup, F, self.esz, self.dXp, D, n, beta=1.0), E, F, D, self.act, self.math)
+            q.moe_scatter_add(self.dXp, prm, dx, N, D)
+
+
+@pytest.mark.parametrize("math,N,E,D,F,K", [("f32", 96, 4, 128, 256, 2), ("f32", 300, 8, 256, 384, 2),
+                                            ("mfma", 512, 4, 256, 384, 2), ("mfma", 1024, 8, 768, 2048, 2)])
+def test_layer_forward_backward_vs_oracle(q, orc, math, N, E, D, F, K):
+    import torch
+    mth = pkg.MATH_MFMA if math == "mfma" else pkg.MATH_F32
+    # bf16 storage of the intermediates (ap, dyp, dgp, dup) alone is worth 2^-9/sqrt(3) = 1.1e-3 of relative
+    # error per element; the reference holds its own bf16 path to 3e-2 (cudalm.cu:10430)
+    tol = 4e-3 if math == "mfma" else 1e-5
+    d, s, P, n = encode_layer(orc, 40 + N, E, D, F)
+    x = orc.normal(N * D, 41, 1)
+    dout = orc.normal(N * D, 41, 2)
+    if math == "mfma":                                   # bf16 activations, as the training config feeds them
+        x = orc.bf16_round(x); dout = orc.bf16_round(dout)
+    rt = orc.normal(N * E, 41, 3)
+    pr = np.zeros(N * E, f32); asn = np.zeros(K * N, np.int32); gate = np.zeros(K * N, f32)
+    orc.router_topk(rt, pr, asn, gate, N, E, K)
+    # oracle
+    w_out = np.zeros(N * D, f32)
+    rc, ws = orc.moe_forward(x, P[:n], P[n:2 * n], P[2 * n:], asn, gate, w_out, N, D, F, E, K)
+    assert rc == 0
+    w_dx = np.zeros(N * D, f32); w_dgate = np.zeros(K * N, f32)
+    w_G = [np.zeros(n, f32) for _ in range(3)]
+    orc.moe_backward(ws, x, P[:n], P[n:2 * n], P[2 * n:], gate, dout, w_dx, w_dgate, w_G[0], w_G[1], w_G[2])
+    orc.moe_ws_free(ws)
+    # library: router and grouping on the device too
+    dpr, dasn, dgt = zeros(N * E), zeros(K * N, torch.int32), zeros(K * N)
+    q.router_topk(dev(rt), dpr, dasn, dgt, N, E, K)
+    L = GpuLayer(q, dev(d), dev(s), n, N, D, F, E, K, mth)
+    out = zeros(N * D)
+    dx_ = dev(x); ddout = dev(dout)
+    L.forward(dx_, dasn, dgt, out)
+    dx, dgate = zeros(N * D), zeros(K * N)
+    G = [zeros(n) for _ in range(3)]
+    L.backward(dx_, dgt, ddout, dx, dgate, G[0], G[1], G[2])
+    torch.cuda.synchronize()
+    assert np.array_equal(dasn.cpu().numpy(), asn)
+    assert orc.relerr(out.cpu().numpy(), w_out) < tol
+    assert orc.relerr(dx.cpu().numpy(), w_dx) < tol
+    assert orc.relerr(dgate.cpu().numpy(), w_dgate) < tol
+    for got, want in zip(G, w_G):
+        assert orc.relerr(got.cpu().numpy(), want) < tol

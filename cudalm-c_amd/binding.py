@@ -81,6 +81,9 @@ SIGNATURES = {
     "qlmx_moe_dgate": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_vp]),
     "qlmx_swiglu": (c_i, [c_vp, c_vp, c_vp, c_sz, c_i, c_vp]),
     "qlmx_swiglu_bwd": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_i, c_vp]),
+    "qlmx_q4n_bound": (c_sz, [c_sz, c_i]),
+    "qlmx_q4n_quantize": (c_i, [c_vp, c_sz, c_i, c_vp, c_sz, c_vp, c_vp]),
+    "qlmx_q4n_dequantize": (c_i, [c_vp, c_sz, c_vp, c_sz, c_i, c_vp]),
 }
 
 
@@ -180,6 +183,23 @@ class Qlmx:
 
     def swiglu_bwd(self, Gg, U, dact, dg, du, n, out_dtype=ACT_F32, stream=None):
         self.call("qlmx_swiglu_bwd", Gg, U, dact, dg, du, n, out_dtype, stream)
+
+    # q4n wire format (host memory, numpy arrays)
+    def q4n_quantize(self, P, group):
+        """P: fp32 numpy array -> (uint8 numpy array in the wire format, number of raw groups)"""
+        import numpy as np
+        cap = int(self.lib.qlmx_q4n_bound(P.size, group))
+        out = np.zeros(max(cap, 1), np.uint8)
+        n, raw = C.c_size_t(0), C.c_size_t(0)
+        self.call("qlmx_q4n_quantize", P, P.size, group, out, cap, C.addressof(n), C.addressof(raw))
+        return out[:n.value].copy(), int(raw.value)
+
+    def q4n_dequantize(self, buf, n, group):
+        import numpy as np
+        P = np.zeros(n, np.float32)
+        used = C.c_size_t(0)
+        self.call("qlmx_q4n_dequantize", buf, buf.size, P, n, group, C.addressof(used))
+        return P, int(used.value)
 
     def sync(self, stream=None):
         self.call("qlmx_sync", stream)

@@ -202,6 +202,18 @@ int qlmx_moe_dgate(const float *dout, const float *yp, const int *perm, const fl
 int qlmx_swiglu(const float *G, const float *U, void *O, size_t n, int out_dtype, void *stream);
 int qlmx_swiglu_bwd(const float *Gg, const float *U, const float *dact, void *dg, void *du, size_t n, int out_dtype, void *stream);
 
+/* =====================================================================================
+ * q4n wire format (host only, no device needed): quantize_params / dequantize_params with qtype 3
+ * (cudalm.cu:638-656 and 688-696). Per group: fp32 scale + packed nibbles, or a NaN scale followed by
+ * the raw fp32 values when the group is not on a 4-bit grid. Byte-identical to the reference's
+ * writer; the reader reproduces every value bit for bit.
+ * qlmx_q4n_bound: bytes that always suffice for n values. quantize: *out_len bytes written, *nraw
+ * (may be NULL) = groups stored raw. dequantize: *used (may be NULL) = bytes consumed.
+ * ===================================================================================== */
+size_t qlmx_q4n_bound(size_t n, int group);
+int qlmx_q4n_quantize(const float *P, size_t n, int group, unsigned char *out, size_t cap, size_t *out_len, size_t *nraw);
+int qlmx_q4n_dequantize(const unsigned char *buf, size_t len, float *P, size_t n, int group, size_t *used);
+
 #ifdef __cplusplus
 }
 #endif

@@ -104,6 +104,8 @@ class Oracle(_Lib):
         self._dgate = s("orc_moe_dgate", None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i])
         self._swiglu = s("orc_swiglu", None, [c_vp, c_vp, c_vp, c_sz])
         self._swiglu_bwd = s("orc_swiglu_bwd", None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz])
+        self._q4n_q = s("orc_q4n_quantize", c_sz, [c_vp, c_sz, c_i, c_vp, c_sz, c_vp])
+        self._q4n_d = s("orc_q4n_dequantize", c_i, [c_vp, c_sz, c_vp, c_sz, c_i])
         self._ws_new = s("orc_moe_ws_new", c_vp, [c_i, c_i, c_i, c_i, c_i])
         self._ws_free = s("orc_moe_ws_free", None, [c_vp])
         self._moe_fwd = s("orc_moe_forward", c_i, [c_vp] * 8)
@@ -203,6 +205,19 @@ class Oracle(_Lib):
     def swiglu_bwd(self, Gg, U, dact, dg, du):
         self._swiglu_bwd(_p(Gg), _p(U), _p(dact), _p(dg), _p(du), Gg.size)
 
+    def q4n_quantize(self, P, group):
+        """returns (bytes as uint8 array, number of raw groups)"""
+        cap = 4 * P.size + 4 * ((P.size + group - 1) // group) + 16
+        out = np.zeros(cap, np.uint8)
+        nraw = C.c_size_t(0)
+        n = self._q4n_q(_p(P), P.size, group, _p(out), cap, C.addressof(nraw))
+        return out[:n].copy(), int(nraw.value)
+
+    def q4n_dequantize(self, buf, n, group):
+        P = np.zeros(n, np.float32)
+        ok = self._q4n_d(_p(buf), buf.size, _p(P), n, group)
+        return ok, P
+
     def moe_forward(self, x, w1, w3, w2, assign, gate, out, N, D, F, E, K):
         """returns (rc, ws) -- keep ws for moe_backward, free with moe_ws_free"""
         ws = self._ws_new(N, D, F, E, K)
@@ -286,6 +301,8 @@ class Ref(_Lib):
         self._dgate = s("ref_moe_dgate", None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i])
         self._swiglu = s("ref_swiglu", None, [c_vp, c_vp, c_vp, c_sz])
         self._swiglu_bwd = s("ref_swiglu_bwd", None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz])
+        self._q4n_q = s("ref_q4n_quantize", c_sz, [c_vp, c_sz, c_i, c_vp, c_sz])
+        self._q4n_d = s("ref_q4n_dequantize", c_i, [c_vp, c_sz, c_vp, c_sz, c_i])
         self._relerr = s("ref_relerr", c_f, [c_vp, c_vp, c_sz])
 
     def qd_get(self, d, i, packed):
@@ -346,6 +363,23 @@ class Ref(_Lib):
 
     def swiglu_bwd(self, Gg, U, dact, dg, du):
         self._swiglu_bwd(_p(Gg), _p(U), _p(dact), _p(dg), _p(du), Gg.size)
+
+
+def _ref_q4n_quantize(self, P, group):
+    cap = 4 * P.size + 4 * ((P.size + group - 1) // group) + 16
+    out = np.zeros(cap, np.uint8)
+    n = self._q4n_q(_p(P), P.size, group, _p(out), cap)
+    return out[:n].copy()
+
+
+def _ref_q4n_dequantize(self, buf, n, group):
+    P = np.zeros(n, np.float32)
+    ok = self._q4n_d(_p(buf), buf.size, _p(P), n, group)
+    return ok, P
+
+
+Ref.q4n_quantize = _ref_q4n_quantize
+Ref.q4n_dequantize = _ref_q4n_dequantize
 
 
 def have_ref():

@@ -12,6 +12,8 @@
  *   gather/scatter/dgate                      closed form + ref lib
  *   swiglu fwd/bwd                            libm closed form to 1e-6 (the reference's AVX2 body uses
  *                                             explicit FMA, so tolerance rather than bits) + ref lib
+ *   q4n quantize/dequantize                   fixtures (byte-exact: grid groups, off-grid raw groups, an
+ *                                             all-zero group, a short tail) + round trip + ref lib
  *   moe_forward/backward                      double-precision scalar expert FFN in the tests
  *                                             (cudalm.cu:10366-10387 style) + composition of ref lib calls
  * No function here is "parity unpinned".
@@ -632,6 +634,63 @@ void orc_moe_backward(orc_moe_ws *w, const float *x, const float *w1, const floa
         }
         orc_scatter_add(w->dXp, prm, dx, N, D);
     }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * q4n wire format
+ * ---------------------------------------------------------------------------------------- */
+/* cudalm.cu:638-656. For each group: amax; candidate scales amax/k for k = 7..1 and their two
+ * neighbours on each side; the first candidate for which every value is exactly scale * an integer
+ * of magnitude <= 7 wins. An all-zero group keeps scale 0. */
+size_t orc_q4n_quantize(const float *P, size_t n, int group, unsigned char *out, size_t cap, size_t *nraw){
+    size_t o = 0, raw = 0;
+    for(size_t i = 0; i < n; i += (size_t)group){
+        int g = (i + (size_t)group <= n) ? group : (int)(n - i), ok = 0;
+        float amax = 0, s = 0;
+        for(int j = 0; j < g; j++){ float a = fabsf(P[i+j]); if(a > amax) amax = a; }
+        if(amax == 0) ok = 1;
+        for(int k = 7; k >= 1 && !ok; k--){
+            float s0 = amax / (float)k, c[5];
+            c[0] = s0; c[1] = nextafterf(s0, 0); c[2] = nextafterf(s0, INFINITY);
+            c[3] = nextafterf(c[1], 0); c[4] = nextafterf(c[2], INFINITY);
+            for(int t = 0; t < 5 && !ok; t++){
+                s = c[t]; ok = 1;
+                for(int j = 0; j < g && ok; j++){ float d = rintf(P[i+j] / s); if(fabsf(d) > 7 || d * s != P[i+j]) ok = 0; }
+            }
+        }
+        if(!ok){
+            float nanv = NAN;
+            if(o + 4 + 4*(size_t)g <= cap){ memcpy(out + o, &nanv, 4); memcpy(out + o + 4, P + i, 4*(size_t)g); }
+            o += 4 + 4*(size_t)g; raw++; continue;
+        }
+        if(o + 4 <= cap) memcpy(out + o, &s, 4);
+        o += 4;
+        for(int j = 0; j < g; j += 2){
+            int a = s ? (int)rintf(P[i+j] / s) : 0, b = (j + 1 < g && s) ? (int)rintf(P[i+j+1] / s) : 0;
+            if(o < cap) out[o] = (unsigned char)((a & 15) | ((b & 15) << 4));
+            o++;
+        }
+    }
+    if(nraw) *nraw = raw;
+    return o;
+}
+/* cudalm.cu:688-696; returns 0 on a short buffer */
+int orc_q4n_dequantize(const unsigned char *buf, size_t len, float *P, size_t n, int group){
+    size_t o = 0;
+    for(size_t i = 0; i < n; i += (size_t)group){
+        int g = (i + (size_t)group <= n) ? group : (int)(n - i);
+        float s;
+        if(o + 4 > len) return 0;
+        memcpy(&s, buf + o, 4); o += 4;
+        if(s != s){ if(o + 4*(size_t)g > len) return 0; memcpy(P + i, buf + o, 4*(size_t)g); o += 4*(size_t)g; continue; }
+        for(int j = 0; j < g; j += 2){
+            if(o + 1 > len) return 0;
+            unsigned char b = buf[o++];
+            P[i+j] = (float)((int)((b & 15) ^ 8) - 8) * s;
+            if(j + 1 < g) P[i+j+1] = (float)((int)((b >> 4) ^ 8) - 8) * s;
+        }
+    }
+    return 1;
 }
 
 /* ------------------------------------------------------------------------------------------

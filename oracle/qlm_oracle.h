@@ -102,6 +102,13 @@ void orc_moe_backward(orc_moe_ws *w, const float *x, const float *w1, const floa
                       const float *gate, const float *dout, float *dx, float *dgate,
                       float *Gw1, float *Gw3, float *Gw2);
 
+/* ---- q4n wire format (cudalm.cu:638-656 writer, 688-696 reader): per group one fp32 scale and
+ *      ceil(g/2) nibble bytes (same nibble rule as the packed digits); a group whose values are not
+ *      s * integers in [-7,7] for any candidate scale is written as NaN + raw fp32. Returns the
+ *      number of bytes (written only if <= cap); *nraw counts the raw groups. ---- */
+size_t orc_q4n_quantize(const float *P, size_t n, int group, unsigned char *out, size_t cap, size_t *nraw);
+int    orc_q4n_dequantize(const unsigned char *buf, size_t len, float *P, size_t n, int group);
+
 /* ---- deterministic synthetic inputs: splitmix64 keyed by (seed, tensor id), top 24 bits as a
  *      uniform, Irwin-Hall sum of 12 uniforms minus 6 as a normal. Integer and exactly-rounded
  *      fp32 operations only, so every machine produces the same bits. ---- */

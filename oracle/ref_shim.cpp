@@ -100,4 +100,14 @@ void ref_swiglu_bwd(const float*Gg,const float*U,const float*dact,float*dg,float
 }
 float ref_relerr(const float*a,const float*b,size_t n){ return relerr(a,b,n); }
 
+/* ---- cudalm.cu:638-656, 688-696: the q4n wire format (qtype 3) ---- */
+size_t ref_q4n_quantize(const float*P,size_t n,int group,unsigned char*out,size_t cap){
+    size_t len=0; uint8_t*q=quantize_params(P,n,3,group,&len);
+    if(len<=cap) memcpy(out,q,len);
+    free(q); return len;
+}
+int ref_q4n_dequantize(const unsigned char*buf,size_t len,float*P,size_t n,int group){
+    Rd r; r.p=buf; r.end=buf+len; return dequantize_params(&r,P,n,3,group);
+}
+
 } /* extern "C" */

@@ -222,7 +222,30 @@ def golden_glue():
          dout=dout, dgate=dgate, dyp=dyp, G=G, U=U, dA=dA, O=O, dg=dg, du=du)
 
 
+def golden_q4n():
+    """q4n wire format (cudalm.cu:638-656): groups on the 4-bit grid (rendered QLM view), groups off
+    the grid (stored raw), an all-zero group, a one-hot group and a short tail."""
+    group = 128
+    n = 128 * 7 + 50
+    tab, nq, ng = make_spans([128 * 8], group)
+    P0 = gen.normal(128 * 8, 0, 900, 0.02)
+    d = np.zeros(nq // 2, np.int8); r = np.zeros(nq, np.int8); s = np.zeros(ng, f32)
+    ref.encode(P0, d, r, s, tab, group, 7, 1, ng)
+    ref.render(P0, d, s, tab, group, 1, 0, ng)            # P0 = s * digit: on the grid
+    P = P0[:n].copy()
+    P[128:256] = gen.normal(128, 0, 901, 0.02)            # off the grid -> raw
+    P[256:384] = 0.0                                      # all zero -> scale 0
+    P[384:512] = 0.0; P[400] = -0.0371                    # one value -> scale = |v| / 7 .. / 1 candidates
+    P[512:640] *= f32(0.5)                                # still on a grid (power of two)
+    buf = ref.q4n_quantize(P, group)
+    ok, back = ref.q4n_dequantize(buf, n, group)
+    assert ok == 1
+    buf64 = ref.q4n_quantize(P[:300], 64)
+    save("q4n", dims=np.array([n, group]), P=P, buf=buf, back=back, buf64=buf64)
+
+
 if __name__ == "__main__":
+    golden_q4n()
     golden_hash()
     golden_nibble()
     golden_qlm()

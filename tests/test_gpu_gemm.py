@@ -166,6 +166,18 @@ def test_mfma_f32_acts_are_rounded_once(q, orc):
     assert orc.relerr(got32, want) < TOL_MFMA
 
 
+@pytest.mark.parametrize("math", ["f32", "mfma"])
+def test_attention_projection_spans_are_one_expert(q, orc, math):
+    """wq/wk/wv/wo are QLM spans too (qlm.cuh:480-483): a dense [D,D] or [D,KD] projection is the
+    grouped GEMM with a single problem. D=768, KD=256, 1536 rows; forward, dgrad and wgrad."""
+    act, mth, tol = (pkg.ACT_BF16, pkg.MATH_MFMA, TOL_MFMA) if math == "mfma" else (pkg.ACT_F32, pkg.MATH_F32, TOL_F32)
+    for (K, N) in [(768, 768), (768, 256)]:
+        for mode in ["nn", "tn", "nt"]:
+            kk, nn = (K, N) if mode != "tn" else (N, K)
+            got, want = run_case(q, orc, mode, 1, [1536], kk, nn, act, mth, seed=9)
+            assert orc.relerr(got, want) < tol, (mode, K, N)
+
+
 def test_mfma_rejects_unsupported_shapes(q):
     import torch
     x = torch.zeros(4096, device="cuda")

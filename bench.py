@@ -349,9 +349,11 @@ def cpu_gemm(args):
                       % (M, D, F, reps, "cpu_rt.h sg_core via g_ab/g_abt_b/g_atb" if kind == "reference" else "oracle/qlm_oracle.c")}
 
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the 1 GiB copy calibration);
-# the runs, counter values and scale factors are in profiles/*.txt. None where not measured.
-PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": None, "decode": None}
+# HBM bytes from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the 1 GiB copy calibration); the runs,
+# counter values and scale factors are in profiles/*.txt. adamw: per launch. train: per step, i.e. summed over
+# the step's 7 launches (1020 MiB read + 1104 MiB written). decode: per launch = per layer at T=16
+# (56.2 MiB read + 4.5 MiB written).
+PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.227e9, "decode": 6.37e7}
 
 
 def main():

@@ -39,6 +39,21 @@ struct GroupCtx {           /* per-group constants, uniform over the row */
 
 struct ElemRes { float mn, rv; int dd, rr, idl, carry; };
 
+/* Division of many values by one per-group divisor (the requantisation of the moments, qlm.cuh:261-278).
+ * With y = 1/b correctly rounded (one real division per group), q = a*y, r = fma(-q, b, a) exact and
+ * q' = fma(r, y, q), q' is the correctly rounded a/b (Markstein's final-step theorem) as long as nothing
+ * leaves the normal range; checked against a/b on 4e9 pairs on the CPU. The short form is used only
+ * when b is in [2^-60, 2^60] (|a| is at most 255 b here); quotients so small that r is subnormal are
+ * far below 2^-24 and round stochastically to the same integer either way. Anything else divides. */
+struct GroupDiv { float b, y; bool fast; };
+__device__ __forceinline__ GroupDiv qx_mkdiv(float b){
+    GroupDiv d; d.b = b; d.fast = b >= 0x1p-60f && b <= 0x1p60f; d.y = 1.0f / b; return d;
+}
+__device__ __forceinline__ float qx_gdiv(float a, const GroupDiv &d){
+    if(d.fast){ const float q = a * d.y; const float r = fmaf(-q, d.b, a); return fmaf(r, d.y, q); }
+    return a / d.b;
+}
+
 /* New first moment, new (stored form of the) second moment and the clamped Adam ratio u of one
  * element: qlm.cuh:209-229. */
 template<bool ADAM>
@@ -160,16 +175,17 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
         am = qx_row16_max(am); vm = qx_row16_max(vm);
         const float ms = am > 0.0f ? am / 127.0f : 1e-12f;
         const float vs = vm > 0.0f ? vm / 255.0f : 1e-12f;
+        const GroupDiv dms = qx_mkdiv(ms), dvs = qx_mkdiv(vs);
         if(lane16 == 0){ a.m8s[gi] = ms; if(ADAM) a.v8s[gi] = vs; }
         uint32_t mo0 = 0, mo1 = 0, vo0 = 0, vo1 = 0;
         key = q * QLMX_KI;
 #pragma unroll
         for(int k = 0; k < 8; k++){
             const int sh = 8 * (k & 3);
-            int mq = qx_clamp(qx_sround(mn[k] / ms, key + ktm), -127, 127);
+            int mq = qx_clamp(qx_sround(qx_gdiv(mn[k], dms), key + ktm), -127, 127);
             if(k < 4) mo0 |= ((uint32_t)mq & 0xFFu) << sh; else mo1 |= ((uint32_t)mq & 0xFFu) << sh;
             if(ADAM){
-                int vq = qx_clamp(qx_sround(rv[k] / vs, key + ktv), 0, 255);
+                int vq = qx_clamp(qx_sround(qx_gdiv(rv[k], dvs), key + ktv), 0, 255);
                 if(vq == 0 && rv[k] > 0.0f) vq = 1;
                 if(k < 4) vo0 |= (uint32_t)vq << sh; else vo1 |= (uint32_t)vq << sh;
             }

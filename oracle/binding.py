@@ -104,6 +104,7 @@ class Oracle(_Lib):
         self._dgate = s("orc_moe_dgate", None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i])
         self._swiglu = s("orc_swiglu", None, [c_vp, c_vp, c_vp, c_sz])
         self._swiglu_bwd = s("orc_swiglu_bwd", None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz])
+        self._recip = s("orc_recip_div_mismatches", c_sz, [C.c_uint64, c_sz])
         self._q4n_q = s("orc_q4n_quantize", c_sz, [c_vp, c_sz, c_i, c_vp, c_sz, c_vp])
         self._q4n_d = s("orc_q4n_dequantize", c_i, [c_vp, c_sz, c_vp, c_sz, c_i])
         self._ws_new = s("orc_moe_ws_new", c_vp, [c_i, c_i, c_i, c_i, c_i])
@@ -204,6 +205,9 @@ class Oracle(_Lib):
 
     def swiglu_bwd(self, Gg, U, dact, dg, du):
         self._swiglu_bwd(_p(Gg), _p(U), _p(dact), _p(dg), _p(du), Gg.size)
+
+    def recip_div_mismatches(self, seed, n):
+        return int(self._recip(seed, n))
 
     def q4n_quantize(self, P, group):
         """returns (bytes as uint8 array, number of raw groups)"""

@@ -694,6 +694,25 @@ int orc_q4n_dequantize(const unsigned char *buf, size_t len, float *P, size_t n,
 }
 
 /* ------------------------------------------------------------------------------------------
+ * Reciprocal-and-correct division identity (used by the GPU step kernel for the per-group divisors)
+ * ---------------------------------------------------------------------------------------- */
+size_t orc_recip_div_mismatches(uint64_t seed, size_t n){
+    size_t bad = 0;
+    #pragma omp parallel for reduction(+:bad) schedule(static)
+    for(long i = 0; i < (long)n; i++){
+        uint64_t h = orc_splitmix64(seed * 0x9E3779B97F4A7C15ULL + (uint64_t)i), h2 = orc_splitmix64(h);
+        uint32_t be = 127 - 60 + (uint32_t)(h % 121), bm = (uint32_t)(h >> 20) & 0x7FFFFF;
+        uint32_t bb = (be << 23) | bm;
+        int ae = (int)be + 8 - (int)(h2 % 40); if(ae < 1) ae = 1;
+        uint32_t ab = ((uint32_t)ae << 23) | ((uint32_t)(h2 >> 10) & 0x7FFFFF) | ((uint32_t)(h2 >> 63) << 31);
+        float a, b; memcpy(&a, &ab, 4); memcpy(&b, &bb, 4);
+        float y = 1.0f / b, q = a * y, r = fmaf(-q, b, a), q2 = fmaf(r, y, q), ref = a / b;
+        if(memcmp(&q2, &ref, 4) != 0) bad++;
+    }
+    return bad;
+}
+
+/* ------------------------------------------------------------------------------------------
  * Deterministic synthetic inputs
  * ---------------------------------------------------------------------------------------- */
 uint64_t orc_splitmix64(uint64_t x){

@@ -109,6 +109,11 @@ void orc_moe_backward(orc_moe_ws *w, const float *x, const float *w1, const floa
 size_t orc_q4n_quantize(const float *P, size_t n, int group, unsigned char *out, size_t cap, size_t *nraw);
 int    orc_q4n_dequantize(const unsigned char *buf, size_t len, float *P, size_t n, int group);
 
+/* ---- check of an identity the GPU step kernel relies on (not part of the reference): for b in
+ *      [2^-60, 2^60] and |a| <= 2^9 b, with y = 1/b, q = a*y, r = fma(-q,b,a): fma(r,y,q) == a/b bit for
+ *      bit. Returns the number of mismatches over n pseudo-random pairs drawn from `seed`. ---- */
+size_t orc_recip_div_mismatches(uint64_t seed, size_t n);
+
 /* ---- deterministic synthetic inputs: splitmix64 keyed by (seed, tensor id), top 24 bits as a
  *      uniform, Irwin-Hall sum of 12 uniforms minus 6 as a normal. Integer and exactly-rounded
  *      fp32 operations only, so every machine produces the same bits. ---- */

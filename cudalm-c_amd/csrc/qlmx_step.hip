@@ -29,6 +29,9 @@ struct StepParams {
     unsigned long long t; unsigned long long *stat;
     int packed, gi_base, ng, v4;
     int vec_ok;      /* base pointers are aligned for the 128/64/32-bit accesses of the fast path */
+    /* touched-group form (k_ng_q4_step, cudalm.cu:4472): team w steps group touched[w] of one span
+     * that starts at element 0, and its gradient is the compact row Gc[w*group ..] */
+    const int *touched; qlmx_span one;
 };
 
 struct GroupCtx {           /* per-group constants, uniform over the row */
@@ -100,13 +103,13 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
     const int lane16 = threadIdx.x & 15;
     const int team = (int)((blockIdx.x * (unsigned)blockDim.x + threadIdx.x) >> 4);
     if(team >= a.ng) return;                       /* whole rows leave together */
-    const int gi = a.gi_base + team;
-    const int si = qx_span_of(a.sp, a.nspan, gi);
-    const qlmx_span S = a.sp[si];
+    const int gi = a.touched ? a.touched[team] : a.gi_base + team;
+    const qlmx_span S = a.touched ? a.one : a.sp[qx_span_of(a.sp, a.nspan, gi)];
     const uint64_t j0 = (uint64_t)(gi - S.gi0) * (uint64_t)a.group;
     const uint64_t left = S.n - j0;
     const int n = (int)((uint64_t)a.group < left ? (uint64_t)a.group : left);
-    const uint64_t pof = S.pof + j0, qi0 = S.qi0 + j0, gof = S.gof + j0;
+    const uint64_t pof = S.pof + j0, qi0 = S.qi0 + j0;
+    const uint64_t gof = a.touched ? (uint64_t)team * (uint64_t)a.group : S.gof + j0;
 
     GroupCtx c;
     c.gs = a.gsp ? *a.gsp : a.gscale;
@@ -289,6 +292,7 @@ extern "C" int qlmx_step(float *P, const float *G, signed char *d, signed char *
     a.lr = lr; a.b1 = b1; a.b2 = b2; a.wd = wd; a.gscale = gscale; a.gsp = gsp;
     a.inv_bc1 = inv_bc1; a.inv_sqrt_bc2 = inv_sqrt_bc2; a.lrmode = lrmode;
     a.t = t; a.stat = (unsigned long long *)stat; a.packed = packed; a.gi_base = gi_base; a.ng = ng; a.v4 = v4;
+    a.touched = nullptr;
     a.vec_ok = (((uintptr_t)P | (uintptr_t)G) & 15) == 0 && (((uintptr_t)r | (uintptr_t)m8 | (uintptr_t)v8) & 7) == 0
                && ((uintptr_t)d & 3) == 0;
     const unsigned blocks = (unsigned)((ng + 15) / 16);
@@ -296,5 +300,39 @@ extern "C" int qlmx_step(float *P, const float *G, signed char *d, signed char *
     if(adam) hipLaunchKernelGGL(k_qlmx_step<true>,  dim3(blocks), dim3(256), 0, st, a);
     else     hipLaunchKernelGGL(k_qlmx_step<false>, dim3(blocks), dim3(256), 0, st, a);
     QLMX_LAUNCH_CHECK("qlmx_step launch");
+    return QLMX_OK;
+}
+
+/* k_ng_q4_step (cudalm.cu:4472-4520; CPU twin cpu_kern.h:620-648): the step restricted to a list of
+ * touched groups of ONE packed 4-bit span that starts at element 0 of d/r/m8/v8/P (the n-gram
+ * table). Same arithmetic as qlmx_step with adam = 1, relative LR through the frozen `sref`,
+ * no statistics, clip multiplier *gs (1 when NULL); group w of the list reads its gradient from the
+ * compact buffer Gc[w*group .. w*group+group). A group must appear at most once in the list. */
+extern "C" int qlmx_step_touched(float *P, const float *Gc, signed char *d, signed char *r, const float *s,
+              signed char *m8, float *m8s, unsigned char *v8, float *v8s,
+              const int *touched_gi, int ntouched, int group, int dmax,
+              float lr, float b1, float b2, float wd, float sref,
+              float inv_bc1, float inv_sqrt_bc2, unsigned long long t, unsigned long long nt,
+              const float *gs, int v4, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(Gc && d && r && s && m8 && m8s && v8 && v8s && touched_gi, "qlmx_step_touched: NULL buffer");
+    QLMX_REQUIRE(group >= 2 && group <= 256 && (group & 1) == 0, "qlmx_step_touched: group %d must be even and in [2,256]", group);
+    QLMX_REQUIRE(dmax >= 1 && dmax <= 7, "qlmx_step_touched: dmax %d (packed digits)", dmax);
+    QLMX_REQUIRE(ntouched >= 0 && nt > 0, "qlmx_step_touched: bad sizes");
+    if(ntouched == 0) return QLMX_OK;
+    StepParams a;
+    a.P = P; a.G = Gc; a.d = d; a.r = r; a.s = s; a.m8 = m8; a.m8s = m8s; a.v8 = v8; a.v8s = v8s;
+    a.sp = nullptr; a.nspan = 1; a.group = group; a.dmax = dmax;
+    a.lr = lr; a.b1 = b1; a.b2 = b2; a.wd = wd; a.gscale = 1.0f; a.gsp = gs;
+    a.inv_bc1 = inv_bc1; a.inv_sqrt_bc2 = inv_sqrt_bc2; a.lrmode = 0;
+    a.t = t; a.stat = nullptr; a.packed = 1; a.gi_base = 0; a.ng = ntouched; a.v4 = v4;
+    a.vec_ok = (((uintptr_t)P | (uintptr_t)Gc) & 15) == 0 && (((uintptr_t)r | (uintptr_t)m8 | (uintptr_t)v8) & 7) == 0
+               && ((uintptr_t)d & 3) == 0;
+    a.touched = touched_gi;
+    a.one.pof = 0; a.one.gof = 0; a.one.qi0 = 0; a.one.n = nt; a.one.gi0 = 0;
+    a.one.ngrp = (int)((nt + (unsigned long long)group - 1) / (unsigned long long)group); a.one.sref = sref;
+    const unsigned blocks = (unsigned)((ntouched + 15) / 16);
+    hipLaunchKernelGGL(k_qlmx_step<true>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+    QLMX_LAUNCH_CHECK("qlmx_step_touched launch");
     return QLMX_OK;
 }

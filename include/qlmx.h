@@ -91,6 +91,19 @@ int qlmx_step(float *P, const float *G, signed char *d, signed char *r, const fl
               unsigned long long t, int adam, long long *stat, int packed,
               int gi_base, int ng, int v4, void *stream);
 
+/* ---- k_ng_q4_step (cudalm.cu:4472-4520; cpu_kern.h:620-648), called from the n-gram table update
+ * (cudalm.cu:4752): the Integer AdamW step over a LIST of touched groups of one packed span that
+ * starts at element 0 of d/r/m8/v8/P and has `nt` elements. Group w of the list is touched_gi[w] and
+ * its gradient is the compact row Gc[w*group .. +group). Relative LR through the frozen `sref`,
+ * gscale = *gs (1 when NULL), no statistics; otherwise the arithmetic of qlmx_step, bit for bit.
+ * A group may be listed at most once. ---- */
+int qlmx_step_touched(float *P, const float *Gc, signed char *d, signed char *r, const float *s,
+                      signed char *m8, float *m8s, unsigned char *v8, float *v8s,
+                      const int *touched_gi, int ntouched, int group, int dmax,
+                      float lr, float b1, float b2, float wd, float sref,
+                      float inv_bc1, float inv_sqrt_bc2, unsigned long long t, unsigned long long nt,
+                      const float *gs, int v4, void *stream);
+
 /* ---- k_qlm_servo (qlm.cuh:404-441; launched from cudalm.cu:6099): rail-fraction scale servo
  * and re-encode of (d, r) for the groups whose scale moved. ---- */
 int qlmx_servo(signed char *d, signed char *r, float *s,

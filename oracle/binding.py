@@ -105,6 +105,8 @@ class Oracle(_Lib):
         self._swiglu = s("orc_swiglu", None, [c_vp, c_vp, c_vp, c_sz])
         self._swiglu_bwd = s("orc_swiglu_bwd", None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz])
         self._recip = s("orc_recip_div_mismatches", c_sz, [C.c_uint64, c_sz])
+        self._step_touched = s("orc_step_touched", None, [c_vp] * 10 + [c_i, c_i, c_i, c_f, c_f, c_f, c_f, c_f, c_f, c_f,
+                                                                       C.c_uint64, C.c_uint64, c_vp, c_i])
         self._q4n_q = s("orc_q4n_quantize", c_sz, [c_vp, c_sz, c_i, c_vp, c_sz, c_vp])
         self._q4n_d = s("orc_q4n_dequantize", c_i, [c_vp, c_sz, c_vp, c_sz, c_i])
         self._ws_new = s("orc_moe_ws_new", c_vp, [c_i, c_i, c_i, c_i, c_i])
@@ -206,6 +208,12 @@ class Oracle(_Lib):
     def swiglu_bwd(self, Gg, U, dact, dg, du):
         self._swiglu_bwd(_p(Gg), _p(U), _p(dact), _p(dg), _p(du), Gg.size)
 
+    def step_touched(self, P, Gc, d, r, s, m8, m8s, v8, v8s, touched, group, dmax, lr, b1, b2, wd, sref,
+                     inv_bc1, inv_sqrt_bc2, t, nt, gs=None, v4=0):
+        self._step_touched(_p(P), _p(Gc), _p(d), _p(r), _p(s), _p(m8), _p(m8s), _p(v8), _p(v8s), _p(touched),
+                           touched.size, group, dmax, lr, b1, b2, wd, sref, inv_bc1, inv_sqrt_bc2, t, nt,
+                           _p(gs) if gs is not None else None, v4)
+
     def recip_div_mismatches(self, seed, n):
         return int(self._recip(seed, n))
 
@@ -306,6 +314,8 @@ class Ref(_Lib):
         self._swiglu = s("ref_swiglu", None, [c_vp, c_vp, c_vp, c_sz])
         self._swiglu_bwd = s("ref_swiglu_bwd", None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz])
         self._q4n_q = s("ref_q4n_quantize", c_sz, [c_vp, c_sz, c_i, c_vp, c_sz])
+        self._ng_step = s("ref_ng_q4_step", None, [c_vp] * 10 + [c_i, c_i, c_i, c_f, c_f, c_f, c_f, c_f, c_f, c_f,
+                                                                 C.c_uint64, C.c_uint64, c_vp])
         self._q4n_d = s("ref_q4n_dequantize", c_i, [c_vp, c_sz, c_vp, c_sz, c_i])
         self._relerr = s("ref_relerr", c_f, [c_vp, c_vp, c_sz])
 
@@ -382,6 +392,14 @@ def _ref_q4n_dequantize(self, buf, n, group):
     return ok, P
 
 
+def _ref_step_touched(self, P, Gc, d, r, s, m8, m8s, v8, v8s, touched, group, dmax, lr, b1, b2, wd, sref,
+                      inv_bc1, inv_sqrt_bc2, t, nt, gs=None):
+    self._ng_step(_p(P), _p(Gc), _p(d), _p(r), _p(s), _p(m8), _p(m8s), _p(v8), _p(v8s), _p(touched),
+                  touched.size, group, dmax, lr, b1, b2, wd, sref, inv_bc1, inv_sqrt_bc2, t, nt,
+                  _p(gs) if gs is not None else None)
+
+
+Ref.step_touched = _ref_step_touched
 Ref.q4n_quantize = _ref_q4n_quantize
 Ref.q4n_dequantize = _ref_q4n_dequantize
 

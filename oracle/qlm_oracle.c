@@ -6,6 +6,9 @@
  *   encode/render                             fixtures (bit-exact) + half-step / 15-level invariants
  *   step (adam, lion, both lrmodes, gsp,      fixtures incl. forced carry cases (bit-exact), ref lib
  *         tail groups, unpacked, v4)          on 1e6-element seeded inputs when present
+ *   step_touched                              fixture written by the reference's k_ng_q4_step (bit-exact) +
+ *                                             equality with step() on a full gradient whose untouched
+ *                                             groups are left out
  *   servo                                     fixtures with forced grow / shrink / idle groups
  *   gemm nn/tn/nt                             double-precision triple loop + ref lib
  *   fexp / router_topk / perm                 fixtures (bit-exact) + brute force stable-sort check
@@ -192,7 +195,7 @@ static void step_group(int gi, float *P, const float *G, int8_t *d, int8_t *r, c
                        const orc_span *sp, int nspan, int group, int dmax,
                        float lr, float b1, float b2, float wd, float gs,
                        float inv_bc1, float inv_sqrt_bc2, int lrmode, uint64_t t, int adam,
-                       int packed, int v4, long long *st){
+                       int packed, int v4, long long *st, const float *Gcompact){
     grp_loc L = locate(sp, nspan, gi, group);
     const orc_span *S = &sp[L.si];
     uint64_t pof = S->pof + L.j0, qi0 = S->qi0 + L.j0, gof = S->gof + L.j0;
@@ -205,7 +208,7 @@ static void step_group(int gi, float *P, const float *G, int8_t *d, int8_t *r, c
 
     for(int j = 0; j < L.n; j++){
         uint64_t qi = qi0 + j;
-        float gr = G[gof + j] * gs;
+        float gr = (Gcompact ? Gcompact[j] : G[gof + j]) * gs;
         float mv = (float)m8[qi] * ms_old;
         float u;
         rnew[j] = 0.0f;
@@ -278,10 +281,25 @@ void orc_step(float *P, const float *G, int8_t *d, int8_t *r, const float *s, in
         long long st[4] = {0, 0, 0, 0};
         step_group(gi_base + w, P, G, d, r, s, m8, m8s, v8, v8s, sp, nspan, group, dmax,
                    lr, b1, b2, wd, gs, inv_bc1, inv_sqrt_bc2, lrmode, t, adam, packed, v4,
-                   stat ? st : NULL);
+                   stat ? st : NULL, NULL);
         s0 += st[0]; s1 += st[1]; s2 += st[2]; if(st[3] > s3) s3 = st[3];
     }
     if(stat){ stat[0] += s0; stat[1] += s1; stat[2] += s2; if(s3 > stat[3]) stat[3] = s3; }
+}
+
+/* cpu_kern.h:620-648 (k_ng_q4_step, GPU form cudalm.cu:4472-4520): the same group update driven by a
+ * list of touched groups of one packed span that starts at element 0; group w reads its gradient
+ * from the compact row Gc[w*group ..]. adam, relative LR through sref, gscale = *gs or 1. */
+void orc_step_touched(float *P, const float *Gc, int8_t *d, int8_t *r, const float *s, int8_t *m8, float *m8s,
+                      uint8_t *v8, float *v8s, const int *touched_gi, int ntouched, int group, int dmax,
+                      float lr, float b1, float b2, float wd, float sref, float inv_bc1, float inv_sqrt_bc2,
+                      uint64_t t, uint64_t nt, const float *gs, int v4){
+    orc_span one; memset(&one, 0, sizeof one);
+    one.n = nt; one.ngrp = (int)((nt + (uint64_t)group - 1) / (uint64_t)group); one.sref = sref;
+    #pragma omp parallel for schedule(static)
+    for(int w = 0; w < ntouched; w++)
+        step_group(touched_gi[w], P, NULL, d, r, s, m8, m8s, v8, v8s, &one, 1, group, dmax, lr, b1, b2, wd,
+                   gs ? gs[0] : 1.0f, inv_bc1, inv_sqrt_bc2, 0, t, 1, 1, v4, NULL, Gc + (size_t)w * group);
 }
 
 /* ------------------------------------------------------------------------------------------

@@ -50,6 +50,11 @@ void orc_step(float *P, const float *G, int8_t *d, int8_t *r, const float *s, in
               float lr, float b1, float b2, float wd, float gscale, const float *gsp,
               float inv_bc1, float inv_sqrt_bc2, int lrmode, uint64_t t, int adam,
               long long *stat, int packed, int gi_base, int ng, int v4);
+/* cpu_kern.h:620-648 / cudalm.cu:4472-4520: touched-group form over one span starting at element 0 */
+void orc_step_touched(float *P, const float *Gc, int8_t *d, int8_t *r, const float *s, int8_t *m8, float *m8s,
+                      uint8_t *v8, float *v8s, const int *touched_gi, int ntouched, int group, int dmax,
+                      float lr, float b1, float b2, float wd, float sref, float inv_bc1, float inv_sqrt_bc2,
+                      uint64_t t, uint64_t nt, const float *gs, int v4);
 void orc_servo(int8_t *d, int8_t *r, float *s, const orc_span *sp, int nspan, int group, int dmax,
                float f_hi, float f_lo, int packed, int ngrp);
 

@@ -62,6 +62,14 @@ void ref_step_block(float*P,const float*G,signed char*d,signed char*r,float*s,si
     KL(k_qlm_step,(unsigned)ng,group,group)(P,G,d,r,s,m8,m8s,v8,v8s,sp,nspan,group,dmax,
         lr,b1,b2,wd,gscale,inv_bc1,inv_sqrt_bc2,lrmode,t,adam,stat,packed,gi_base);
 }
+/* cudalm.cu:4472 through its CPU twin cpu_kern.h:620-648 */
+void ref_ng_q4_step(float*P,const float*Gc,signed char*d,signed char*r,float*s,signed char*m8,float*m8s,
+                    unsigned char*v8,float*v8s,const int*touched,int ntouched,int group,int dmax,
+                    float lr,float b1,float b2,float wd,float sref,float inv_bc1,float inv_sqrt_bc2,
+                    unsigned long long t,unsigned long long nt,const float*gs){
+    KL(k_ng_q4_step,(unsigned)ntouched,group,group)(P,Gc,d,r,s,m8,m8s,v8,v8s,touched,group,dmax,
+        lr,b1,b2,wd,sref,inv_bc1,inv_sqrt_bc2,t,nt,gs);
+}
 void ref_servo(signed char*d,signed char*r,float*s,const QSpanD*sp,int nspan,int group,int dmax,
                float f_hi,float f_lo,int packed,int ngrp){
     KL(k_qlm_servo,(unsigned)ngrp,group,group)(d,r,s,sp,nspan,group,dmax,f_hi,f_lo,packed);

@@ -222,6 +222,40 @@ def golden_glue():
          dout=dout, dgate=dgate, dyp=dyp, G=G, U=U, dA=dA, O=O, dg=dg, du=du)
 
 
+def golden_step_touched():
+    """k_ng_q4_step (cpu_kern.h:620-648): two steps over a list of touched groups of one packed span of
+    128*10 + 64 weights (the last group is a short tail), compact gradients, the second step with a
+    device clip scalar and a large learning rate (carries)."""
+    group, dmax = 128, 7
+    nt = 128 * 10 + 64
+    ng = 11
+    d = gen.digits(nt, 0, 950)
+    r = gen.int8(nt, 0, 951, -64, 64)
+    m8 = gen.int8(nt, 0, 952, -127, 127)
+    v8 = gen.u8(nt, 0, 953, 0, 255)
+    s = (0.02 * 3 / 7) * gen.uniform(ng, 0, 954, 0.5, 1.5)
+    m8s = (3e-3 / 127) * gen.uniform(ng, 0, 955, 0.5, 1.5)
+    v8s = (3e-3 / 255) * gen.uniform(ng, 0, 956, 0.5, 1.5)
+    sref = float(np.mean(s.astype(np.float64)))
+    P = np.zeros(nt, f32)
+    out = {"dims": np.array([nt, group, dmax]), "sref": np.array([sref], f32),
+           "d0": d.copy(), "r0": r.copy(), "m8_0": m8.copy(), "v8_0": v8.copy(), "s": s.copy(),
+           "m8s_0": m8s.copy(), "v8s_0": v8s.copy()}
+    b1, b2, wd = 0.9, 0.95, 0.1
+    for t, touched, lr, gs in [(1, [0, 3, 7, 10], 3e-4, None), (2, [10, 2, 3], 0.05, np.array([0.37], f32))]:
+        touched = np.array(touched, np.int32)
+        Gc = gen.normal(touched.size * group, 0, 960 + t, 1e-3 if t == 1 else 0.2)
+        bc1 = f32(1) - f32(b1) ** f32(t); bc2 = f32(1) - f32(b2) ** f32(t)
+        inv_bc1 = float(f32(1) / bc1); inv_sqrt_bc2 = float(f32(1) / np.sqrt(bc2))
+        ref.step_touched(P, Gc, d, r, s, m8, m8s, v8, v8s, touched, group, dmax, lr, b1, b2, wd, sref,
+                         inv_bc1, inv_sqrt_bc2, t, nt, gs)
+        out.update({"touched%d" % t: touched, "Gc%d" % t: Gc, "hp%d" % t: np.array([lr, b1, b2, wd, inv_bc1, inv_sqrt_bc2], f32),
+                    "P%d" % t: P.copy(), "d%d" % t: d.copy(), "r%d" % t: r.copy(), "m8_%d" % t: m8.copy(),
+                    "v8_%d" % t: v8.copy(), "m8s_%d" % t: m8s.copy(), "v8s_%d" % t: v8s.copy()})
+    out["gs2"] = np.array([0.37], f32)
+    save("step_touched", **out)
+
+
 def golden_q4n():
     """q4n wire format (cudalm.cu:638-656): groups on the 4-bit grid (rendered QLM view), groups off
     the grid (stored raw), an all-zero group, a one-hot group and a short tail."""
@@ -246,6 +280,7 @@ def golden_q4n():
 
 if __name__ == "__main__":
     golden_q4n()
+    golden_step_touched()
     golden_hash()
     golden_nibble()
     golden_qlm()

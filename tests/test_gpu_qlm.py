@@ -136,6 +136,56 @@ def test_encode_render_vs_oracle_and_invariants(q, orc):
     assert float((P2 - P).abs().max()) <= float(s.max()) * 1e-6 and int(r2.abs().max()) <= 1
 
 
+def test_step_touched_vs_reference_fixture(q, golden):
+    """k_ng_q4_step (cudalm.cu:4472): list-driven step, bytes and bits against the reference's output."""
+    import torch
+    g = golden("step_touched")
+    nt, group, dmax = (int(v) for v in g["dims"])
+    d, r, m8, v8 = dev(g["d0"]), dev(g["r0"]), dev(g["m8_0"]), dev(g["v8_0"])
+    s, m8s, v8s = dev(g["s"]), dev(g["m8s_0"]), dev(g["v8s_0"])
+    P = torch.zeros(nt, device="cuda")
+    gs2 = dev(g["gs2"])
+    for t in (1, 2):
+        lr, b1, b2, wd, ib1, ib2 = (float(v) for v in g["hp%d" % t])
+        touched = dev(g["touched%d" % t])
+        q.step_touched(P, dev(g["Gc%d" % t]), d, r, s, m8, m8s, v8, v8s, touched, touched.numel(), group, dmax,
+                       lr, b1, b2, wd, float(g["sref"][0]), ib1, ib2, t, nt, gs2 if t == 2 else None)
+        torch.cuda.synchronize()
+        for name, got in (("d", d), ("r", r), ("m8_", m8), ("v8_", v8), ("m8s_", m8s), ("v8s_", v8s), ("P", P)):
+            assert beq(got, g["%s%d" % (name, t)]), (name, t)
+
+
+@pytest.mark.parametrize("v4", [0, 1])
+def test_step_touched_vs_oracle_sparse_table(q, orc, v4):
+    """A 4 M-weight table of which 3000 random groups are touched (plus the short tail group)."""
+    import torch
+    group, dmax = 128, 7
+    nt = 128 * 32768 + 96
+    ng = (nt + group - 1) // group
+    d, r = orc.digits(nt, 6, 1), orc.int8(nt, 6, 2, -64, 64)
+    m8, v8 = orc.int8(nt, 6, 3, -127, 127), orc.u8(nt, 6, 4, 0, 255)
+    s = (0.02 * 3 / 7) * orc.uniform(ng, 6, 5, 0.5, 1.5)
+    m8s = (3e-3 / 127) * orc.uniform(ng, 6, 6, 0.5, 1.5)
+    v8s = (3e-3 / 255) * orc.uniform(ng, 6, 7, 0.5, 1.5)
+    if v4:
+        v8s = np.sqrt(v8s).astype(f32)
+    rng = np.random.default_rng(6)
+    touched = np.concatenate([rng.choice(ng - 1, 3000, replace=False), [ng - 1]]).astype(np.int32)
+    Gc = orc.normal(touched.size * group, 6, 8, 1e-3)
+    gs = np.array([0.81], f32)
+    sref = float(np.mean(s.astype(np.float64)))
+    dd, dr, dm8, dv8, dm8s, dv8s = dev(d), dev(r), dev(m8), dev(v8), dev(m8s), dev(v8s)
+    P = torch.zeros(nt, device="cuda")
+    q.step_touched(P, dev(Gc), dd, dr, dev(s), dm8, dm8s, dv8, dv8s, dev(touched), touched.size, group, dmax,
+                   3e-4, 0.9, 0.95, 0.1, sref, 10.0, 4.47, 7, nt, dev(gs), v4)
+    torch.cuda.synchronize()
+    Ph = np.zeros(nt, f32)
+    orc.step_touched(Ph, Gc, d, r, s, m8, m8s, v8, v8s, touched, group, dmax, 3e-4, 0.9, 0.95, 0.1, sref, 10.0, 4.47,
+                     7, nt, gs, v4)
+    for got, want in ((dd, d), (dr, r), (dm8, m8), (dv8, v8), (dm8s, m8s), (dv8s, v8s), (P, Ph)):
+        assert beq(got, want)
+
+
 def test_argument_errors(q):
     import torch
     x = torch.zeros(256, device="cuda")

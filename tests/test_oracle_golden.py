@@ -419,3 +419,59 @@ def test_reciprocal_division_identity(orc):
     would differ from the reference's: no mismatch on 2e8 pseudo-random pairs over the range the
     kernel admits (b in [2^-60, 2^60], |a| up to 2^9 b and down to 2^-31 b)."""
     assert orc.recip_div_mismatches(1, 200_000_000) == 0
+
+
+def _touched_state(g):
+    return (g["d0"].copy(), g["r0"].copy(), g["m8_0"].copy(), g["v8_0"].copy(), g["m8s_0"].copy(), g["v8s_0"].copy())
+
+
+def test_step_touched_vs_reference_fixture(orc, golden):
+    """k_ng_q4_step (cpu_kern.h:620-648): bytes of d, r, m8, v8 and bits of the scales and of P after
+    each of two steps over different touched-group lists (short tail group, clip scalar, carries)."""
+    g = golden("step_touched")
+    nt, group, dmax = (int(v) for v in g["dims"])
+    d, r, m8, v8, m8s, v8s = _touched_state(g)
+    P = np.zeros(nt, np.float32)
+    for t in (1, 2):
+        lr, b1, b2, wd, ib1, ib2 = (float(v) for v in g["hp%d" % t])
+        orc.step_touched(P, g["Gc%d" % t], d, r, g["s"], m8, m8s, v8, v8s, g["touched%d" % t], group, dmax,
+                         lr, b1, b2, wd, float(g["sref"][0]), ib1, ib2, t, nt, g["gs2"] if t == 2 else None)
+        for name, got in (("d", d), ("r", r), ("m8_", m8), ("v8_", v8)):
+            assert np.array_equal(got, g["%s%d" % (name, t)]), (name, t)
+        for name, got in (("m8s_", m8s), ("v8s_", v8s), ("P", P)):
+            assert np.array_equal(got.view(np.uint32), g["%s%d" % (name, t)].view(np.uint32)), (name, t)
+
+
+def test_step_touched_equals_full_step_on_the_touched_groups(orc):
+    """The list-driven form is the ordinary step restricted to the listed groups: run both from the
+    same state, with the compact gradient scattered into a full one, and compare the listed groups."""
+    from oracle.binding import make_spans
+    group, dmax, nt = 128, 7, 128 * 20
+    tab, nq, ng = make_spans([nt], group)
+    mk = lambda: (orc.digits(nt, 3, 1), orc.int8(nt, 3, 2, -64, 64), orc.int8(nt, 3, 3, -127, 127), orc.u8(nt, 3, 4, 0, 255),
+                  (3e-3 / 127) * orc.uniform(ng, 3, 5, 0.5, 1.5), (3e-3 / 255) * orc.uniform(ng, 3, 6, 0.5, 1.5))
+    s = (0.02 * 3 / 7) * orc.uniform(ng, 3, 7, 0.5, 1.5)
+    orc.span_sref(tab, s)
+    touched = np.array([1, 4, 5, 19, 11], np.int32)
+    Gc = orc.normal(touched.size * group, 3, 8, 1e-3)
+    G = np.zeros(nt, np.float32)
+    for w, gi in enumerate(touched):
+        G[gi * group:(gi + 1) * group] = Gc[w * group:(w + 1) * group]
+    a, b = mk(), mk()
+    Pa, Pb = np.zeros(nt, np.float32), np.zeros(nt, np.float32)
+    orc.step_touched(Pa, Gc, a[0], a[1], s, a[2], a[4], a[3], a[5], touched, group, dmax, 3e-4, 0.9, 0.95, 0.1,
+                     float(tab[0]["sref"]), 10.0, 4.47, 1, nt)
+    orc.step(Pb, G, b[0], b[1], s, b[2], b[4], b[3], b[5], tab, group, dmax, 3e-4, 0.9, 0.95, 0.1, 1.0, None,
+             10.0, 4.47, 0, 1, 1, None, 1, 0, ng)
+    for gi in touched:
+        sl = slice(gi * group, (gi + 1) * group)
+        assert np.array_equal(a[0][gi * 64:(gi + 1) * 64], b[0][gi * 64:(gi + 1) * 64])
+        for k in (1, 2, 3):
+            assert np.array_equal(a[k][sl], b[k][sl])
+        assert a[4][gi] == b[4][gi] and a[5][gi] == b[5][gi]
+        assert np.array_equal(Pa[sl], Pb[sl])
+    untouched = np.setdiff1d(np.arange(ng), touched)
+    base = mk()
+    for gi in untouched:
+        sl = slice(gi * group, (gi + 1) * group)
+        assert np.array_equal(a[1][sl], base[1][sl]) and np.array_equal(a[2][sl], base[2][sl])

@@ -37,8 +37,10 @@ typedef float  f32x2  __attribute__((ext_vector_type(2)));
 typedef float  f32x16 __attribute__((ext_vector_type(16)));
 
 #define BN 128
-#define BK 32
+#define BK 32                /* contraction depth of a step for nn and nt */
 #define KO 4                 /* 16-byte items per row per step */
+#define BK_TN 64             /* tn: 64 deep, so that a step reads whole 128-byte lines of the bf16 rows and
+                              * carries 16 MFMAs per wavefront between barriers */
 
 struct MfmaArgs { const DevProb *pr; int nprob, ntiles, tiles_n, rows_p; const signed char *d; const float *s; int group, gshift; int K, N; };
 
@@ -51,7 +53,8 @@ __device__ __forceinline__ uint4 pk8_bf16(const float *p){
     const float4 a = *(const float4 *)p, b = *(const float4 *)(p + 4);
     return make_uint4(pk_bf16(a.x, a.y), pk_bf16(a.z, a.w), pk_bf16(b.x, b.y), pk_bf16(b.z, b.w));
 }
-template<int ROWS> __device__ __forceinline__ int item_at(int ko, int row){
+template<int ROWS, int KOT = KO> __device__ __forceinline__ int item_at(int ko, int row){
+    if constexpr(KOT == 8) return ko * ROWS + (row ^ ((ko << 1) & 15));      /* 128-bit accesses only: 8 items x 2 rows fill the banks */
     return ko * ROWS + (row ^ (((row >> 4) ^ (ko << 2)) & 15));
 }
 
@@ -59,7 +62,9 @@ template<int MODE, bool BF16, int WM, bool DEEP>
 __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
     constexpr int BM = 64 * WM;
     constexpr int NB = MODE == GEMM_NN ? 2 : 1;                 /* B planes: hi (+ lo) */
-    constexpr int A_BYTES = KO * BM * 16, B_BYTES = KO * BN * 16;
+    constexpr int KOT = MODE == GEMM_TN ? BK_TN / 8 : KO;      /* items per row per step */
+    constexpr int BKT = KOT * 8;                               /* contraction depth of a step */
+    constexpr int A_BYTES = KOT * BM * 16, B_BYTES = KOT * BN * 16;
     /* one LDS block: [buffer 0: A | B hi | B lo][buffer 1: ...] */
     constexpr int BUF_BYTES = A_BYTES + NB * B_BYTES;
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * BUF_BYTES];
@@ -98,13 +103,13 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
      * (advanced by a constant per step), LDS byte offsets of this thread's stores and of its MFMA
      * operand reads. Rows past the end of a problem are clamped to its last row instead of being
      * zero-filled when they only feed output rows that are never stored. ---- */
-    constexpr int NA = MODE == GEMM_NT ? 4 : WM;       /* 16-byte A-side loads per thread per step */
+    constexpr int NA = MODE == GEMM_NT ? 4 : WM * KOT / 4;    /* 16-byte A-side loads per thread per step */
     constexpr int ESZ = BF16 ? 2 : 4;
     const char *pa[NA];                                /* A-side source pointers                    */
     const char *pb[2];                                 /* nt: B-side source pointers                */
     const signed char *pw0 = a.d, *pw1 = a.d;          /* nn: digit rows k, k+1; tn: row n          */
     const float *ps0 = a.s, *ps1 = a.s;                /* nn: their scales                          */
-    int sa_off[MODE == GEMM_NT ? 2 : WM];              /* LDS store offsets, A side (nt: per task)  */
+    int sa_off[MODE == GEMM_NT ? 2 : NA];              /* LDS store offsets, A side (nt: per task)  */
     int sj_off[8];                                     /* transposing stores: the 8 row offsets     */
     int sb_off = 0, sbj_off[8];                        /* B side                                    */
     size_t astep, bstep = 0, wstep = 0, sstep = 0;     /* per-step advances in bytes / elements     */
@@ -132,13 +137,13 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
         astep = (size_t)BK * a.K * ESZ; bstep = (size_t)BK * a.N * ESZ;
     } else {
 #pragma unroll
-        for(int h = 0; h < WM; h++){
-            const int id = tid + 256 * h, kq = id & 3, r = id >> 2;
+        for(int h = 0; h < NA; h++){
+            const int id = tid + 256 * h, kq = id & (KOT - 1), r = id / KOT;
             const int rr = (i0 + r < rows) ? i0 + r : rows - 1;            /* clamp: feeds unstored rows only */
             pa[h] = (const char *)P.A + ((size_t)rr * a.K + kq * 8) * ESZ;
-            sa_off[h] = item_at<BM>(kq, r) * 16;
+            sa_off[h] = item_at<BM, KOT>(kq, r) * 16;
         }
-        astep = (size_t)BK * ESZ;
+        astep = (size_t)BKT * ESZ;
         if constexpr(MODE == GEMM_NN){
             const int oc = tid & 15, kp = tid >> 4, ko = kp >> 2;
             const size_t e0 = (size_t)(2 * kp) * a.N + j0 + oc * 8;
@@ -150,21 +155,22 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
 #pragma unroll
             for(int j = 0; j < 8; j++) sbj_off[j] = ((oc * 8 + j) ^ sw) * 16;
         } else {
-            const int n = tid & (BN - 1);
-            pw0 = a.d + ((P.wq + (size_t)(j0 + n) * a.K) >> 1);
-            wstep = BK >> 1;
+            /* thread = (row n, half of the step's 64 digits): 16 bytes = 32 digits = 4 items */
+            const int n = tid & (BN - 1), half = tid >> 7;
+            pw0 = a.d + ((P.wq + (size_t)(j0 + n) * a.K) >> 1) + half * 16;
+            wstep = BKT >> 1;
 #pragma unroll
-            for(int ko = 0; ko < KO; ko++) sbj_off[ko] = A_BYTES + item_at<BN>(ko, n) * 16;
+            for(int ko = 0; ko < 4; ko++) sbj_off[ko] = A_BYTES + item_at<BN, KOT>(half * 4 + ko, n) * 16;
         }
     }
     /* MFMA operand read offsets: [k16 half][tile] */
-    int ra_off[2][WM], rb_off[2][2];
+    int ra_off[KOT / 2][WM], rb_off[KOT / 2][2];
 #pragma unroll
-    for(int ks = 0; ks < 2; ks++){
+    for(int ks = 0; ks < KOT / 2; ks++){
 #pragma unroll
-        for(int i = 0; i < WM; i++) ra_off[ks][i] = item_at<BM>(ks * 2 + hf, wi + i * 32 + fr) * 16;
+        for(int i = 0; i < WM; i++) ra_off[ks][i] = item_at<BM, KOT>(ks * 2 + hf, wi + i * 32 + fr) * 16;
 #pragma unroll
-        for(int j = 0; j < 2; j++) rb_off[ks][j] = A_BYTES + item_at<BN>(ks * 2 + hf, wj + j * 32 + fr) * 16;
+        for(int j = 0; j < 2; j++) rb_off[ks][j] = A_BYTES + item_at<BN, KOT>(ks * 2 + hf, wj + j * 32 + fr) * 16;
     }
 
     struct Stage {
@@ -206,13 +212,13 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
             G.rw.x = (uint32_t)p0;                     /* remembered for the zeroing at store time */
         } else {
 #pragma unroll
-            for(int h = 0; h < WM; h++){ G.ra[h] = ld16(pa[h]); pa[h] += astep; }
+            for(int h = 0; h < NA; h++){ G.ra[h] = ld16(pa[h]); pa[h] += astep; }
             if constexpr(MODE == GEMM_NN){
                 G.rw.x = *(const uint32_t *)pw0; G.rw.y = *(const uint32_t *)pw1;
                 G.rs0 = *ps0; G.rs1 = *ps1;
                 pw0 += wstep; pw1 += wstep; ps0 += sstep; ps1 += sstep;
             } else {
-                if(tid < BN) G.rw = *(const uint4 *)pw0;
+                G.rw = *(const uint4 *)pw0;
                 pw0 += wstep;
             }
         }
@@ -240,7 +246,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
                   *(uint32_t *)(L + sb_off + sbj_off[j]) = __builtin_amdgcn_perm(y1[j >> 1], y0[j >> 1], (j & 1) ? 0x07060302u : 0x05040100u); }
         } else {
 #pragma unroll
-            for(int h = 0; h < WM; h++) *(uint4 *)(L + sa_off[h]) = G.ra[h];
+            for(int h = 0; h < NA; h++) *(uint4 *)(L + sa_off[h]) = G.ra[h];
             if constexpr(MODE == GEMM_NN){
 #pragma unroll
                 for(int j = 0; j < 8; j++){
@@ -251,17 +257,15 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
                     *(uint32_t *)(L + sb_off + B_BYTES + sbj_off[j]) = pk_bf16(l0, l1);
                 }
             } else {
-                if(tid < BN){
-                    const uint32_t wd[4] = {G.rw.x, G.rw.y, G.rw.z, G.rw.w};
+                const uint32_t wd[4] = {G.rw.x, G.rw.y, G.rw.z, G.rw.w};
 #pragma unroll
-                    for(int ko = 0; ko < KO; ko++){
-                        uint4 v;
-                        v.x = pk_bf16((float)qx_nib(wd[ko], 0), (float)qx_nib(wd[ko], 1));
-                        v.y = pk_bf16((float)qx_nib(wd[ko], 2), (float)qx_nib(wd[ko], 3));
-                        v.z = pk_bf16((float)qx_nib(wd[ko], 4), (float)qx_nib(wd[ko], 5));
-                        v.w = pk_bf16((float)qx_nib(wd[ko], 6), (float)qx_nib(wd[ko], 7));
-                        *(uint4 *)(L + sbj_off[ko]) = v;
-                    }
+                for(int ko = 0; ko < 4; ko++){
+                    uint4 v;
+                    v.x = pk_bf16((float)qx_nib(wd[ko], 0), (float)qx_nib(wd[ko], 1));
+                    v.y = pk_bf16((float)qx_nib(wd[ko], 2), (float)qx_nib(wd[ko], 3));
+                    v.z = pk_bf16((float)qx_nib(wd[ko], 4), (float)qx_nib(wd[ko], 5));
+                    v.w = pk_bf16((float)qx_nib(wd[ko], 6), (float)qx_nib(wd[ko], 7));
+                    *(uint4 *)(L + sbj_off[ko]) = v;
                 }
             }
         }
@@ -270,7 +274,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
     auto compute = [&](int cb){
         const unsigned char *L = lds + cb * BUF_BYTES;
 #pragma unroll
-        for(int ks = 0; ks < 2; ks++){
+        for(int ks = 0; ks < KOT / 2; ks++){
             bf16x8 fa[WM], fb[2], fl[2];
 #pragma unroll
             for(int i = 0; i < WM; i++) fa[i] = __builtin_bit_cast(bf16x8, *(const uint4 *)(L + ra_off[ks][i]));
@@ -294,8 +298,8 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
         }
     };
 
-    const int steps = (depth + BK - 1) / BK;
-    const int steps_per_group = MODE == GEMM_TN ? (1 << a.gshift) / BK : 1;
+    const int steps = (depth + BKT - 1) / BKT;
+    const int steps_per_group = MODE == GEMM_TN ? (1 << a.gshift) / BKT : 1;
     const float *pfold[2] = {a.s, a.s};                /* tn: scale of (this lane's column, current group) */
     if constexpr(MODE == GEMM_TN){
 #pragma unroll
@@ -325,20 +329,20 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
      * with DEEP, which keeps two sets of staging registers; one otherwise). */
     if constexpr(DEEP){
         load_step(S0, 0);
-        if(steps > 1) load_step(S1, BK);
+        if(steps > 1) load_step(S1, BKT);
         store_step(S0, 0);
-        if(steps > 2) load_step(S0, 2 * BK);
+        if(steps > 2) load_step(S0, 2 * BKT);
         __syncthreads();
         for(int st = 0; st < steps; st += 2){
             compute(0);
             if(st + 1 < steps) store_step(S1, 1);
-            if(st + 3 < steps) load_step(S1, (st + 3) * BK);
+            if(st + 3 < steps) load_step(S1, (st + 3) * BKT);
             fold_group(st);
             __syncthreads();
             if(st + 1 < steps){
                 compute(1);
                 if(st + 2 < steps) store_step(S0, 0);
-                if(st + 4 < steps) load_step(S0, (st + 4) * BK);
+                if(st + 4 < steps) load_step(S0, (st + 4) * BKT);
                 fold_group(st + 1);
                 __syncthreads();
             }
@@ -346,12 +350,12 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
     } else {
         load_step(S0, 0);
         store_step(S0, 0);
-        if(steps > 1) load_step(S0, BK);
+        if(steps > 1) load_step(S0, BKT);
         __syncthreads();
         for(int st = 0; st < steps; st++){
             compute(st & 1);
             if(st + 1 < steps) store_step(S0, (st + 1) & 1);
-            if(st + 2 < steps) load_step(S0, (st + 2) * BK);
+            if(st + 2 < steps) load_step(S0, (st + 2) * BKT);
             fold_group(st);
             __syncthreads();
         }
@@ -411,8 +415,11 @@ int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int 
     /* shapes the tiling assumes; anything else must use QLMX_MATH_F32 */
     QLMX_REQUIRE(N % BN == 0, "mfma gemm: N=%d is not a multiple of %d (use QLMX_MATH_F32)", N, BN);
     if(mode == GEMM_NT) QLMX_REQUIRE(K % 8 == 0, "mfma gemm nt: K=%d is not a multiple of 8 (use QLMX_MATH_F32)", K);
-    else                QLMX_REQUIRE(K % BK == 0, "mfma gemm: K=%d is not a multiple of %d (use QLMX_MATH_F32)", K, BK);
-    if(mode != GEMM_NT) QLMX_REQUIRE(group >= BK && (group & (group - 1)) == 0, "mfma gemm: group %d must be a power of two >= %d (use QLMX_MATH_F32)", group, BK);
+    else {
+        const int bk = mode == GEMM_TN ? BK_TN : BK;
+        QLMX_REQUIRE(K % bk == 0, "mfma gemm: K=%d is not a multiple of %d (use QLMX_MATH_F32)", K, bk);
+        QLMX_REQUIRE(group >= bk && (group & (group - 1)) == 0, "mfma gemm: group %d must be a power of two >= %d (use QLMX_MATH_F32)", group, bk);
+    }
     for(int i = 0; i < nprob; i++){
         QLMX_REQUIRE(((uintptr_t)probs[i].A & 15) == 0 && (mode != GEMM_NT || ((uintptr_t)probs[i].B & 15) == 0),
                      "mfma gemm: problem %d operand is not 16-byte aligned", i);

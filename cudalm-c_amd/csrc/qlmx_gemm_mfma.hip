@@ -30,6 +30,7 @@
  * every expert of the call through a flattened (problem, row tile, column tile) list.
  */
 #include "qlmx_gemm.h"
+int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -426,6 +427,8 @@ int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int 
         QLMX_REQUIRE(mode == GEMM_NT || (probs[i].wq & 31ULL) == 0, "mfma gemm: problem %d weight offset not a multiple of 32", i);
     }
     QLMX_REQUIRE(mode == GEMM_NT || ((uintptr_t)d & 15) == 0, "mfma gemm: digit array is not 16-byte aligned");
+    /* bf16 weight gradients take the direct-to-LDS kernel; fp32 activations need the converting one */
+    if(mode == GEMM_NT && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nt_lds_launch(probs, nprob, K, N, st);
     if(mode == GEMM_NN) return launch_mfma<GEMM_NN, 4, true>(d, s, group, probs, nprob, K, N, act_dtype, st);
     if(mode == GEMM_TN) return launch_mfma<GEMM_TN, 2, false>(d, s, group, probs, nprob, K, N, act_dtype, st);
     return launch_mfma<GEMM_NT, 4, false>(d, s, group, probs, nprob, K, N, act_dtype, st);

@@ -30,6 +30,7 @@
  * every expert of the call through a flattened (problem, row tile, column tile) list.
  */
 #include "qlmx_gemm.h"
+int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
 int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -427,7 +428,14 @@ int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int 
         QLMX_REQUIRE(mode == GEMM_NT || (probs[i].wq & 31ULL) == 0, "mfma gemm: problem %d weight offset not a multiple of 32", i);
     }
     QLMX_REQUIRE(mode == GEMM_NT || ((uintptr_t)d & 15) == 0, "mfma gemm: digit array is not 16-byte aligned");
-    /* bf16 weight gradients take the direct-to-LDS kernel; fp32 activations need the converting one */
+    /* bf16 operands take the direct-to-LDS kernels; fp32 activations need the converting ones */
+    if(mode == GEMM_TN && act_dtype == QLMX_ACT_BF16){
+        /* measured: the direct-to-LDS input-gradient kernel wins from about 1000 rows per expert on
+         * (437 against 401 TFLOP/s at 2048), the register-staged one below that (421 against 398 at 512) */
+        long long rows = 0; int live = 0;
+        for(int i = 0; i < nprob; i++) if(probs[i].M > 0){ rows += probs[i].M; live++; }
+        if(live && rows / live >= 1024) return qlmx_gemm_tn_lds_launch(d, s, group, probs, nprob, K, N, st);
+    }
     if(mode == GEMM_NT && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nt_lds_launch(probs, nprob, K, N, st);
     if(mode == GEMM_NN) return launch_mfma<GEMM_NN, 4, true>(d, s, group, probs, nprob, K, N, act_dtype, st);
     if(mode == GEMM_TN) return launch_mfma<GEMM_TN, 2, false>(d, s, group, probs, nprob, K, N, act_dtype, st);

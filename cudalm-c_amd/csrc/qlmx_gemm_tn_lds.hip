@@ -1,0 +1,257 @@
+/* qlmx_gemm_tn_lds.hip -- input-gradient grouped GEMM (tn) for bf16 activations with the activation
+ * tiles loaded straight into LDS.
+ *
+ * dX_e[M,N] (= or +=) dY_e[M,K] . W_e[N,K]^T   (mg_abt_b, cudalm.cu:3204-3256; call sites 4340-4366)
+ * W_e[N,K] packed 4-bit, scale groups along K (the contraction), so the exact integer digits go to
+ * the matrix core and every 128-deep partial sum is folded in with its fp32 scale (see
+ * qlmx_gemm_mfma.hip for why).
+ *
+ * 128x128 output tile, 64-deep steps, four wavefronts 2x2 with 2x2 accumulators each (plus the
+ * per-group partial sums). Activations: each 16-byte piece goes from global memory into one of three
+ * LDS stages without touching a register (lane l of a wave instruction lands at base + 16*l; the
+ * rows keep their global order, 8 pieces = 128 bytes per row, piece ko of row r stored at position
+ * ko ^ ((r >> 1) & 7), which makes the MFMA operand reads conflict-free). Weights: 32 digits per
+ * thread and step through registers, converted to bf16 and written to one of two LDS buffers a step
+ * ahead. One barrier per step; the wait in front of it lets the activation tile requested last stay
+ * in flight. LDS accesses in the loop are inline assembly: the compiler would otherwise wait for
+ * every outstanding load-to-LDS before any LDS access.
+ */
+#include "qlmx_gemm.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float  f32x2  __attribute__((ext_vector_type(2)));
+typedef float  f32x16 __attribute__((ext_vector_type(16)));
+typedef int    i32x4  __attribute__((ext_vector_type(4)));
+
+#define TN3_BM 128
+#define TN3_BN 128
+#define TN3_BK 64
+#define TN3_A_BYTES (TN3_BM * TN3_BK * 2)     /* 16384 */
+#define TN3_B_BYTES (TN3_BN * TN3_BK * 2)     /* 16384 */
+#define TN3_A_STAGES 3
+#define TN3_B_OFF (TN3_A_STAGES * TN3_A_BYTES)
+
+struct Tn3Args { const DevProb *pr; int nprob, ntiles; const signed char *d; const float *s; int gshift; int K, N; };
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void glb_void;
+
+__device__ __forceinline__ uint32_t tn3_pk(float lo, float hi){
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+template<int OFF> __device__ __forceinline__ i32x4 tn3_rd(uint32_t addr){
+    i32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
+__device__ __forceinline__ void tn3_wr(uint32_t addr, i32x4 v){
+    asm volatile("ds_write_b128 %0, %1" :: "v"(addr), "v"(v) : "memory");
+}
+/* Register loads of the loop are inline assembly as well, and the step's wait names their
+ * destinations as in/out operands: the compiler then neither adds a wait of its own (it would be
+ * vmcnt(0) at the loop head, which also waits for the activation tile requested last) nor moves a
+ * use of the loaded values above the wait. */
+__device__ __forceinline__ i32x4 tn3_gld16(const void *p){
+    i32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ float tn3_gld4(const void *p){
+    float v;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+struct Tn3Ops { i32x4 a[2], b[2]; };
+__device__ __forceinline__ void tn3_wait(Tn3Ops &o){
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(o.a[0]), "+v"(o.a[1]), "+v"(o.b[0]), "+v"(o.b[1]));
+}
+
+__global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
+    __shared__ __attribute__((aligned(16))) unsigned char lds[TN3_A_STAGES * TN3_A_BYTES + 2 * TN3_B_BYTES];
+    const int t = qx_xcd_tile(blockIdx.x, gridDim.x);
+    if(t >= a.ntiles) return;
+    const DevProb P = a.pr[qx_find_problem(a.pr, a.nprob, t)];
+    const int lt = t - P.tile0;
+    const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
+    const int i0 = ti * TN3_BM, j0 = tj * TN3_BN;
+    const int rows = P.M;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;
+    const int fr = lane & 31, hf = lane >> 5;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
+
+    /* ---- activation pieces of this thread: position p = h*256 + tid of a stage is row p/8, stored
+     * piece p%8 = ko ^ ((row >> 1) & 7) ---- */
+    const char *srcA[4];
+#pragma unroll
+    for(int h = 0; h < 4; h++){
+        const int p = h * 256 + tid, r = p >> 3, ko = (p & 7) ^ ((r >> 1) & 7);
+        const int rr = (i0 + r < rows) ? i0 + r : rows - 1;               /* clamp: feeds unstored rows only */
+        srcA[h] = (const char *)P.A + ((size_t)rr * a.K + ko * 8) * 2;
+    }
+    const int wave_off = __builtin_amdgcn_readfirstlane(wave * 1024);
+    const int steps = a.K / TN3_BK;
+    auto issue_a = [&](int tile, int stage){
+        const int tl = tile < steps ? tile : steps - 1;                   /* past the end: the last tile again, into a stage nobody reads */
+        unsigned char *base = lds + stage * TN3_A_BYTES + wave_off;
+#pragma unroll
+        for(int h = 0; h < 4; h++)
+            __builtin_amdgcn_global_load_lds((glb_void *)(srcA[h] + (size_t)tl * (TN3_BK * 2)), (lds_void *)(base + h * 4096), 16, 0, 0);
+    };
+
+    /* ---- weights: thread = (row n, half of the step's 64 digits) ---- */
+    const int wn = tid & 127, whalf = tid >> 7;
+    const signed char *pw = a.d + ((P.wq + (size_t)(j0 + wn) * a.K) >> 1) + whalf * 16;
+    uint32_t wr_off[4];
+#pragma unroll
+    for(int j = 0; j < 4; j++){
+        const int ko = whalf * 4 + j;
+        wr_off[j] = TN3_B_OFF + (uint32_t)(ko * TN3_BN + (wn ^ ((ko << 1) & 15))) * 16;
+    }
+    auto load_w = [&](int tile) -> i32x4 {
+        const int tl = tile < steps ? tile : steps - 1;                   /* past the end: re-read the last one, never used */
+        return tn3_gld16(pw + (size_t)tl * (TN3_BK / 2));
+    };
+    auto store_w = [&](const i32x4 w, int buf){
+        const uint32_t wd[4] = {(uint32_t)w[0], (uint32_t)w[1], (uint32_t)w[2], (uint32_t)w[3]};
+        const uint32_t bb = lds_base + buf * TN3_B_BYTES;
+#pragma unroll
+        for(int j = 0; j < 4; j++){
+            i32x4 v;
+            v[0] = (int)tn3_pk((float)qx_nib(wd[j], 0), (float)qx_nib(wd[j], 1));
+            v[1] = (int)tn3_pk((float)qx_nib(wd[j], 2), (float)qx_nib(wd[j], 3));
+            v[2] = (int)tn3_pk((float)qx_nib(wd[j], 4), (float)qx_nib(wd[j], 5));
+            v[3] = (int)tn3_pk((float)qx_nib(wd[j], 6), (float)qx_nib(wd[j], 7));
+            tn3_wr(bb + wr_off[j], v);
+        }
+    };
+
+    /* ---- operand read offsets: [k16 slice]; the second tile of a pair is a constant further ---- */
+    uint32_t ra[4], rb[4];
+    {
+        const int r = wi + fr, f = (r >> 1) & 7;                          /* rows r and r+32 share f */
+        const int n = wj + fr;
+#pragma unroll
+        for(int ks = 0; ks < 4; ks++){
+            const int ko = ks * 2 + hf;
+            ra[ks] = (uint32_t)(r * 128 + ((ko ^ f) << 4));
+            rb[ks] = TN3_B_OFF + (uint32_t)(ko * TN3_BN + (n ^ ((ko << 1) & 15))) * 16;
+        }
+    }
+
+    /* ---- fp32 scale of (this lane's output column, scale group) ---- */
+    const int ngroups = a.K >> a.gshift, spg = (1 << a.gshift) / TN3_BK;
+    const float *pfold[2];
+#pragma unroll
+    for(int j = 0; j < 2; j++) pfold[j] = a.s + P.wg + (size_t)(j0 + wj + j * 32 + fr) * ngroups;
+    auto load_scale = [&](int step, int j) -> float {
+        int g = step / spg; g = g < ngroups ? g : ngroups - 1;
+        return tn3_gld4(pfold[j] + g);
+    };
+
+    f32x16 acc[2][2], part[2][2];
+#pragma unroll
+    for(int i = 0; i < 2; i++)
+#pragma unroll
+        for(int j = 0; j < 2; j++){ acc[i][j] = (f32x16)(0.0f); part[i][j] = (f32x16)(0.0f); }
+
+    /* ---- prologue. Issue order matters: each wait below lets the four activation requests issued
+     * last stay in flight and nothing else. A value loaded by inline assembly is never carried around
+     * the loop: it is requested after the barrier of a step and consumed, behind a wait that names it,
+     * at the end of the same step (the compiler may copy a loop-carried value before it has arrived). ---- */
+    float fs_cur[2];
+    {
+        i32x4 w0 = load_w(0);
+        float f0 = load_scale(0, 0), f1 = load_scale(0, 1);
+        issue_a(0, 0);
+        asm volatile("s_waitcnt vmcnt(4)" : "+v"(w0), "+v"(f0), "+v"(f1) :: "memory");
+        store_w(w0, 0);
+        fs_cur[0] = f0; fs_cur[1] = f1;
+        issue_a(1, 1);
+    }
+
+    for(int st = 0; st < steps; st++){
+        /* tile st is in, own LDS writes are done; tile st+1 may still be on its way */
+        asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        i32x4 wnext = load_w(st + 1);                      /* digits and scales of step st+1: used at the end of this step */
+        float fn0 = load_scale(st + 1, 0), fn1 = load_scale(st + 1, 1);
+        issue_a(st + 2, (st + 2) % TN3_A_STAGES);
+
+        const uint32_t sa = lds_base + (uint32_t)(st % TN3_A_STAGES) * TN3_A_BYTES;
+        const uint32_t sbuf = lds_base + (uint32_t)(st & 1) * TN3_B_BYTES;
+        Tn3Ops o[2];
+        o[0].a[0] = tn3_rd<0>(sa + ra[0]); o[0].a[1] = tn3_rd<32 * 128>(sa + ra[0]);
+        o[0].b[0] = tn3_rd<0>(sbuf + rb[0]); o[0].b[1] = tn3_rd<32 * 16>(sbuf + rb[0]);
+        tn3_wait(o[0]);
+#pragma unroll
+        for(int ks = 0; ks < 4; ks++){
+            Tn3Ops &cur = o[ks & 1], &nxt = o[(ks + 1) & 1];
+            if(ks < 3){
+                nxt.a[0] = tn3_rd<0>(sa + ra[ks + 1]); nxt.a[1] = tn3_rd<32 * 128>(sa + ra[ks + 1]);
+                nxt.b[0] = tn3_rd<0>(sbuf + rb[ks + 1]); nxt.b[1] = tn3_rd<32 * 16>(sbuf + rb[ks + 1]);
+            }
+#pragma unroll
+            for(int i = 0; i < 2; i++)
+#pragma unroll
+                for(int j = 0; j < 2; j++)
+                    part[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, cur.a[i]), __builtin_bit_cast(bf16x8, cur.b[j]), part[i][j], 0, 0, 0);
+            if(ks < 3) tn3_wait(nxt);
+        }
+        if((st + 1) % spg == 0){
+            /* one scale group of the contraction is complete: fold it in with its fp32 scale */
+#pragma unroll
+            for(int j = 0; j < 2; j++){
+#pragma unroll
+                for(int i = 0; i < 2; i++){
+#pragma unroll
+                    for(int e = 0; e < 16; e++) acc[i][j][e] = fmaf(fs_cur[j], part[i][j][e], acc[i][j][e]);
+                    part[i][j] = (f32x16)(0.0f);
+                }
+            }
+        }
+        /* digits and scales of step st+1 have arrived (only the four activation requests are younger);
+         * the buffer they go to was last read in step st-1 */
+        asm volatile("s_waitcnt vmcnt(4)" : "+v"(wnext), "+v"(fn0), "+v"(fn1) :: "memory");
+        store_w(wnext, (st + 1) & 1);
+        fs_cur[0] = fn0; fs_cur[1] = fn1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       /* no request may outlive the workgroup's LDS */
+
+    /* ---- epilogue: lane holds column fr of each 32x32 tile, rows (e/4)*8 + (lane/32)*4 + e%4 ---- */
+    const bool accumulate = P.beta != 0.0f;
+#pragma unroll
+    for(int i = 0; i < 2; i++)
+#pragma unroll
+        for(int j = 0; j < 2; j++){
+            const int rbase = i0 + wi + i * 32 + hf * 4;
+            float *col = P.C + (size_t)rbase * a.N + (j0 + wj + j * 32 + fr);
+            float old[16];
+#pragma unroll
+            for(int e = 0; e < 16; e++){
+                const int ro = (e >> 2) * 8 + (e & 3);
+                old[e] = (accumulate && rbase + ro < rows) ? col[(size_t)ro * a.N] : 0.0f;
+            }
+#pragma unroll
+            for(int e = 0; e < 16; e++){
+                const int ro = (e >> 2) * 8 + (e & 3);
+                if(rbase + ro < rows) col[(size_t)ro * a.N] = old[e] + acc[i][j][e];
+            }
+        }
+}
+
+/* bf16 activations only; N % 128 == 0, K % 64 == 0, group a power of two >= 64 (checked by the caller) */
+int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob,
+                            int K, int N, hipStream_t st){
+    ProbUpload up; int slot;
+    int rc = qlmx_upload_problems(probs, nprob, GEMM_TN, K, N, TN3_BM, TN3_BN, st, &up, &slot); if(rc) return rc;
+    if(up.ntiles == 0) return QLMX_OK;
+    Tn3Args a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.d = d; a.s = s; a.K = K; a.N = N;
+    a.gshift = 0; while((1 << a.gshift) < group) a.gshift++;
+    const int grid = (up.ntiles + 7) / 8 * 8;
+    hipLaunchKernelGGL(k_gemm_tn_lds, dim3(grid), dim3(256), 0, st, a);
+    QLMX_LAUNCH_CHECK("grouped gemm tn (direct-to-LDS) launch");
+    return qlmx_upload_done(slot, st);
+}

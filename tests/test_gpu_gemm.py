@@ -178,6 +178,14 @@ def test_attention_projection_spans_are_one_expert(q, orc, math):
             assert orc.relerr(got, want) < tol, (mode, K, N)
 
 
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_mfma_tn_many_rows_per_expert(q, orc, beta):
+    """Experts with well over a thousand rows on average take the input-gradient kernel whose
+    activation tiles go straight to LDS; a ragged tail expert and an empty one ride along."""
+    got, want = run_case(q, orc, "tn", 4, [2100, 1500, 0, 1311], 384, 256, pkg.ACT_BF16, pkg.MATH_MFMA, seed=4, beta=beta)
+    assert orc.relerr(got, want) < TOL_MFMA
+
+
 def test_mfma_rejects_unsupported_shapes(q):
     import torch
     x = torch.zeros(4096, device="cuda")

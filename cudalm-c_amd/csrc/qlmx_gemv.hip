@@ -47,8 +47,6 @@ struct GvArgs {
 };
 
 __device__ __forceinline__ float ub(uint32_t w, int k){ return (float)((w >> (8 * k)) & 0xFFu); }
-/* position of output column n inside a partial-sum row (natural order) */
-__device__ __forceinline__ int part_index(int n, int){ return n; }
 
 #define GV_MAXSPLIT 16
 /* sum of S <= GV_MAXSPLIT partial sums `stride` apart, added in slice order; all loads are issued
@@ -184,9 +182,8 @@ __global__ void __launch_bounds__(256) k_qlmx_gemv_finish(const GvProb *pr, cons
     const int p = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
     if(n >= N) return;
     const int M = pr[p].M; float *out = pr[p].out;
-    const int ix = part_index(n, N);
     for(int m = 0; m < M; m++){
-        const float *src = part + (((size_t)p * S) * MR + m) * N + ix;
+        const float *src = part + (((size_t)p * S) * MR + m) * N + n;
         out[(size_t)m * N + n] = sum_slices(src, (size_t)MR * N, S);
     }
 }

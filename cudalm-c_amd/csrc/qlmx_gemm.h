@@ -62,6 +62,98 @@ __device__ __forceinline__ int qx_xcd_tile_rows(int b, int g){
     return (x + 8 * (k / g)) * g + k % g;
 }
 
+typedef float qx_f32x16 __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(1))) float qx_gfloat;      /* known to be global memory: loads and stores complete in order */
+
+/* Writes the NI x NJ accumulator tiles (32x32 each, as v_mfma_f32_32x32x16 leaves them) of one
+ * wavefront: element e of a lane belongs to row (e/4)*8 + e%4 of the lane's four-row band and to the
+ * lane's column. `c` points at the lane's element of tile (0,0) -- row `row` of the output, which has
+ * `rows` valid rows and leading dimension ld; tile (i,j) lies 32*i rows and 32*j columns further.
+ * The two cases are separate code paths on purpose: the counter that a wait for loaded values uses
+ * also counts stores, so one path that may or may not load the old values waits, tile after tile, for
+ * all stores of the tile before -- measured, that made the epilogue of a 256x128 tile 45,000 cycles
+ * long. Without accumulation nothing waits; with it the old values of tile n+1 are requested before
+ * the stores of tile n, so the wait for them leaves those stores in flight. That needs exact counts
+ * and straight-line code: a wavefront whose tiles lie wholly inside the output stores without
+ * conditions, the others -- the last tile row of a problem -- take the slow path. */
+__device__ __forceinline__ float qx_gld_f32(const qx_gfloat *p){
+    float v;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+/* at most N younger memory operations may still be in flight; names the 16 values it guards */
+template<int N> __device__ __forceinline__ void qx_wait_old(float (&o)[16]){
+    asm volatile("s_waitcnt vmcnt(%16)"
+        : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(o[4]), "+v"(o[5]), "+v"(o[6]), "+v"(o[7]),
+          "+v"(o[8]), "+v"(o[9]), "+v"(o[10]), "+v"(o[11]), "+v"(o[12]), "+v"(o[13]), "+v"(o[14]), "+v"(o[15])
+        : "n"(N) : "memory");
+}
+
+/* edge path: per-row conditions, the compiler places the waits (every one of them a full drain) */
+template<int NI, int NJ>
+__device__ __forceinline__ void qx_store_tiles_edge(const qx_f32x16 (&acc)[NI][NJ], qx_gfloat *c, int row, int rows, size_t ld, bool accumulate){
+#pragma unroll
+    for(int i = 0; i < NI; i++)
+#pragma unroll
+        for(int j = 0; j < NJ; j++){
+            qx_gfloat *col = c + (size_t)(i * 32) * ld + j * 32;
+            float old[16];
+#pragma unroll
+            for(int e = 0; e < 16; e++){
+                const int ro = (e >> 2) * 8 + (e & 3);
+                old[e] = (accumulate && row + i * 32 + ro < rows) ? col[(size_t)ro * ld] : 0.0f;
+            }
+#pragma unroll
+            for(int e = 0; e < 16; e++){
+                const int ro = (e >> 2) * 8 + (e & 3);
+                if(row + i * 32 + ro < rows) col[(size_t)ro * ld] = old[e] + acc[i][j][e];
+            }
+        }
+}
+/* wavefront wholly inside the output: no conditions */
+template<int NI, int NJ>
+__device__ __forceinline__ void qx_store_tiles_full(const qx_f32x16 (&acc)[NI][NJ], qx_gfloat *c, size_t ld, bool accumulate){
+    if(!accumulate){
+#pragma unroll
+        for(int i = 0; i < NI; i++)
+#pragma unroll
+            for(int j = 0; j < NJ; j++){
+                qx_gfloat *col = c + (size_t)(i * 32) * ld + j * 32;
+#pragma unroll
+                for(int e = 0; e < 16; e++) col[(size_t)((e >> 2) * 8 + (e & 3)) * ld] = acc[i][j][e];
+            }
+        return;
+    }
+    /* Old values by inline assembly with explicit waits: request tile n+1, wait for tile n while the
+     * 16 requests of n+1 and the 16 stores of n-1 (both younger than the requests of n) stay in
+     * flight, store n. The compiler itself drains everything at each such point in these kernels. */
+    constexpr int NT = NI * NJ;
+    float old[2][16];
+    auto load_old = [&](int n, float (&o)[16]){
+        const qx_gfloat *col = c + (size_t)((n / NJ) * 32) * ld + (n % NJ) * 32;
+#pragma unroll
+        for(int e = 0; e < 16; e++) o[e] = qx_gld_f32(col + (size_t)((e >> 2) * 8 + (e & 3)) * ld);
+    };
+    load_old(0, old[0]);
+#pragma unroll
+    for(int n = 0; n < NT; n++){
+        if(n + 1 < NT) load_old(n + 1, old[(n + 1) & 1]);
+        if(n == 0) qx_wait_old<(NT > 1 ? 16 : 0)>(old[0]);
+        else if(n + 1 < NT) qx_wait_old<32>(old[n & 1]);
+        else qx_wait_old<16>(old[n & 1]);
+        qx_gfloat *col = c + (size_t)((n / NJ) * 32) * ld + (n % NJ) * 32;
+#pragma unroll
+        for(int e = 0; e < 16; e++) col[(size_t)((e >> 2) * 8 + (e & 3)) * ld] = old[n & 1][e] + acc[n / NJ][n % NJ][e];
+        __builtin_amdgcn_sched_barrier(0);                                /* the waits count on this order */
+    }
+}
+/* `row` is the lane's first row, `wave_row` the first row of the wavefront's tiles */
+template<int NI, int NJ>
+__device__ __forceinline__ void qx_store_tiles(const qx_f32x16 (&acc)[NI][NJ], float *c, int row, int wave_row, int rows, size_t ld, bool accumulate){
+    if(wave_row + NI * 32 <= rows) qx_store_tiles_full<NI, NJ>(acc, (qx_gfloat *)c, ld, accumulate);
+    else                           qx_store_tiles_edge<NI, NJ>(acc, (qx_gfloat *)c, row, rows, ld, accumulate);
+}
+
 __device__ __forceinline__ float qx_bf16_to_f32(unsigned short h){ return __uint_as_float((uint32_t)h << 16); }
 /* round to nearest even, as cudalm.cu:334-338 */
 __device__ __forceinline__ unsigned short qx_f32_to_bf16(float f){

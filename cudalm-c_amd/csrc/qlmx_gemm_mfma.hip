@@ -31,6 +31,7 @@
  */
 #include "qlmx_gemm.h"
 int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
+int qlmx_gemm_nn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
 int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -363,33 +364,9 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(MfmaArgs a){
         }
     }
 
-    /* ---- epilogue: lane holds column fr of each 32x32 tile, rows (v/4)*8 + (lane/32)*4 + v%4.
-     * When accumulating, the 16 old values of a tile are all requested before the first store: a
-     * load-add-store chain per element would cost one memory round trip each. ---- */
-    const bool accumulate = P.beta != 0.0f;
-#pragma unroll
-    for(int i = 0; i < WM; i++)
-#pragma unroll
-        for(int j = 0; j < 2; j++){
-            float *col = P.C + (size_t)(i0 + wi + i * 32 + hf * 4) * a.N + (j0 + wj + j * 32 + fr);
-            const int rbase = i0 + wi + i * 32 + hf * 4;
-            float old[16];
-            if(accumulate){
-#pragma unroll
-                for(int v = 0; v < 16; v++){
-                    const int ro = (v >> 2) * 8 + (v & 3);
-                    old[v] = (rbase + ro < rows) ? col[(size_t)ro * a.N] : 0.0f;
-                }
-            } else {
-#pragma unroll
-                for(int v = 0; v < 16; v++) old[v] = 0.0f;
-            }
-#pragma unroll
-            for(int v = 0; v < 16; v++){
-                const int ro = (v >> 2) * 8 + (v & 3);
-                if(rbase + ro < rows) col[(size_t)ro * a.N] = old[v] + acc[i][j][v];
-            }
-        }
+    /* ---- epilogue: the lane holds column lane%32 of each 32x32 tile, four-row band lane/32 ---- */
+    const int row = i0 + wi + hf * 4;
+    qx_store_tiles<WM, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
 }
 
 template<int MODE, int WM, bool DEEP>
@@ -437,6 +414,7 @@ int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int 
         if(live && rows / live >= 1024) return qlmx_gemm_tn_lds_launch(d, s, group, probs, nprob, K, N, st);
     }
     if(mode == GEMM_NT && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nt_lds_launch(probs, nprob, K, N, st);
+    if(mode == GEMM_NN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nn_lds_launch(d, s, group, probs, nprob, K, N, st);
     if(mode == GEMM_NN) return launch_mfma<GEMM_NN, 4, true>(d, s, group, probs, nprob, K, N, act_dtype, st);
     if(mode == GEMM_TN) return launch_mfma<GEMM_TN, 2, false>(d, s, group, probs, nprob, K, N, act_dtype, st);
     return launch_mfma<GEMM_NT, 4, false>(d, s, group, probs, nprob, K, N, act_dtype, st);

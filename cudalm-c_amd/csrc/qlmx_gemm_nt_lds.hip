@@ -106,19 +106,21 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
     const size_t stepA = (size_t)NT3_BK * a.K * 2, stepB = (size_t)NT3_BK * a.N * 2;
     const int wave_off = __builtin_amdgcn_readfirstlane(wave * 1024);
 
-    auto issue = [&](int tile, int stage){
+    /* request h of a tile: 0..3 are the X pieces, 4..5 the dY pieces */
+    auto issue_one = [&](int tile, int stage, int h){
         const int k0 = tile * NT3_BK;
         unsigned char *base = lds + stage * NT3_STAGE_BYTES + wave_off;
-#pragma unroll
-        for(int h = 0; h < 4; h++){
+        if(h < 4){
             const char *g = (k0 + rowA[h] < depth) ? srcA[h] + (size_t)tile * stepA : (const char *)a.zeros;
             __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(base + h * 4096), 16, 0, 0);
+        } else {
+            const char *g = (k0 + rowB[h - 4] < depth) ? srcB[h - 4] + (size_t)tile * stepB : (const char *)a.zeros;
+            __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(base + NT3_A_BYTES + (h - 4) * 4096), 16, 0, 0);
         }
+    };
+    auto issue = [&](int tile, int stage){
 #pragma unroll
-        for(int h = 0; h < 2; h++){
-            const char *g = (k0 + rowB[h] < depth) ? srcB[h] + (size_t)tile * stepB : (const char *)a.zeros;
-            __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(base + NT3_A_BYTES + h * 4096), 16, 0, 0);
-        }
+        for(int h = 0; h < 6; h++) issue_one(tile, stage, h);
     };
 
     /* ---- operand read addresses inside a stage (k16 slice 0; slice 1 is 16 rows further) ---- */
@@ -151,7 +153,6 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
         /* tile st has landed once at most the 6 requests of tile st+1 are still in flight */
         asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
         __builtin_amdgcn_s_barrier();                       /* everybody's pieces are in; stage (st+2)%3 is free again */
-        issue(st + 2, (st + 2) % NT3_STAGES);
         const uint32_t sb = lds_base + (uint32_t)(st % NT3_STAGES) * NT3_STAGE_BYTES;
         uint32_t adA[4], adB[2];
 #pragma unroll
@@ -162,42 +163,32 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
         nt3_read<0>(o0, adA, adB);
         nt3_wait_reads(o0);
         nt3_read<1>(o1, adA, adB);                          /* in flight while slice 0 multiplies */
+        /* The six requests of tile st+2 go out between the multiplications, one after every other
+         * MFMA: a request can wait a hundred cycles for the address unit when eight wavefronts ask at
+         * once, and behind an MFMA that wait costs nothing. The fences keep the compiler from
+         * gathering them again. */
+        const int nt = st + 2, ns = (st + 2) % NT3_STAGES;
 #pragma unroll
-        for(int i = 0; i < 4; i++)
+        for(int i = 0; i < 4; i++){
 #pragma unroll
             for(int j = 0; j < 2; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nt3_pack(o0.a[i][0], o0.a[i][1]), nt3_pack(o0.b[j][0], o0.b[j][1]), acc[i][j], 0, 0, 0);
+            if(i < 3){ __builtin_amdgcn_sched_barrier(0); issue_one(nt, ns, i); __builtin_amdgcn_sched_barrier(0); }
+        }
         nt3_wait_reads(o1);
 #pragma unroll
-        for(int i = 0; i < 4; i++)
+        for(int i = 0; i < 4; i++){
 #pragma unroll
             for(int j = 0; j < 2; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nt3_pack(o1.a[i][0], o1.a[i][1]), nt3_pack(o1.b[j][0], o1.b[j][1]), acc[i][j], 0, 0, 0);
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        /* no request may outlive the workgroup's LDS */
-
-    /* ---- epilogue: lane holds column fr of each 32x32 tile, rows (v/4)*8 + (lane/32)*4 + v%4; all old
-     * values of a tile are requested before the first store ---- */
-    const int fr = lane & 31, hf = lane >> 5;
-    const bool accumulate = P.beta != 0.0f;
-#pragma unroll
-    for(int i = 0; i < 4; i++)
-#pragma unroll
-        for(int j = 0; j < 2; j++){
-            const int rbase = i0 + wi + i * 32 + hf * 4;
-            float *col = P.C + (size_t)rbase * a.N + (j0 + wj + j * 32 + fr);
-            float old[16];
-#pragma unroll
-            for(int e = 0; e < 16; e++){
-                const int ro = (e >> 2) * 8 + (e & 3);
-                old[e] = (accumulate && rbase + ro < a.K) ? col[(size_t)ro * a.N] : 0.0f;
-            }
-#pragma unroll
-            for(int e = 0; e < 16; e++){
-                const int ro = (e >> 2) * 8 + (e & 3);
-                if(rbase + ro < a.K) col[(size_t)ro * a.N] = old[e] + acc[i][j][e];
-            }
+            if(i < 3){ __builtin_amdgcn_sched_barrier(0); issue_one(nt, ns, 3 + i); __builtin_amdgcn_sched_barrier(0); }
         }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);                    /* vmcnt(0), as a builtin so that the compiler knows it: no request may outlive the workgroup's LDS */
+
+    /* ---- epilogue: the lane holds column lane%32 of each 32x32 tile, four-row band lane/32 ---- */
+    const int fr = lane & 31, hf = lane >> 5, row = i0 + wi + hf * 4;
+    qx_store_tiles<4, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, a.K, (size_t)a.N, P.beta != 0.0f);
 }
 
 static void *g_nt3_zeros = nullptr;

@@ -218,28 +218,11 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
         store_w(wnext, (st + 1) & 1);
         fs_cur[0] = fn0; fs_cur[1] = fn1;
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       /* no request may outlive the workgroup's LDS */
+    __builtin_amdgcn_s_waitcnt(0x0F70);                    /* vmcnt(0), as a builtin so that the compiler knows it: no request may outlive the workgroup's LDS */
 
-    /* ---- epilogue: lane holds column fr of each 32x32 tile, rows (e/4)*8 + (lane/32)*4 + e%4 ---- */
-    const bool accumulate = P.beta != 0.0f;
-#pragma unroll
-    for(int i = 0; i < 2; i++)
-#pragma unroll
-        for(int j = 0; j < 2; j++){
-            const int rbase = i0 + wi + i * 32 + hf * 4;
-            float *col = P.C + (size_t)rbase * a.N + (j0 + wj + j * 32 + fr);
-            float old[16];
-#pragma unroll
-            for(int e = 0; e < 16; e++){
-                const int ro = (e >> 2) * 8 + (e & 3);
-                old[e] = (accumulate && rbase + ro < rows) ? col[(size_t)ro * a.N] : 0.0f;
-            }
-#pragma unroll
-            for(int e = 0; e < 16; e++){
-                const int ro = (e >> 2) * 8 + (e & 3);
-                if(rbase + ro < rows) col[(size_t)ro * a.N] = old[e] + acc[i][j][e];
-            }
-        }
+    /* ---- epilogue: the lane holds column lane%32 of each 32x32 tile, four-row band lane/32 ---- */
+    const int row = i0 + wi + hf * 4;
+    qx_store_tiles<2, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
 }
 
 /* bf16 activations only; N % 128 == 0, K % 64 == 0, group a power of two >= 64 (checked by the caller) */

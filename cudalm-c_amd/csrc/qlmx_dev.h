@@ -9,6 +9,7 @@
 
 /* ---- error plumbing (host) ---- */
 void qlmx_set_error(const char *fmt, ...);
+int qlmx_cu_count(void);
 int  qlmx_check_ready(void);
 #define QLMX_HIP(call, what)                                                                  \
     do { hipError_t e_ = (call);                                                              \

@@ -13,6 +13,8 @@ struct DevProb {
     int M; float beta;
     int tile0;              /* first tile of this problem in the flattened tile list */
     int tiles_n;            /* tiles along the output's second dimension             */
+    int chunk;              /* scheduled launches: rows per slice of the contraction */
+    int flag0;              /*   and the chain flag of the problem's first tile      */
 };
 
 /* Copies `nprob` problems into the next ring slot, fills tile0/tiles_n with the given tile shape
@@ -24,14 +26,20 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
                          int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot);
 int qlmx_upload_done(int slot, hipStream_t stream);
 
-/* locate the problem owning flattened tile t (tile0 ascending) */
+/* Locate the problem owning flattened tile t: the last one whose tile0 <= t (tile0 ascending, empty
+ * problems share the tile0 of their successor). Every lane reads the tile0 of one problem and the
+ * wavefront counts the hits, so the lookup costs one memory round trip per 64 problems; a binary
+ * search costs one per level, and at 24 contraction steps per tile those five or six dependent
+ * round trips were a fifth of a workgroup's life. Call with all lanes active and t uniform. */
 __device__ __forceinline__ int qx_find_problem(const DevProb *pr, int nprob, int t){
-    int lo = 0, hi = nprob - 1;
-    while(lo < hi){
-        int mid = (lo + hi + 1) >> 1;
-        if(pr[mid].tile0 <= t) lo = mid; else hi = mid - 1;
+    const int lane = threadIdx.x & 63;
+    int count = 0;
+    for(int base = 0; base < nprob; base += 64){
+        const int p = base + lane;
+        const int t0 = p < nprob ? pr[p].tile0 : 0x7FFFFFFF;
+        count += __popcll(__ballot(t0 <= t));
     }
-    return lo;
+    return __builtin_amdgcn_readfirstlane(count - 1);
 }
 
 /* Tile handled by workgroup b when workgroups go round-robin to 8 XCDs and the grid has been
@@ -76,10 +84,17 @@ typedef __attribute__((address_space(1))) float qx_gfloat;      /* known to be g
  * the stores of tile n, so the wait for them leaves those stores in flight. That needs exact counts
  * and straight-line code: a wavefront whose tiles lie wholly inside the output stores without
  * conditions, the others -- the last tile row of a problem -- take the slow path. */
-__device__ __forceinline__ float qx_gld_f32(const qx_gfloat *p){
+/* SYS: the access goes past both cache levels (system scope), for tiles that several workgroups
+ * on different XCDs -- each with an L2 of its own -- add to in turn */
+template<bool SYS> __device__ __forceinline__ float qx_gld_f32(const qx_gfloat *p){
     float v;
-    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    if(SYS) asm volatile("global_load_dword %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+    else    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
     return v;
+}
+template<bool SYS> __device__ __forceinline__ void qx_gst_f32(qx_gfloat *p, float v){
+    if(SYS) asm volatile("global_store_dword %0, %1, off sc0 sc1" :: "v"(p), "v"(v) : "memory");
+    else    *p = v;
 }
 /* at most N younger memory operations may still be in flight; names the 16 values it guards */
 template<int N> __device__ __forceinline__ void qx_wait_old(float (&o)[16]){
@@ -90,7 +105,7 @@ template<int N> __device__ __forceinline__ void qx_wait_old(float (&o)[16]){
 }
 
 /* edge path: per-row conditions, the compiler places the waits (every one of them a full drain) */
-template<int NI, int NJ>
+template<int NI, int NJ, bool SYS>
 __device__ __forceinline__ void qx_store_tiles_edge(const qx_f32x16 (&acc)[NI][NJ], qx_gfloat *c, int row, int rows, size_t ld, bool accumulate){
 #pragma unroll
     for(int i = 0; i < NI; i++)
@@ -101,17 +116,22 @@ __device__ __forceinline__ void qx_store_tiles_edge(const qx_f32x16 (&acc)[NI][N
 #pragma unroll
             for(int e = 0; e < 16; e++){
                 const int ro = (e >> 2) * 8 + (e & 3);
-                old[e] = (accumulate && row + i * 32 + ro < rows) ? col[(size_t)ro * ld] : 0.0f;
+                old[e] = 0.0f;
+                if(accumulate && row + i * 32 + ro < rows)
+                    old[e] = SYS ? __hip_atomic_load((float *)(col + (size_t)ro * ld), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) : col[(size_t)ro * ld];
             }
 #pragma unroll
             for(int e = 0; e < 16; e++){
                 const int ro = (e >> 2) * 8 + (e & 3);
-                if(row + i * 32 + ro < rows) col[(size_t)ro * ld] = old[e] + acc[i][j][e];
+                if(row + i * 32 + ro < rows){
+                    if(SYS) __hip_atomic_store((float *)(col + (size_t)ro * ld), old[e] + acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    else    col[(size_t)ro * ld] = old[e] + acc[i][j][e];
+                }
             }
         }
 }
 /* wavefront wholly inside the output: no conditions */
-template<int NI, int NJ>
+template<int NI, int NJ, bool SYS>
 __device__ __forceinline__ void qx_store_tiles_full(const qx_f32x16 (&acc)[NI][NJ], qx_gfloat *c, size_t ld, bool accumulate){
     if(!accumulate){
 #pragma unroll
@@ -120,7 +140,7 @@ __device__ __forceinline__ void qx_store_tiles_full(const qx_f32x16 (&acc)[NI][N
             for(int j = 0; j < NJ; j++){
                 qx_gfloat *col = c + (size_t)(i * 32) * ld + j * 32;
 #pragma unroll
-                for(int e = 0; e < 16; e++) col[(size_t)((e >> 2) * 8 + (e & 3)) * ld] = acc[i][j][e];
+                for(int e = 0; e < 16; e++) qx_gst_f32<SYS>(col + (size_t)((e >> 2) * 8 + (e & 3)) * ld, acc[i][j][e]);
             }
         return;
     }
@@ -132,7 +152,7 @@ __device__ __forceinline__ void qx_store_tiles_full(const qx_f32x16 (&acc)[NI][N
     auto load_old = [&](int n, float (&o)[16]){
         const qx_gfloat *col = c + (size_t)((n / NJ) * 32) * ld + (n % NJ) * 32;
 #pragma unroll
-        for(int e = 0; e < 16; e++) o[e] = qx_gld_f32(col + (size_t)((e >> 2) * 8 + (e & 3)) * ld);
+        for(int e = 0; e < 16; e++) o[e] = qx_gld_f32<SYS>(col + (size_t)((e >> 2) * 8 + (e & 3)) * ld);
     };
     load_old(0, old[0]);
 #pragma unroll
@@ -143,15 +163,49 @@ __device__ __forceinline__ void qx_store_tiles_full(const qx_f32x16 (&acc)[NI][N
         else qx_wait_old<16>(old[n & 1]);
         qx_gfloat *col = c + (size_t)((n / NJ) * 32) * ld + (n % NJ) * 32;
 #pragma unroll
-        for(int e = 0; e < 16; e++) col[(size_t)((e >> 2) * 8 + (e & 3)) * ld] = old[n & 1][e] + acc[n / NJ][n % NJ][e];
+        for(int e = 0; e < 16; e++) qx_gst_f32<SYS>(col + (size_t)((e >> 2) * 8 + (e & 3)) * ld, old[n & 1][e] + acc[n / NJ][n % NJ][e]);
         __builtin_amdgcn_sched_barrier(0);                                /* the waits count on this order */
     }
 }
 /* `row` is the lane's first row, `wave_row` the first row of the wavefront's tiles */
-template<int NI, int NJ>
+template<int NI, int NJ, bool SYS = false>
 __device__ __forceinline__ void qx_store_tiles(const qx_f32x16 (&acc)[NI][NJ], float *c, int row, int wave_row, int rows, size_t ld, bool accumulate){
-    if(wave_row + NI * 32 <= rows) qx_store_tiles_full<NI, NJ>(acc, (qx_gfloat *)c, ld, accumulate);
-    else                           qx_store_tiles_edge<NI, NJ>(acc, (qx_gfloat *)c, row, rows, ld, accumulate);
+    if(wave_row + NI * 32 <= rows) qx_store_tiles_full<NI, NJ, SYS>(acc, (qx_gfloat *)c, ld, accumulate);
+    else                           qx_store_tiles_edge<NI, NJ, SYS>(acc, (qx_gfloat *)c, row, rows, ld, accumulate);
+}
+
+/* ---- scheduled launches: instead of deriving its tile from its index, workgroup b reads unit b of a
+ * table the host has laid out -- which problem, which output tile, which slice of the contraction
+ * (a table of up to 16 KB together with the problems travels about 12 us faster than a larger one,
+ * hence the packing). Slices of one output tile form a chain: slice seq waits until flag holds
+ * (epoch << 4 | seq), adds its product to what is there and publishes seq + 1. A slice always sits at
+ * a higher workgroup index than its predecessor, and workgroups start in index order, so whatever a
+ * resident workgroup waits for is resident or done; the wait is bounded all the same. ---- */
+typedef uint32_t DevUnit;                 /* prob:10 | tile row:6 | tile column:8 | seq:4 | nseq:4; all ones = nothing to do */
+#define QX_UNIT_NONE 0xFFFFFFFFu
+#define QX_UNIT(prob, ti, tj, seq, nseq) ((uint32_t)(prob) << 22 | (uint32_t)(ti) << 16 | (uint32_t)(tj) << 8 | (uint32_t)(seq) << 4 | (uint32_t)(nseq))
+#define QLMX_MAX_UNITS 16384
+#define QX_CHAIN_SPINS (1 << 22)
+struct UnitUpload { DevProb *hprob; DevUnit *hunit; const DevProb *dprob; const DevUnit *dunit; int *flags; unsigned *status; };
+int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot);                         /* host tables to fill; waits for the slot's last user */
+int qlmx_unit_commit(int slot, int nprob, int nunits, hipStream_t stream);         /* copies them to the device, asynchronously */
+int qlmx_unit_done(int slot, hipStream_t stream);                                  /* after the kernel launch */
+int qlmx_chain_reserve(int nflags, int *first, unsigned *epoch);                   /* flags for one launch */
+
+/* chain hand-over; every thread of the workgroup calls both */
+__device__ __forceinline__ void qx_chain_wait(int *flags, int flag, unsigned epoch, int seq, unsigned *status){
+    if(threadIdx.x == 0){
+        const int want = (int)((epoch << 4) | (unsigned)seq);
+        int spins = 0;
+        while(__hip_atomic_load(flags + flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want && ++spins < QX_CHAIN_SPINS) __builtin_amdgcn_s_sleep(16);
+        if(spins >= QX_CHAIN_SPINS) __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    __syncthreads();
+}
+__device__ __forceinline__ void qx_chain_publish(int *flags, int flag, unsigned epoch, int seq){
+    __builtin_amdgcn_s_waitcnt(0x0F70);                 /* vmcnt(0): this wavefront's system-scope stores are out */
+    __syncthreads();
+    if(threadIdx.x == 0) __hip_atomic_store(flags + flag, (int)((epoch << 4) | (unsigned)(seq + 1)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ float qx_bf16_to_f32(unsigned short h){ return __uint_as_float((uint32_t)h << 16); }

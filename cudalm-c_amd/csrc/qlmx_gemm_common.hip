@@ -63,7 +63,7 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
         DevProb &q = h[n++];
         q.A = p.A; q.B = p.B; q.C = p.C; q.wq = p.wq; q.wg = p.wg; q.M = p.M;
         q.beta = mode == GEMM_NN ? 0.0f : p.beta;
-        q.tile0 = (int)tiles; q.tiles_n = tiles_n;
+        q.tile0 = (int)tiles; q.tiles_n = tiles_n; q.chunk = 0; q.flag0 = 0;
         tiles += (long long)((rows + tile_rows - 1) / tile_rows) * tiles_n;
         QLMX_REQUIRE(tiles < (1LL << 30), "grouped gemm: too many tiles");
     }
@@ -76,5 +76,76 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
 int qlmx_upload_done(int slot, hipStream_t stream){
     QLMX_HIP(hipEventRecord(g_ring_ev[slot], stream), "problem ring record");
     g_ring_used[slot] = true;
+    return QLMX_OK;
+}
+
+/* ---- unit tables of scheduled launches: a ring of pinned/device slot pairs like the one above, each
+ * holding a problem table and a unit table; chain flags handed out round the ring of a fixed array
+ * (a launch's flags carry its epoch, so nothing is ever cleared). ---- */
+#define UNIT_SLOTS 32
+#define CHAIN_FLAGS (1 << 18)
+static char      *g_unit_h = nullptr, *g_unit_d = nullptr;
+static hipEvent_t g_unit_ev[UNIT_SLOTS];
+static bool       g_unit_used[UNIT_SLOTS];
+static int        g_unit_next = 0;
+static int       *g_chain_flags = nullptr;
+static unsigned  *g_chain_status = nullptr;      /* pinned: a kernel whose wait ran out sets it */
+static int        g_chain_cursor = 0;
+static unsigned   g_chain_epoch = 0;
+static const size_t UNIT_SLOT_BYTES = (size_t)QLMX_MAX_PROBLEMS * sizeof(DevProb) + (size_t)QLMX_MAX_UNITS * sizeof(DevUnit);
+
+/* the unit table follows the problem table, so that one copy moves both */
+static size_t unit_offset(int nprob){ return ((size_t)nprob * sizeof(DevProb) + 63) & ~(size_t)63; }
+
+static int unit_init(void){
+    if(g_unit_h) return QLMX_OK;
+    QLMX_HIP(hipHostMalloc((void **)&g_unit_h, UNIT_SLOTS * UNIT_SLOT_BYTES, hipHostMallocDefault), "unit ring (pinned)");
+    QLMX_HIP(hipMalloc((void **)&g_unit_d, UNIT_SLOTS * UNIT_SLOT_BYTES), "unit ring (device)");
+    QLMX_HIP(hipMalloc((void **)&g_chain_flags, CHAIN_FLAGS * sizeof(int)), "chain flags");
+    QLMX_HIP(hipMemset(g_chain_flags, 0, CHAIN_FLAGS * sizeof(int)), "chain flags clear");
+    QLMX_HIP(hipHostMalloc((void **)&g_chain_status, sizeof(unsigned), hipHostMallocDefault), "chain status (pinned)");
+    *g_chain_status = 0;
+    for(int i = 0; i < UNIT_SLOTS; i++){
+        QLMX_HIP(hipEventCreateWithFlags(&g_unit_ev[i], hipEventDisableTiming), "unit ring event");
+        g_unit_used[i] = false;
+    }
+    return QLMX_OK;
+}
+
+int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot_out){
+    int rc = unit_init(); if(rc) return rc;
+    if(*(volatile unsigned *)g_chain_status){
+        qlmx_set_error("grouped gemm: an earlier launch gave up waiting for a partial sum of a split contraction; its output is incomplete");
+        return QLMX_E_HIP;
+    }
+    const int slot = g_unit_next; g_unit_next = (g_unit_next + 1) % UNIT_SLOTS;
+    if(g_unit_used[slot]) QLMX_HIP(hipEventSynchronize(g_unit_ev[slot]), "unit ring wait");
+    char *h = g_unit_h + slot * UNIT_SLOT_BYTES, *d = g_unit_d + slot * UNIT_SLOT_BYTES;
+    const size_t uoff = unit_offset(nprob);
+    out->hprob = (DevProb *)h; out->hunit = (DevUnit *)(h + uoff);
+    out->dprob = (const DevProb *)d; out->dunit = (const DevUnit *)(d + uoff);
+    out->flags = g_chain_flags; out->status = g_chain_status;
+    *slot_out = slot;
+    return QLMX_OK;
+}
+
+int qlmx_unit_commit(int slot, int nprob, int nunits, hipStream_t stream){
+    char *h = g_unit_h + slot * UNIT_SLOT_BYTES, *d = g_unit_d + slot * UNIT_SLOT_BYTES;
+    QLMX_HIP(hipMemcpyAsync(d, h, unit_offset(nprob) + (size_t)nunits * sizeof(DevUnit), hipMemcpyHostToDevice, stream), "problem and unit tables h2d");
+    return QLMX_OK;
+}
+
+int qlmx_unit_done(int slot, hipStream_t stream){
+    QLMX_HIP(hipEventRecord(g_unit_ev[slot], stream), "unit ring record");
+    g_unit_used[slot] = true;
+    return QLMX_OK;
+}
+
+int qlmx_chain_reserve(int nflags, int *first, unsigned *epoch){
+    QLMX_REQUIRE(nflags <= CHAIN_FLAGS / 4, "grouped gemm: %d chained tiles in one launch", nflags);
+    if(g_chain_cursor + nflags > CHAIN_FLAGS) g_chain_cursor = 0;
+    *first = g_chain_cursor; g_chain_cursor += nflags;
+    g_chain_epoch = (g_chain_epoch + 1) & 0x0FFFFFFFu;
+    *epoch = g_chain_epoch;
     return QLMX_OK;
 }

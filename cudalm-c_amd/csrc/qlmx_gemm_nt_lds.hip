@@ -20,6 +20,7 @@
  * Rows past the end of an expert are fetched from a zero block instead of being masked.
  */
 #include "qlmx_gemm.h"
+#include <algorithm>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short  s16x4  __attribute__((ext_vector_type(4)));
@@ -34,7 +35,8 @@ typedef float  f32x16 __attribute__((ext_vector_type(16)));
 #define NT3_B_BYTES (NT3_BK * NT3_BN * 2)      /*  8192 */
 #define NT3_STAGE_BYTES (NT3_A_BYTES + NT3_B_BYTES)
 
-struct Nt3Args { const DevProb *pr; int nprob, ntiles, tiles_n, rows_p; int K, N; const void *zeros; };
+struct Nt3Args { const DevProb *pr; const DevUnit *units; int *flags; unsigned *status; unsigned epoch;
+                 int nprob, ntiles, tiles_n, rows_p; int K, N; const void *zeros; };
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void glb_void;
@@ -75,15 +77,36 @@ __device__ __forceinline__ bf16x8 nt3_pack(const i32x2 lo, const i32x2 hi){
     return __builtin_bit_cast(bf16x8, v);
 }
 
+__device__ __forceinline__ int t_of(int b, const Nt3Args &a){
+    return (a.rows_p & 7) ? qx_xcd_tile_probs(b, a.tiles_n, a.rows_p) : qx_xcd_tile_rows(b, a.tiles_n);
+}
+
 __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
     __shared__ __attribute__((aligned(16))) unsigned char lds[NT3_STAGES * NT3_STAGE_BYTES];
-    const int t = (a.rows_p & 7) ? qx_xcd_tile_probs(blockIdx.x, a.tiles_n, a.rows_p) : qx_xcd_tile_rows(blockIdx.x, a.tiles_n);
-    if(t >= a.ntiles) return;
-    const DevProb P = a.pr[qx_find_problem(a.pr, a.nprob, t)];
-    const int lt = t - P.tile0;
-    const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
-    const int i0 = ti * NT3_BM, j0 = tj * NT3_BN;
-    const int depth = P.M;
+    /* scheduled launch: the unit table says what to do; otherwise the tile follows from the index */
+    int pi, i0, j0, k0 = 0, depth = -1, seq = 0, nseq = 1, flag = 0;
+    DevUnit u = QX_UNIT_NONE;
+    if(a.units){
+        u = a.units[blockIdx.x];
+        if(u == QX_UNIT_NONE) return;
+        pi = (int)(u >> 22);
+    } else {
+        const int t = t_of(blockIdx.x, a);
+        if(t >= a.ntiles) return;
+        pi = qx_find_problem(a.pr, a.nprob, t);
+    }
+    const DevProb P = a.pr[pi];
+    if(a.units){
+        const int ti = (u >> 16) & 63, tj = (u >> 8) & 255;
+        seq = (u >> 4) & 15; nseq = u & 15;
+        i0 = ti * NT3_BM; j0 = tj * NT3_BN; k0 = seq * P.chunk;
+        depth = P.M - k0 < P.chunk ? P.M - k0 : P.chunk;
+        flag = P.flag0 + ti * P.tiles_n + tj;
+    } else {
+        const int lt = t_of(blockIdx.x, a) - P.tile0;
+        const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
+        i0 = ti * NT3_BM; j0 = tj * NT3_BN; depth = P.M;
+    }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wi = (wave >> 1) * 128, wj = (wave & 1) * 64;
 
@@ -95,26 +118,26 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
         const int p = h * 256 + tid, row = p >> 5, lu = (p & 31) ^ ((row & 3) << 2);
         const int col = i0 + lu * 8;
         rowA[h] = row;
-        srcA[h] = (const char *)P.A + ((size_t)row * a.K + (col < a.K ? col : 0)) * 2;   /* columns past K feed rows that are never stored */
+        srcA[h] = (const char *)P.A + ((size_t)(k0 + row) * a.K + (col < a.K ? col : 0)) * 2;   /* columns past K feed rows that are never stored */
     }
 #pragma unroll
     for(int h = 0; h < 2; h++){
         const int p = h * 256 + tid, row = p >> 4, lu = (p & 15) ^ ((row & 3) << 2);
         rowB[h] = row;
-        srcB[h] = (const char *)P.B + ((size_t)row * a.N + j0 + lu * 8) * 2;
+        srcB[h] = (const char *)P.B + ((size_t)(k0 + row) * a.N + j0 + lu * 8) * 2;
     }
     const size_t stepA = (size_t)NT3_BK * a.K * 2, stepB = (size_t)NT3_BK * a.N * 2;
     const int wave_off = __builtin_amdgcn_readfirstlane(wave * 1024);
 
     /* request h of a tile: 0..3 are the X pieces, 4..5 the dY pieces */
     auto issue_one = [&](int tile, int stage, int h){
-        const int k0 = tile * NT3_BK;
+        const int kt = tile * NT3_BK;
         unsigned char *base = lds + stage * NT3_STAGE_BYTES + wave_off;
         if(h < 4){
-            const char *g = (k0 + rowA[h] < depth) ? srcA[h] + (size_t)tile * stepA : (const char *)a.zeros;
+            const char *g = (kt + rowA[h] < depth) ? srcA[h] + (size_t)tile * stepA : (const char *)a.zeros;
             __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(base + h * 4096), 16, 0, 0);
         } else {
-            const char *g = (k0 + rowB[h - 4] < depth) ? srcB[h - 4] + (size_t)tile * stepB : (const char *)a.zeros;
+            const char *g = (kt + rowB[h - 4] < depth) ? srcB[h - 4] + (size_t)tile * stepB : (const char *)a.zeros;
             __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(base + NT3_A_BYTES + (h - 4) * 4096), 16, 0, 0);
         }
     };
@@ -188,10 +211,74 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
 
     /* ---- epilogue: the lane holds column lane%32 of each 32x32 tile, four-row band lane/32 ---- */
     const int fr = lane & 31, hf = lane >> 5, row = i0 + wi + hf * 4;
-    qx_store_tiles<4, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, a.K, (size_t)a.N, P.beta != 0.0f);
+    float *c = P.C + (size_t)row * a.N + (j0 + wj + fr);
+    if(nseq == 1){
+        qx_store_tiles<4, 2>(acc, c, row, i0 + wi, a.K, (size_t)a.N, P.beta != 0.0f);
+        return;
+    }
+    /* one slice of a split contraction: add to what the slices before have left, past the caches */
+    if(seq > 0) qx_chain_wait(a.flags, flag, a.epoch, seq, a.status);
+    qx_store_tiles<4, 2, true>(acc, c, row, i0 + wi, a.K, (size_t)a.N, seq > 0 || P.beta != 0.0f);
+    if(seq + 1 < nseq) qx_chain_publish(a.flags, flag, a.epoch, seq);
 }
 
 static void *g_nt3_zeros = nullptr;
+
+/* Lays out a scheduled launch. Every live problem owns T = tile rows x tile columns output tiles whose
+ * cost is its row count, so a Zipf-loaded layer has a few tiles that outlast all others: contractions
+ * longer than about the mean load of a workgroup slot are cut into slices that add up through a
+ * chain. Groups (problem, tile row) -- the tiles that share the activation slab -- are dealt to the
+ * XCDs heaviest first, each to the XCD with the least work so far; workgroup 8k + x is the k-th unit
+ * of XCD x. Returns the grid size, or 0 when the launch does not fit the table. */
+struct Nt3Group { int prob, ti, cost; };
+static int nt3_schedule(DevProb *pr, int n, int K, int N, int cus, DevUnit *units, int *nflags_out){
+    const int g = N / NT3_BN, rp = (K + NT3_BM - 1) / NT3_BM;
+    if(g > 256 || rp > 64) return 0;                                   /* the packed unit has 8 and 6 bits for them */
+    long long work = 0;
+    for(int p = 0; p < n; p++) work += (long long)pr[p].M * rp * g;
+    const long long slots = 2LL * cus;
+    long long mean = (work + slots - 1) / slots;                       /* rows of contraction per workgroup slot */
+    if(mean < 256) mean = 256;
+    static int nchunk[QLMX_MAX_PROBLEMS], chunk[QLMX_MAX_PROBLEMS];
+    long long nunits = 0;
+    for(int p = 0; p < n; p++){
+        int nc = 1;
+        if(pr[p].M > mean + mean / 4){ nc = (int)((pr[p].M + mean - 1) / mean); if(nc > 15) nc = 15; }
+        nchunk[p] = nc;
+        chunk[p] = ((pr[p].M + nc - 1) / nc + NT3_BK - 1) / NT3_BK * NT3_BK;
+        nunits += (long long)nc * rp * g;
+    }
+    if(nunits + 8LL * (long long)(rp * g * 15) > QLMX_MAX_UNITS) return 0;
+    static Nt3Group groups[QLMX_MAX_UNITS];
+    int ng = 0;
+    for(int p = 0; p < n; p++) for(int ti = 0; ti < rp; ti++) groups[ng++] = {p, ti, pr[p].M};
+    std::stable_sort(groups, groups + ng, [](const Nt3Group &x, const Nt3Group &y){ return x.cost > y.cost; });
+    static int gx[QLMX_MAX_UNITS];
+    long long load[8] = {0, 0, 0, 0, 0, 0, 0, 0}; int len[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for(int i = 0; i < ng; i++){
+        int x = 0;
+        for(int y = 1; y < 8; y++) if(load[y] < load[x]) x = y;
+        gx[i] = x; load[x] += (long long)groups[i].cost * g; len[x] += nchunk[groups[i].prob] * g;
+    }
+    int longest = 0;
+    for(int x = 0; x < 8; x++) if(len[x] > longest) longest = len[x];
+    const int grid = 8 * longest;
+    if(grid > QLMX_MAX_UNITS) return 0;
+    for(int b = 0; b < grid; b++) units[b] = QX_UNIT_NONE;
+    int nflags = 0;
+    for(int p = 0; p < n; p++){
+        pr[p].chunk = chunk[p]; pr[p].flag0 = nflags;
+        if(nchunk[p] > 1) nflags += rp * g;
+    }
+    int pos[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for(int i = 0; i < ng; i++){
+        const int p = groups[i].prob, x = gx[i], nc = nchunk[p];
+        for(int tj = 0; tj < g; tj++)
+            for(int c = 0; c < nc; c++) units[8 * pos[x]++ + x] = QX_UNIT(p, groups[i].ti, tj, c, nc);
+    }
+    *nflags_out = nflags;
+    return grid;
+}
 
 /* bf16 operands only; N % 128 == 0, K % 8 == 0, operands 16-byte aligned (checked by the caller) */
 int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st){
@@ -199,10 +286,43 @@ int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N
         QLMX_HIP(hipMalloc(&g_nt3_zeros, 256), "nt zero block");
         QLMX_HIP(hipMemset(g_nt3_zeros, 0, 256), "nt zero block clear");
     }
+    /* scheduled launch when the unit table holds it; the index-mapped one otherwise */
+    {
+        int live = 0;
+        for(int i = 0; i < nprob; i++) if(probs[i].M > 0) live++;
+        if(live == 0) return QLMX_OK;
+        if(nprob <= QLMX_MAX_PROBLEMS){
+            UnitUpload uu; int uslot;
+            int rc = qlmx_unit_slot(live, &uu, &uslot); if(rc) return rc;
+            int n = 0;
+            for(int i = 0; i < nprob; i++){
+                const qlmx_gemm_prob &p = probs[i];
+                QLMX_REQUIRE(p.M >= 0, "grouped gemm: problem %d has M=%d", i, p.M);
+                if(p.M == 0) continue;
+                QLMX_REQUIRE(p.A && p.B && p.C, "grouped gemm nt: problem %d has a NULL operand", i);
+                QLMX_REQUIRE(p.beta == 0.0f || p.beta == 1.0f, "grouped gemm: beta must be 0 or 1");
+                DevProb &q = uu.hprob[n++];
+                q.A = p.A; q.B = p.B; q.C = p.C; q.wq = 0; q.wg = 0; q.M = p.M; q.beta = p.beta; q.tile0 = 0; q.tiles_n = N / NT3_BN;
+            }
+            int nflags = 0;
+            const int grid = nt3_schedule(uu.hprob, n, K, N, qlmx_cu_count(), uu.hunit, &nflags);
+            if(grid > 0){
+                Nt3Args a; a.pr = uu.dprob; a.units = uu.dunit; a.flags = uu.flags; a.status = uu.status;
+                a.nprob = n; a.ntiles = grid; a.tiles_n = N / NT3_BN; a.rows_p = 1; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
+                int first = 0; a.epoch = 0;
+                if(nflags){ rc = qlmx_chain_reserve(nflags, &first, &a.epoch); if(rc) return rc; }
+                for(int p = 0; p < n; p++) uu.hprob[p].flag0 += first;
+                rc = qlmx_unit_commit(uslot, n, grid, st); if(rc) return rc;
+                hipLaunchKernelGGL(k_gemm_nt_lds, dim3(grid), dim3(256), 0, st, a);
+                QLMX_LAUNCH_CHECK("grouped gemm nt (scheduled) launch");
+                return qlmx_unit_done(uslot, st);
+            }
+        }
+    }
     ProbUpload up; int slot;
     int rc = qlmx_upload_problems(probs, nprob, GEMM_NT, K, N, NT3_BM, NT3_BN, st, &up, &slot); if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;
-    Nt3Args a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.tiles_n = N / NT3_BN; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
+    Nt3Args a; a.units = nullptr; a.flags = nullptr; a.status = nullptr; a.epoch = 0; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.tiles_n = N / NT3_BN; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
     a.rows_p = up.ntiles / (a.tiles_n * up.nprob);
     int grid;
     if(a.rows_p & 7) grid = 8 * a.tiles_n * a.rows_p * ((up.nprob + 7) / 8);

@@ -22,6 +22,9 @@ int qlmx_check_ready(void){
     return QLMX_E_NODEV;
 }
 
+static int g_cus = 256;
+int qlmx_cu_count(void){ return g_cus; }                   /* compute units of the initialised device */
+
 extern "C" int qlmx_version(void){ return QLMX_VERSION; }
 extern "C" const char *qlmx_last_error(void){ return g_err; }
 extern "C" const char *qlmx_device_name(void){ return g_devname; }
@@ -38,6 +41,7 @@ extern "C" int qlmx_init(int device){
     hipDeviceProp_t pr;
     QLMX_HIP(hipGetDeviceProperties(&pr, device), "hipGetDeviceProperties");
     snprintf(g_devname, sizeof g_devname, "%s (%s, %d CUs)", pr.name, pr.gcnArchName, pr.multiProcessorCount);
+    g_cus = pr.multiProcessorCount;
     if(strncmp(pr.gcnArchName, "gfx950", 6) != 0){
         qlmx_set_error("qlmx_init: device is %s; this library carries gfx950 code only", pr.gcnArchName);
         return QLMX_E_NODEV;

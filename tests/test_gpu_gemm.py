@@ -49,7 +49,7 @@ def zipf_rows(total, E, seed):
     return [int(c) for c in cnt]
 
 
-def run_case(q, orc, mode, E, rowsM, K, N, act, math, seed=0, beta=0.0, group=128):
+def run_case(q, orc, mode, E, rowsM, K, N, act, math, seed=0, beta=0.0, group=128, nt_beta=1.0):
     """One grouped call over E experts with the given row counts. Returns (got list, want list)."""
     import torch
     tot = sum(rowsM)
@@ -64,7 +64,7 @@ def run_case(q, orc, mode, E, rowsM, K, N, act, math, seed=0, beta=0.0, group=12
         pa = to_bf16_bits(dA) if bf else dA
         pb = to_bf16_bits(dB) if bf else dB
         esz = 2 if bf else 4
-        items = [(pa.data_ptr() + off[e] * K * esz, pb.data_ptr() + off[e] * N * esz, dC.data_ptr() + e * K * N * 4, 0, 0, rowsM[e], 1.0)
+        items = [(pa.data_ptr() + off[e] * K * esz, pb.data_ptr() + off[e] * N * esz, dC.data_ptr() + e * K * N * 4, 0, 0, rowsM[e], nt_beta)
                  for e in range(E)]
         pr = q.problems(items)
         q.gemm_nt(pr, E, K, N, act, math)
@@ -72,6 +72,8 @@ def run_case(q, orc, mode, E, rowsM, K, N, act, math, seed=0, beta=0.0, group=12
         want = C0.copy()
         for e in range(E):
             if rowsM[e]:
+                if nt_beta == 0.0:
+                    want[e * K * N:(e + 1) * K * N] = 0.0
                 orc.gemm_nt(A[off[e] * K:], B[off[e] * N:], want[e * K * N:(e + 1) * K * N], rowsM[e], K, N)
         return dC.cpu().numpy(), want
     wr, wc = (K, N) if mode == "nn" else (N, K)
@@ -184,6 +186,20 @@ def test_mfma_tn_many_rows_per_expert(q, orc, beta):
     activation tiles go straight to LDS; a ragged tail expert and an empty one ride along."""
     got, want = run_case(q, orc, "tn", 4, [2100, 1500, 0, 1311], 384, 256, pkg.ACT_BF16, pkg.MATH_MFMA, seed=4, beta=beta)
     assert orc.relerr(got, want) < TOL_MFMA
+
+
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_mfma_nt_split_contraction(q, orc, beta):
+    """One expert with far more rows than the others: its contraction is cut into slices that add up
+    in turn. Overwriting and accumulating, next to a small, an empty and a ragged expert; untouched
+    experts keep their gradient."""
+    got, want = run_case(q, orc, "nt", 4, [1700, 40, 0, 333], 256, 256, pkg.ACT_BF16, pkg.MATH_MFMA, seed=6, nt_beta=beta)
+    assert orc.relerr(got, want) < TOL_MFMA
+    K = N = 256
+    assert np.array_equal(got[2 * K * N:3 * K * N], want[2 * K * N:3 * K * N])
+    # twice in a row: the flags of the first launch must not satisfy the second
+    got2, want2 = run_case(q, orc, "nt", 4, [1700, 40, 0, 333], 256, 256, pkg.ACT_BF16, pkg.MATH_MFMA, seed=7, nt_beta=beta)
+    assert orc.relerr(got2, want2) < TOL_MFMA
 
 
 def test_mfma_rejects_unsupported_shapes(q):

@@ -80,26 +80,23 @@ __device__ __forceinline__ bf16x8 nn3_pack(const i32x2 lo, const i32x2 hi){
     return __builtin_bit_cast(bf16x8, v);
 }
 
-__global__ void __launch_bounds__(256, 2) k_gemm_nn_lds(Nn3Args a){
-    __shared__ __attribute__((aligned(16))) unsigned char lds[NN3_A_STAGES * NN3_A_BYTES + 2 * NN3_B_BYTES];
-    const int t = qx_xcd_tile(blockIdx.x, gridDim.x);
-    if(t >= a.ntiles) return;
-    const DevProb P = a.pr[qx_find_problem(a.pr, a.nprob, t)];
-    const int lt = t - P.tile0;
-    const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
-    const int i0 = ti * NN3_BM, j0 = tj * NN3_BN;
+/* One output tile of NI*64 rows: the four wavefronts 2x2, each NI x 2 accumulators. NI = 4 is the
+ * full tile; the last tile of a problem takes the smallest NI that holds its rows, so that an expert
+ * with 130 rows does a 192-row tile's work rather than a 256-row tile's. */
+template<int NI>
+__device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int i0, int j0, unsigned char *lds){
     const int rows = P.M;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wi = (wave >> 1) * 128, wj = (wave & 1) * 64;
+    const int wi = (wave >> 1) * (NI * 32), wj = (wave & 1) * 64;
     const int fr = lane & 31, hf = lane >> 5;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
     const int steps = a.K / NN3_BK;
 
     /* ---- activation pieces of this thread: position p = h*256 + tid of a stage is row p/4, stored
      * piece p%4 = ko ^ ((row >> 2) & 3) ---- */
-    const char *srcA[4];
+    const char *srcA[NI];
 #pragma unroll
-    for(int h = 0; h < 4; h++){
+    for(int h = 0; h < NI; h++){
         const int p = h * 256 + tid, r = p >> 2, ko = (p & 3) ^ ((r >> 2) & 3);
         const int rr = (i0 + r < rows) ? i0 + r : rows - 1;               /* clamp: feeds unstored rows only */
         srcA[h] = (const char *)P.A + ((size_t)rr * a.K + ko * 8) * 2;
@@ -109,7 +106,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nn_lds(Nn3Args a){
         const int tl = tile < steps ? tile : steps - 1;                   /* past the end: the last tile again, into a stage nobody reads */
         unsigned char *base = lds + stage * NN3_A_BYTES + wave_off;
 #pragma unroll
-        for(int h = 0; h < 4; h++)
+        for(int h = 0; h < NI; h++)
             __builtin_amdgcn_global_load_lds((glb_void *)(srcA[h] + (size_t)tl * (NN3_BK * 2)), (lds_void *)(base + h * 4096), 16, 0, 0);
     };
 
@@ -151,9 +148,9 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nn_lds(Nn3Args a){
     };
 
     /* ---- operand read offsets ---- */
-    uint32_t ra[2][4];                                   /* [k16 slice][row tile] activations, 128-bit */
+    uint32_t ra[2][NI];                                  /* [k16 slice][row tile] activations, 128-bit */
 #pragma unroll
-    for(int i = 0; i < 4; i++){
+    for(int i = 0; i < NI; i++){
         const int r = wi + i * 32 + fr, f = (r >> 2) & 3;
 #pragma unroll
         for(int ks = 0; ks < 2; ks++) ra[ks][i] = (uint32_t)(r * 64 + (((ks * 2 + hf) ^ f) << 4));
@@ -169,34 +166,83 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nn_lds(Nn3Args a){
         }
     }
 
-    f32x16 acc[4][2];
+    f32x16 acc[NI][2];
 #pragma unroll
-    for(int i = 0; i < 4; i++)
+    for(int i = 0; i < NI; i++)
 #pragma unroll
         for(int j = 0; j < 2; j++) acc[i][j] = (f32x16)(0.0f);
 
-    /* ---- prologue ---- */
+    /* ---- prologue: weights of step 0 into buffer 0, those of step 1 into registers ---- */
+    WLoad wcur;
     {
         WLoad w0 = load_w(0);
         issue_a(0, 0);
-        asm volatile("s_waitcnt vmcnt(4)" : "+v"(w0.d0), "+v"(w0.d1), "+v"(w0.s0), "+v"(w0.s1) :: "memory");
+        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(w0.d0), "+v"(w0.d1), "+v"(w0.s0), "+v"(w0.s1) : "n"(NI) : "memory");
         store_w(w0, 0);
+        wcur = load_w(1);
         issue_a(1, 1);
+        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(wcur.d0), "+v"(wcur.d1), "+v"(wcur.s0), "+v"(wcur.s1) : "n"(NI) : "memory");
     }
 
+    /* Main loop. A wavefront issues in order, and measured on this chip an MFMA of this shape keeps
+     * the vector ALU to itself for about half of its 32 cycles: some four ALU instructions behind an
+     * MFMA cost nothing, every further one its full four cycles, and whatever stands after the last
+     * MFMA of a step runs alone. Everything else of a step is therefore cut into small items and
+     * dealt evenly into the gaps after the MFMAs of both slices, fences keeping the compiler
+     * from gathering them again:
+     *   the four loads of the weights of step st+2 (into wnext, waited for at the end of the step,
+     *     when they have long arrived: an asynchronously loaded register must not be carried round
+     *     the loop before its wait), the activation requests of tile st+2,
+     *   the dequantisation of the weights of step st+1 (wcur), two weights per pair of items,
+     *   their four LDS writes into the buffer last read in step st-1. */
+    constexpr int SLOTS = NI * 8, ITEMS = 4 + NI + 16 + 4;
     for(int st = 0; st < steps; st++){
         /* tile st is in, own LDS writes are done; tile st+1 may still be on its way */
-        asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"(NI) : "memory");
         __builtin_amdgcn_s_barrier();
-        WLoad wn = load_w(st + 1);                         /* used at the end of this step */
-        issue_a(st + 2, (st + 2) % NN3_A_STAGES);
 
         const uint32_t sa = lds_base + (uint32_t)(st % NN3_A_STAGES) * NN3_A_BYTES;
         const uint32_t sbuf = lds_base + (uint32_t)(st & 1) * NN3_B_BYTES;
+        const uint32_t wbuf = lds_base + (uint32_t)((st + 1) & 1) * NN3_B_BYTES;
+        const int tile2 = st + 2 < steps ? st + 2 : steps - 1, stage2 = (st + 2) % NN3_A_STAGES;   /* past the end: the last one again, never used */
+        WLoad wnext;
+        i32x4 whi[2], wlo[2];
+        float wf[8][2];
+        auto item = [&](int k){
+            if(k == 0)      wnext.d0 = nn3_gld4(pw0 + (size_t)tile2 * wstep);
+            else if(k == 1) wnext.d1 = nn3_gld4(pw1 + (size_t)tile2 * wstep);
+            else if(k == 2) wnext.s0 = nn3_gld4(ps0 + (size_t)tile2 * sstep);
+            else if(k == 3) wnext.s1 = nn3_gld4(ps1 + (size_t)tile2 * sstep);
+            else if(k < 4 + NI)
+                __builtin_amdgcn_global_load_lds((glb_void *)(srcA[k - 4] + (size_t)tile2 * (NN3_BK * 2)),
+                                                 (lds_void *)(lds + stage2 * NN3_A_BYTES + wave_off + (k - 4) * 4096), 16, 0, 0);
+            else if(k < 4 + NI + 16){
+                const int q = k - 4 - NI, p = q >> 1, r = p >> 2, j = p & 3;
+                if((q & 1) == 0){
+                    const uint32_t dg = (uint32_t)(r ? wcur.d1 : wcur.d0);
+                    const float sc = __int_as_float(r ? wcur.s1 : wcur.s0);
+                    wf[p][0] = sc * (float)qx_nib(dg, 2 * j); wf[p][1] = sc * (float)qx_nib(dg, 2 * j + 1);
+                } else {
+                    const uint32_t h = nn3_pk(wf[p][0], wf[p][1]);
+                    whi[r][j] = (int)h;
+                    wlo[r][j] = (int)nn3_pk(wf[p][0] - __uint_as_float(h << 16), wf[p][1] - __uint_as_float(h & 0xFFFF0000u));
+                }
+            } else {
+                const int w = k - 4 - NI - 16;
+                if(w == 0)      nn3_wr128<0>(wbuf + wr0, whi[0]);
+                else if(w == 1) nn3_wr128<NN3_P_BYTES>(wbuf + wr0, wlo[0]);
+                else if(w == 2) nn3_wr128<0>(wbuf + wr1, whi[1]);
+                else            nn3_wr128<NN3_P_BYTES>(wbuf + wr1, wlo[1]);
+            }
+        };
         Nn3Ops o0, o1;
+        if(NI < 4){                                        /* the wait names all four; the spare ones hold nothing */
+#pragma unroll
+            for(int i = NI; i < 4; i++){ o0.a[i] = (i32x4)(0); o1.a[i] = (i32x4)(0); }
+        }
 #define NN3_READ(O, KS)                                                                                   \
         _Pragma("unroll")                                                                                 \
-        for(int i = 0; i < 4; i++) O.a[i] = nn3_rd128<0>(sa + ra[KS][i]);                                 \
+        for(int i = 0; i < NI; i++) O.a[i] = nn3_rd128<0>(sa + ra[KS][i]);                                \
         _Pragma("unroll")                                                                                 \
         for(int j = 0; j < 2; j++){                                                                       \
             O.bh[j][0] = nn3_tr<KS * 16 * 256>(sbuf + rb[j]);                                             \
@@ -204,32 +250,51 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nn_lds(Nn3Args a){
             O.bl[j][0] = nn3_tr<NN3_P_BYTES + KS * 16 * 256>(sbuf + rb[j]);                               \
             O.bl[j][1] = nn3_tr<NN3_P_BYTES + KS * 16 * 256 + 4 * 256>(sbuf + rb[j]);                     \
         }
-#define NN3_MMA(O)                                                                                        \
+#define NN3_MMA(O, BLOCK)                                                                                 \
         _Pragma("unroll")                                                                                 \
-        for(int i = 0; i < 4; i++)                                                                        \
-            _Pragma("unroll")                                                                             \
-            for(int j = 0; j < 2; j++){                                                                   \
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, O.a[i]), nn3_pack(O.bh[j][0], O.bh[j][1]), acc[i][j], 0, 0, 0); \
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, O.a[i]), nn3_pack(O.bl[j][0], O.bl[j][1]), acc[i][j], 0, 0, 0); \
-            }
+        for(int m = 0; m < NI * 4; m++){                   /* all hi parts, then all lo parts */            \
+            const int i = (m >> 1) % NI, j = m & 1;                                                       \
+            if(m < NI * 2) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, O.a[i]), nn3_pack(O.bh[j][0], O.bh[j][1]), acc[i][j], 0, 0, 0); \
+            else           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, O.a[i]), nn3_pack(O.bl[j][0], O.bl[j][1]), acc[i][j], 0, 0, 0); \
+            {                                                                                             \
+                const int slot = BLOCK * (SLOTS / 2) + m;                                                 \
+                __builtin_amdgcn_sched_barrier(0);                                                        \
+                _Pragma("unroll")                                                                         \
+                for(int k = slot * ITEMS / SLOTS; k < (slot + 1) * ITEMS / SLOTS; k++) item(k);           \
+                __builtin_amdgcn_sched_barrier(0);                                                        \
+            }                                                                                             \
+        }
         NN3_READ(o0, 0)
         nn3_wait(o0);
         NN3_READ(o1, 1)                                    /* in flight while slice 0 multiplies */
-        NN3_MMA(o0)
+        NN3_MMA(o0, 0)
         nn3_wait(o1);
-        NN3_MMA(o1)
+        NN3_MMA(o1, 1)
 #undef NN3_READ
 #undef NN3_MMA
-        /* digits and scales of step st+1 have arrived (only the four activation requests are younger);
-         * the buffer they go to was last read in step st-1 */
-        asm volatile("s_waitcnt vmcnt(4)" : "+v"(wn.d0), "+v"(wn.d1), "+v"(wn.s0), "+v"(wn.s1) :: "memory");
-        store_w(wn, (st + 1) & 1);
+        /* the weights of step st+2 have arrived (only the activation requests are younger) */
+        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(wnext.d0), "+v"(wnext.d1), "+v"(wnext.s0), "+v"(wnext.s1) : "n"(NI) : "memory");
+        wcur = wnext;
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);                    /* vmcnt(0), as a builtin so that the compiler knows it: no request may outlive the workgroup's LDS */
 
     /* ---- epilogue: the lane holds column lane%32 of each 32x32 tile, four-row band lane/32 ---- */
     const int row = i0 + wi + hf * 4;
-    qx_store_tiles<4, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
+    qx_store_tiles<NI, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
+}
+
+__global__ void __launch_bounds__(256, 2) k_gemm_nn_lds(Nn3Args a){
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NN3_A_STAGES * NN3_A_BYTES + 2 * NN3_B_BYTES];
+    const int t = qx_xcd_tile(blockIdx.x, gridDim.x);
+    if(t >= a.ntiles) return;
+    const DevProb P = a.pr[qx_find_problem(a.pr, a.nprob, t)];
+    const int lt = t - P.tile0;
+    const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
+    const int i0 = ti * NN3_BM, j0 = tj * NN3_BN, left = P.M - i0;
+    if(left > 192)      nn3_tile<4>(a, P, i0, j0, lds);
+    else if(left > 128) nn3_tile<3>(a, P, i0, j0, lds);
+    else if(left > 64)  nn3_tile<2>(a, P, i0, j0, lds);
+    else                nn3_tile<1>(a, P, i0, j0, lds);
 }
 
 /* bf16 activations only; N % 128 == 0, K % 32 == 0, group a power of two >= 32 (checked by the caller) */

@@ -68,25 +68,21 @@ __device__ __forceinline__ void tn3_wait(Tn3Ops &o){
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(o.a[0]), "+v"(o.a[1]), "+v"(o.b[0]), "+v"(o.b[1]));
 }
 
-__global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
-    __shared__ __attribute__((aligned(16))) unsigned char lds[TN3_A_STAGES * TN3_A_BYTES + 2 * TN3_B_BYTES];
-    const int t = qx_xcd_tile(blockIdx.x, gridDim.x);
-    if(t >= a.ntiles) return;
-    const DevProb P = a.pr[qx_find_problem(a.pr, a.nprob, t)];
-    const int lt = t - P.tile0;
-    const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
-    const int i0 = ti * TN3_BM, j0 = tj * TN3_BN;
+/* One output tile of NI*64 rows: the four wavefronts 2x2, each NI x 2 accumulators. NI = 2 is the
+ * full tile; a last tile with at most 64 rows does half the work. */
+template<int NI>
+__device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, int i0, int j0, unsigned char *lds){
     const int rows = P.M;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;
+    const int wi = (wave >> 1) * (NI * 32), wj = (wave & 1) * 64;
     const int fr = lane & 31, hf = lane >> 5;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
 
     /* ---- activation pieces of this thread: position p = h*256 + tid of a stage is row p/8, stored
      * piece p%8 = ko ^ ((row >> 1) & 7) ---- */
-    const char *srcA[4];
+    const char *srcA[2 * NI];
 #pragma unroll
-    for(int h = 0; h < 4; h++){
+    for(int h = 0; h < 2 * NI; h++){
         const int p = h * 256 + tid, r = p >> 3, ko = (p & 7) ^ ((r >> 1) & 7);
         const int rr = (i0 + r < rows) ? i0 + r : rows - 1;               /* clamp: feeds unstored rows only */
         srcA[h] = (const char *)P.A + ((size_t)rr * a.K + ko * 8) * 2;
@@ -97,7 +93,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
         const int tl = tile < steps ? tile : steps - 1;                   /* past the end: the last tile again, into a stage nobody reads */
         unsigned char *base = lds + stage * TN3_A_BYTES + wave_off;
 #pragma unroll
-        for(int h = 0; h < 4; h++)
+        for(int h = 0; h < 2 * NI; h++)
             __builtin_amdgcn_global_load_lds((glb_void *)(srcA[h] + (size_t)tl * (TN3_BK * 2)), (lds_void *)(base + h * 4096), 16, 0, 0);
     };
 
@@ -151,9 +147,9 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
         return tn3_gld4(pfold[j] + g);
     };
 
-    f32x16 acc[2][2], part[2][2];
+    f32x16 acc[NI][2], part[NI][2];
 #pragma unroll
-    for(int i = 0; i < 2; i++)
+    for(int i = 0; i < NI; i++)
 #pragma unroll
         for(int j = 0; j < 2; j++){ acc[i][j] = (f32x16)(0.0f); part[i][j] = (f32x16)(0.0f); }
 
@@ -166,7 +162,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
         i32x4 w0 = load_w(0);
         float f0 = load_scale(0, 0), f1 = load_scale(0, 1);
         issue_a(0, 0);
-        asm volatile("s_waitcnt vmcnt(4)" : "+v"(w0), "+v"(f0), "+v"(f1) :: "memory");
+        asm volatile("s_waitcnt vmcnt(%3)" : "+v"(w0), "+v"(f0), "+v"(f1) : "n"(2 * NI) : "memory");
         store_w(w0, 0);
         fs_cur[0] = f0; fs_cur[1] = f1;
         issue_a(1, 1);
@@ -174,7 +170,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
 
     for(int st = 0; st < steps; st++){
         /* tile st is in, own LDS writes are done; tile st+1 may still be on its way */
-        asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"(2 * NI) : "memory");
         __builtin_amdgcn_s_barrier();
         i32x4 wnext = load_w(st + 1);                      /* digits and scales of step st+1: used at the end of this step */
         float fn0 = load_scale(st + 1, 0), fn1 = load_scale(st + 1, 1);
@@ -183,18 +179,19 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
         const uint32_t sa = lds_base + (uint32_t)(st % TN3_A_STAGES) * TN3_A_BYTES;
         const uint32_t sbuf = lds_base + (uint32_t)(st & 1) * TN3_B_BYTES;
         Tn3Ops o[2];
-        o[0].a[0] = tn3_rd<0>(sa + ra[0]); o[0].a[1] = tn3_rd<32 * 128>(sa + ra[0]);
+        if(NI < 2){ o[0].a[1] = (i32x4)(0); o[1].a[1] = (i32x4)(0); }   /* the wait names both */
+        o[0].a[0] = tn3_rd<0>(sa + ra[0]); if(NI > 1) o[0].a[1] = tn3_rd<32 * 128>(sa + ra[0]);
         o[0].b[0] = tn3_rd<0>(sbuf + rb[0]); o[0].b[1] = tn3_rd<32 * 16>(sbuf + rb[0]);
         tn3_wait(o[0]);
 #pragma unroll
         for(int ks = 0; ks < 4; ks++){
             Tn3Ops &cur = o[ks & 1], &nxt = o[(ks + 1) & 1];
             if(ks < 3){
-                nxt.a[0] = tn3_rd<0>(sa + ra[ks + 1]); nxt.a[1] = tn3_rd<32 * 128>(sa + ra[ks + 1]);
+                nxt.a[0] = tn3_rd<0>(sa + ra[ks + 1]); if(NI > 1) nxt.a[1] = tn3_rd<32 * 128>(sa + ra[ks + 1]);
                 nxt.b[0] = tn3_rd<0>(sbuf + rb[ks + 1]); nxt.b[1] = tn3_rd<32 * 16>(sbuf + rb[ks + 1]);
             }
 #pragma unroll
-            for(int i = 0; i < 2; i++)
+            for(int i = 0; i < NI; i++)
 #pragma unroll
                 for(int j = 0; j < 2; j++)
                     part[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, cur.a[i]), __builtin_bit_cast(bf16x8, cur.b[j]), part[i][j], 0, 0, 0);
@@ -205,16 +202,16 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
 #pragma unroll
             for(int j = 0; j < 2; j++){
 #pragma unroll
-                for(int i = 0; i < 2; i++){
+                for(int i = 0; i < NI; i++){
 #pragma unroll
                     for(int e = 0; e < 16; e++) acc[i][j][e] = fmaf(fs_cur[j], part[i][j][e], acc[i][j][e]);
                     part[i][j] = (f32x16)(0.0f);
                 }
             }
         }
-        /* digits and scales of step st+1 have arrived (only the four activation requests are younger);
+        /* digits and scales of step st+1 have arrived (only the activation requests are younger);
          * the buffer they go to was last read in step st-1 */
-        asm volatile("s_waitcnt vmcnt(4)" : "+v"(wnext), "+v"(fn0), "+v"(fn1) :: "memory");
+        asm volatile("s_waitcnt vmcnt(%3)" : "+v"(wnext), "+v"(fn0), "+v"(fn1) : "n"(2 * NI) : "memory");
         store_w(wnext, (st + 1) & 1);
         fs_cur[0] = fn0; fs_cur[1] = fn1;
     }
@@ -222,7 +219,19 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
 
     /* ---- epilogue: the lane holds column lane%32 of each 32x32 tile, four-row band lane/32 ---- */
     const int row = i0 + wi + hf * 4;
-    qx_store_tiles<2, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
+    qx_store_tiles<NI, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
+}
+
+__global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
+    __shared__ __attribute__((aligned(16))) unsigned char lds[TN3_A_STAGES * TN3_A_BYTES + 2 * TN3_B_BYTES];
+    const int t = qx_xcd_tile(blockIdx.x, gridDim.x);
+    if(t >= a.ntiles) return;
+    const DevProb P = a.pr[qx_find_problem(a.pr, a.nprob, t)];
+    const int lt = t - P.tile0;
+    const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
+    const int i0 = ti * TN3_BM, j0 = tj * TN3_BN;
+    if(P.M - i0 > 64) tn3_tile<2>(a, P, i0, j0, lds);
+    else              tn3_tile<1>(a, P, i0, j0, lds);
 }
 
 /* bf16 activations only; N % 128 == 0, K % 64 == 0, group a power of two >= 64 (checked by the caller) */

@@ -172,16 +172,17 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int
 #pragma unroll
         for(int j = 0; j < 2; j++) acc[i][j] = (f32x16)(0.0f);
 
-    /* ---- prologue: weights of step 0 into buffer 0, those of step 1 into registers ---- */
+    /* ---- prologue: weights of step 0 into buffer 0, those of step 1 into registers; all requests
+     * go out before the one wait ---- */
     WLoad wcur;
     {
         WLoad w0 = load_w(0);
-        issue_a(0, 0);
-        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(w0.d0), "+v"(w0.d1), "+v"(w0.s0), "+v"(w0.s1) : "n"(NI) : "memory");
-        store_w(w0, 0);
         wcur = load_w(1);
+        issue_a(0, 0);
         issue_a(1, 1);
-        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(wcur.d0), "+v"(wcur.d1), "+v"(wcur.s0), "+v"(wcur.s1) : "n"(NI) : "memory");
+        asm volatile("s_waitcnt vmcnt(%8)" : "+v"(w0.d0), "+v"(w0.d1), "+v"(w0.s0), "+v"(w0.s1),
+                                              "+v"(wcur.d0), "+v"(wcur.d1), "+v"(wcur.s0), "+v"(wcur.s1) : "n"(2 * NI) : "memory");
+        store_w(w0, 0);
     }
 
     /* Main loop. A wavefront issues in order, and measured on this chip an MFMA of this shape keeps

@@ -153,67 +153,105 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, int
 #pragma unroll
         for(int j = 0; j < 2; j++){ acc[i][j] = (f32x16)(0.0f); part[i][j] = (f32x16)(0.0f); }
 
-    /* ---- prologue. Issue order matters: each wait below lets the four activation requests issued
-     * last stay in flight and nothing else. A value loaded by inline assembly is never carried around
-     * the loop: it is requested after the barrier of a step and consumed, behind a wait that names it,
-     * at the end of the same step (the compiler may copy a loop-carried value before it has arrived). ---- */
+    /* ---- prologue: digits of step 0 into buffer 0, those of step 1 into registers, the scales of
+     * step 0; all requests go out before the one wait ---- */
     float fs_cur[2];
+    i32x4 wcur;
     {
         i32x4 w0 = load_w(0);
+        wcur = load_w(1);
         float f0 = load_scale(0, 0), f1 = load_scale(0, 1);
         issue_a(0, 0);
-        asm volatile("s_waitcnt vmcnt(%3)" : "+v"(w0), "+v"(f0), "+v"(f1) : "n"(2 * NI) : "memory");
+        issue_a(1, 1);
+        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(w0), "+v"(wcur), "+v"(f0), "+v"(f1) : "n"(4 * NI) : "memory");
         store_w(w0, 0);
         fs_cur[0] = f0; fs_cur[1] = f1;
-        issue_a(1, 1);
     }
 
+    /* Main loop. A wavefront issues in order, and an MFMA of this shape keeps the vector ALU to itself
+     * for about half of its 32 cycles: some four ALU instructions behind an MFMA cost nothing, every
+     * further one its full four cycles, a memory request more, and whatever stands after the last MFMA
+     * of a step runs alone. Everything else of a step is therefore cut into items and dealt evenly
+     * into the gaps after the MFMAs, fences keeping the compiler from gathering them again:
+     *   the loads of the digits of step st+2 and the scales of step st+1 (waited for at the end of the step, when they have
+     *     long arrived: an asynchronously loaded register must not be carried round the loop before
+     *     its wait) and the activation requests of tile st+2,
+     *   the conversion of the digits of step st+1 (wcur) to bf16, four digits per item, each 16-byte
+     *     unit written to the buffer last read in step st-1 as soon as it is complete.
+     * A scale group's partial sums start from a zero operand instead of cleared registers. */
+    constexpr int SLOTS = NI * 8, ITEMS = 3 + 2 * NI + 8 + 4;
+    const f32x16 zero = (f32x16)(0.0f);
     for(int st = 0; st < steps; st++){
         /* tile st is in, own LDS writes are done; tile st+1 may still be on its way */
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"(2 * NI) : "memory");
         __builtin_amdgcn_s_barrier();
-        i32x4 wnext = load_w(st + 1);                      /* digits and scales of step st+1: used at the end of this step */
-        float fn0 = load_scale(st + 1, 0), fn1 = load_scale(st + 1, 1);
-        issue_a(st + 2, (st + 2) % TN3_A_STAGES);
 
         const uint32_t sa = lds_base + (uint32_t)(st % TN3_A_STAGES) * TN3_A_BYTES;
         const uint32_t sbuf = lds_base + (uint32_t)(st & 1) * TN3_B_BYTES;
+        const uint32_t wbuf = lds_base + (uint32_t)((st + 1) & 1) * TN3_B_BYTES;
+        const int tile2 = st + 2 < steps ? st + 2 : steps - 1, stage2 = (st + 2) % TN3_A_STAGES;   /* past the end: the last one again, never used */
+        i32x4 wnext; float fn[2];
+        i32x4 wv[4];
+        auto item = [&](int k){
+            if(k == 0)      wnext = tn3_gld16(pw + (size_t)tile2 * (TN3_BK / 2));
+            else if(k < 3)  fn[k - 1] = load_scale(st + 1, k - 1);
+            else if(k < 3 + 2 * NI)
+                __builtin_amdgcn_global_load_lds((glb_void *)(srcA[k - 3] + (size_t)tile2 * (TN3_BK * 2)),
+                                                 (lds_void *)(lds + stage2 * TN3_A_BYTES + wave_off + (k - 3) * 4096), 16, 0, 0);
+            else {
+                /* per 16-byte unit: two conversion items, then its write */
+                const int q = k - 3 - 2 * NI, j = q / 3, h = q % 3;
+                if(h < 2){
+                    const uint32_t wd = (uint32_t)wcur[j];
+                    wv[j][2 * h]     = (int)tn3_pk((float)qx_nib(wd, 4 * h),     (float)qx_nib(wd, 4 * h + 1));
+                    wv[j][2 * h + 1] = (int)tn3_pk((float)qx_nib(wd, 4 * h + 2), (float)qx_nib(wd, 4 * h + 3));
+                } else tn3_wr(wbuf + wr_off[j], wv[j]);
+            }
+        };
+        const bool fresh = st % spg == 0, last = (st + 1) % spg == 0;
         Tn3Ops o[2];
         if(NI < 2){ o[0].a[1] = (i32x4)(0); o[1].a[1] = (i32x4)(0); }   /* the wait names both */
         o[0].a[0] = tn3_rd<0>(sa + ra[0]); if(NI > 1) o[0].a[1] = tn3_rd<32 * 128>(sa + ra[0]);
         o[0].b[0] = tn3_rd<0>(sbuf + rb[0]); o[0].b[1] = tn3_rd<32 * 16>(sbuf + rb[0]);
         tn3_wait(o[0]);
-#pragma unroll
-        for(int ks = 0; ks < 4; ks++){
-            Tn3Ops &cur = o[ks & 1], &nxt = o[(ks + 1) & 1];
-            if(ks < 3){
-                nxt.a[0] = tn3_rd<0>(sa + ra[ks + 1]); if(NI > 1) nxt.a[1] = tn3_rd<32 * 128>(sa + ra[ks + 1]);
-                nxt.b[0] = tn3_rd<0>(sbuf + rb[ks + 1]); nxt.b[1] = tn3_rd<32 * 16>(sbuf + rb[ks + 1]);
-            }
-#pragma unroll
-            for(int i = 0; i < NI; i++)
-#pragma unroll
-                for(int j = 0; j < 2; j++)
-                    part[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, cur.a[i]), __builtin_bit_cast(bf16x8, cur.b[j]), part[i][j], 0, 0, 0);
-            if(ks < 3) tn3_wait(nxt);
+#define TN3_KS(KS, ZERO)                                                                                  \
+        {                                                                                                 \
+            Tn3Ops &cur = o[KS & 1], &nxt = o[(KS + 1) & 1];                                              \
+            if(KS < 3){                                                                                   \
+                nxt.a[0] = tn3_rd<0>(sa + ra[(KS + 1) & 3]); if(NI > 1) nxt.a[1] = tn3_rd<32 * 128>(sa + ra[(KS + 1) & 3]); \
+                nxt.b[0] = tn3_rd<0>(sbuf + rb[(KS + 1) & 3]); nxt.b[1] = tn3_rd<32 * 16>(sbuf + rb[(KS + 1) & 3]);         \
+            }                                                                                             \
+            _Pragma("unroll")                                                                             \
+            for(int m = 0; m < NI * 2; m++){                                                              \
+                const int i = m >> 1, j = m & 1;                                                          \
+                part[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, cur.a[i]), __builtin_bit_cast(bf16x8, cur.b[j]), ZERO ? zero : part[i][j], 0, 0, 0); \
+                const int slot = KS * NI * 2 + m;                                                         \
+                __builtin_amdgcn_sched_barrier(0);                                                        \
+                _Pragma("unroll")                                                                         \
+                for(int k = slot * ITEMS / SLOTS; k < (slot + 1) * ITEMS / SLOTS; k++) item(k);           \
+                __builtin_amdgcn_sched_barrier(0);                                                        \
+            }                                                                                             \
+            if(KS < 3) tn3_wait(nxt);                                                                     \
         }
-        if((st + 1) % spg == 0){
-            /* one scale group of the contraction is complete: fold it in with its fp32 scale */
+        if(fresh) TN3_KS(0, true) else TN3_KS(0, false)
+        TN3_KS(1, false)
+        TN3_KS(2, false)
+        TN3_KS(3, false)
+#undef TN3_KS
+        if(last){
+            /* one scale group of the contraction is complete: fold it in with its fp32 scale (spreading
+             * these among the MFMAs as well costs some fifty registers, which spill) */
 #pragma unroll
-            for(int j = 0; j < 2; j++){
+            for(int j = 0; j < 2; j++)
 #pragma unroll
-                for(int i = 0; i < NI; i++){
+                for(int i = 0; i < NI; i++)
 #pragma unroll
                     for(int e = 0; e < 16; e++) acc[i][j][e] = fmaf(fs_cur[j], part[i][j][e], acc[i][j][e]);
-                    part[i][j] = (f32x16)(0.0f);
-                }
-            }
         }
-        /* digits and scales of step st+1 have arrived (only the activation requests are younger);
-         * the buffer they go to was last read in step st-1 */
-        asm volatile("s_waitcnt vmcnt(%3)" : "+v"(wnext), "+v"(fn0), "+v"(fn1) : "n"(2 * NI) : "memory");
-        store_w(wnext, (st + 1) & 1);
-        fs_cur[0] = fn0; fs_cur[1] = fn1;
+        /* the digits of step st+2 and the scales of step st+1 have arrived (only the activation requests are younger) */
+        asm volatile("s_waitcnt vmcnt(%3)" : "+v"(wnext), "+v"(fn[0]), "+v"(fn[1]) : "n"(2 * NI) : "memory");
+        wcur = wnext;
+        fs_cur[0] = fn[0]; fs_cur[1] = fn[1];
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);                    /* vmcnt(0), as a builtin so that the compiler knows it: no request may outlive the workgroup's LDS */
 

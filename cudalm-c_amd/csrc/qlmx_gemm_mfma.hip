@@ -406,15 +406,7 @@ int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int 
     }
     QLMX_REQUIRE(mode == GEMM_NT || ((uintptr_t)d & 15) == 0, "mfma gemm: digit array is not 16-byte aligned");
     /* bf16 operands take the direct-to-LDS kernels; fp32 activations need the converting ones */
-    if(mode == GEMM_TN && act_dtype == QLMX_ACT_BF16){
-        /* measured: the direct-to-LDS input-gradient kernel wins from about 1000 rows per expert on
-         * (575 against 540 TFLOP/s at 2048) and, with fewer rows, when the contraction is long (K = 2048,
-         * Zipf-loaded 512 rows per expert on average: 117 against 122 us); short contractions over few
-         * rows stay with the register-staged kernel (K = 768: 124 against 127 us) */
-        long long rows = 0; int live = 0;
-        for(int i = 0; i < nprob; i++) if(probs[i].M > 0){ rows += probs[i].M; live++; }
-        if(live && (rows / live >= 1024 || K >= 1024)) return qlmx_gemm_tn_lds_launch(d, s, group, probs, nprob, K, N, st);
-    }
+    if(mode == GEMM_TN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_tn_lds_launch(d, s, group, probs, nprob, K, N, st);
     if(mode == GEMM_NT && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nt_lds_launch(probs, nprob, K, N, st);
     if(mode == GEMM_NN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nn_lds_launch(d, s, group, probs, nprob, K, N, st);
     if(mode == GEMM_NN) return launch_mfma<GEMM_NN, 4, true>(d, s, group, probs, nprob, K, N, act_dtype, st);

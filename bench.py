@@ -151,7 +151,7 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2):
         "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tm["wall_ms"], "dtype": "bf16",
         "kernel_ms": tm, "per_launch": per, "gflop_per_step": flops / 1e9,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "kernel": "k_gemm_mfma<nn|tn|nt> (all 7 launches; slowest: %s)" % dom,
+                     "traffic": None, "kernel": "k_gemm_nn_lds, k_gemm_tn_lds, k_gemm_nt_lds (all 7 launches; slowest: %s)" % dom,
                      "note": "algorithmic flops only; the forward issues two MFMAs per product (bf16 hi+lo weight split)"},
     }
 
@@ -353,7 +353,7 @@ def cpu_gemm(args):
 # counter values and scale factors are in profiles/*.txt. adamw: per launch. train: per step, i.e. summed over
 # the step's 7 launches (1020 MiB read + 1104 MiB written). decode: per launch = per layer at T=16
 # (56.2 MiB read + 4.5 MiB written).
-PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.227e9, "decode": 6.37e7}
+PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.50e9, "decode": 6.37e7}
 
 
 def main():

@@ -202,6 +202,28 @@ def test_mfma_nt_split_contraction(q, orc, beta):
     assert orc.relerr(got2, want2) < TOL_MFMA
 
 
+@pytest.mark.parametrize("mode", ["nn", "tn"])
+def test_mfma_last_tile_heights(q, orc, mode):
+    """The last row tile of a problem runs at the smallest height (in steps of 64 rows) that holds it:
+    row counts on both sides of every step, for the forward (256-row tiles) and the input gradient (128)."""
+    rows = [1, 64, 65, 128, 129, 192, 193, 256, 257, 449]
+    K, N = (64, 128) if mode == "nn" else (128, 128)
+    for beta in ([0.0] if mode == "nn" else [0.0, 1.0]):
+        got, want = run_case(q, orc, mode, len(rows), rows, K, N, pkg.ACT_BF16, pkg.MATH_MFMA, seed=11, beta=beta)
+        assert orc.relerr(got, want) < TOL_MFMA, (mode, beta)
+
+
+@pytest.mark.parametrize("mode", ["nn", "tn", "nt"])
+def test_mfma_more_problems_than_lanes(q, orc, mode):
+    """70 experts, some empty: the problem table is longer than one wavefront's lookup pass."""
+    rng = np.random.default_rng(3)
+    rows = [int(r) for r in rng.integers(0, 40, 70)]
+    rows[0] = 0; rows[69] = 37
+    K, N = {"nn": (64, 128), "tn": (128, 128), "nt": (64, 128)}[mode]
+    got, want = run_case(q, orc, mode, 70, rows, K, N, pkg.ACT_BF16, pkg.MATH_MFMA, seed=12)
+    assert orc.relerr(got, want) < TOL_MFMA
+
+
 def test_mfma_rejects_unsupported_shapes(q):
     import torch
     x = torch.zeros(4096, device="cuda")

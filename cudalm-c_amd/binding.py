@@ -72,6 +72,8 @@ SIGNATURES = {
     "qlmx_moe_gemm_nt": (c_i, [c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_decode_forward": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_step_touched": (c_i, [c_vp] * 10 + [c_i, c_i, c_i, c_f, c_f, c_f, c_f, c_f, c_f, c_f, c_u64, c_u64, c_vp, c_i, c_vp]),
+    "qlmx_sqsum": (c_i, [c_vp, c_u64, c_vp, c_vp]),
+    "qlmx_gnorm": (c_i, [c_vp, c_i, c_i, c_vp, c_vp]),
     "qlmx_router_topk": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_vp, c_i, c_vp]),
     "qlmx_moe_perm_workspace": (c_sz, [c_i, c_i, c_i]),
     "qlmx_moe_perm": (c_i, [c_vp, c_i, c_i, c_i, c_vp, c_vp, c_vp, c_vp]),
@@ -158,6 +160,12 @@ class Qlmx:
                      inv_bc1, inv_sqrt_bc2, t, nt, gs=None, v4=0, stream=None):
         self.call("qlmx_step_touched", P, Gc, d, r, s, m8, m8s, v8, v8s, touched, ntouched, group, dmax, lr, b1, b2, wd, sref,
                   inv_bc1, inv_sqrt_bc2, t, nt, gs, v4, stream)
+
+    def sqsum(self, G, n, part64, stream=None):
+        self.call("qlmx_sqsum", G, n, part64, stream)
+
+    def gnorm(self, part, nside, clip_side, gs, stream=None):
+        self.call("qlmx_gnorm", part, nside, clip_side, gs, stream)
 
     # MoE glue (argument order of the reference kernels)
     def router_topk(self, rt, rprobs, assign, gate, N, E, K, bias=None, bs=0, stream=None):

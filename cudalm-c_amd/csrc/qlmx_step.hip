@@ -336,3 +336,54 @@ extern "C" int qlmx_step_touched(float *P, const float *Gc, signed char *d, sign
     QLMX_LAUNCH_CHECK("qlmx_step_touched launch");
     return QLMX_OK;
 }
+
+/* ---- gradient-norm clipping around the step (cudalm.cu:2794-2820, CPU twins cpu_kern.h:533-546) ----
+ * k_sqsum: 64 partial sums of squares; partial c covers G[n*c/64 .. n*(c+1)/64), is accumulated in
+ * double and rounded to float once (the CPU path's definition; the reference's GPU kernel sums
+ * strided in fp32 and differs from its own CPU kernel in the last bits). Here a workgroup sums its
+ * chunk in double, lanes strided, then a fixed tree: the order of the double additions is not the
+ * CPU's, which can move the double sum by a few units in its last place -- far below half a float
+ * ulp except on an exact tie. */
+__global__ void __launch_bounds__(256) k_qlmx_sqsum(const float *G, unsigned long long n, float *part){
+    __shared__ double red[256];
+    const unsigned long long c = blockIdx.x, nb = gridDim.x;
+    const unsigned long long i0 = n * c / nb, i1 = n * (c + 1) / nb;
+    double s = 0.0;
+    for(unsigned long long i = i0 + threadIdx.x; i < i1; i += 256){ const double g = (double)G[i]; s += g * g; }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for(int o = 128; o > 0; o >>= 1){
+        if((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+        __syncthreads();
+    }
+    if(threadIdx.x == 0) part[c] = (float)red[0];
+}
+
+/* k_gnorm (cudalm.cu:2811-2816 = cpu_kern.h:541-546): part = G's 64 partials followed by nside more
+ * slices of 64; gs[0] = clip multiplier (exactly 1 when the norm is <= 1), gs[1] = the norm; a
+ * non-finite side sum makes the norm NaN. One thread, the reference's order of additions. */
+__global__ void k_qlmx_gnorm(const float *part, int nside, int clip_side, float *gs){
+    double ss = 0.0, sd = 0.0;
+    for(int i = 0; i < 64; i++) ss += (double)part[i];
+    for(int i = 64; i < 64 * (1 + nside); i++) sd += (double)part[i];
+    float gn = (float)sqrt(clip_side ? ss + sd : ss);
+    if(!isfinite(sd)) gn = __builtin_nanf("");
+    gs[0] = gn > 1.0f ? 1.0f / gn : 1.0f;
+    gs[1] = gn;
+}
+
+extern "C" int qlmx_sqsum(const float *G, unsigned long long n, float *part64, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(G && part64, "qlmx_sqsum: NULL buffer");
+    hipLaunchKernelGGL(k_qlmx_sqsum, dim3(64), dim3(256), 0, (hipStream_t)stream, G, n, part64);
+    QLMX_LAUNCH_CHECK("qlmx_sqsum launch");
+    return QLMX_OK;
+}
+
+extern "C" int qlmx_gnorm(const float *part, int nside, int clip_side, float *gs, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(part && gs && nside >= 0, "qlmx_gnorm: bad arguments");
+    hipLaunchKernelGGL(k_qlmx_gnorm, dim3(1), dim3(1), 0, (hipStream_t)stream, part, nside, clip_side, gs);
+    QLMX_LAUNCH_CHECK("qlmx_gnorm launch");
+    return QLMX_OK;
+}

@@ -121,6 +121,35 @@ void qlm_gpu_update(Qlm *q, float *P, float *G, float lr, float b1, float b2, fl
         ck(qlmx_servo(q->d, q->r, q->s, q->spanD, q->nspan, q->group, q->dmax, q->f_hi, q->f_lo, q->packed, (int)q->ngrp, NULL), "qlm servo");
 }
 
+/* cudalm.cu:6110-6135 without the float spans' AdamW and the diagnostics */
+void qlm_fused_spans(Qlm *q, float *P, float *G, int span0, int nspans, size_t g0, size_t gn, float *part64,
+                     float lr, float wd, int t, float prev_gn){
+    const float b1 = 0.9f, b2 = 0.95f;
+    const float bc1 = 1.0f - powf(b1, (float)t), bc2 = 1.0f - powf(b2, (float)t);
+    const float inv_bc1 = 1.0f / bc1, inv_sqrt_bc2 = 1.0f / sqrtf(bc2);
+    const float gscale = prev_gn > 1.0f ? 1.0f / prev_gn : 1.0f;
+    ck(qlmx_sqsum(G + g0, (unsigned long long)gn, part64, NULL), "fused sqsum");
+    int gi0 = q->spanH[span0].gi0, ng = 0;
+    for(int i = span0; i < span0 + nspans; i++) ng += q->spanH[i].ngrp;
+    qlm_step_launch(q->render_p ? P : NULL, G, q->d, q->r, q->s, q->m8, q->m8s, q->v8, q->v8s, q->spanD, q->nspan,
+                    q->group, q->dmax, lr, b1, b2, wd, gscale, NULL, inv_bc1, inv_sqrt_bc2, q->lrmode,
+                    (unsigned long long)t, q->adam, NULL, q->packed, gi0, ng);
+}
+void qlm_fused_layer(Qlm *q, float *P, float *G, size_t layer_g0, size_t layer_gn, float *gnpart, int l,
+                     float lr, float wd, int t, float prev_gn){
+    qlm_fused_spans(q, P, G, 7 * l, 7, layer_g0, layer_gn, gnpart + 64 * (size_t)l, lr, wd, t, prev_gn);
+}
+/* cudalm.cu:6176-6186 */
+float qlm_fused_tail(const float *gnpart, int L, const float *extra, int nextra){
+    const size_t nsl = 64 * (size_t)L, nex = 64 * (size_t)nextra;
+    std::vector<float> ph(nsl + nex);
+    if(nsl) ck(qlmx_memcpy_d2h(ph.data(), gnpart, nsl * 4), "fused sqsum d2h");
+    if(nex) ck(qlmx_memcpy_d2h(ph.data() + nsl, extra, nex * 4), "fused tail sqsum d2h");
+    double ss = 0;
+    for(size_t i = 0; i < nsl + nex; i++) ss += ph[i];
+    return (float)sqrt(ss);
+}
+
 /* qlm.cuh:678-683 */
 double qlm_persist_bytes(const Qlm *q){
     return (double)qlmx_qd_bytes(q->nq, q->packed) + (double)q->nq * 1.0 + (double)q->nq * (q->adam ? 2.0 : 1.0)

@@ -2,8 +2,9 @@
  *
  * Same names, argument order and error behaviour as the reference's host code so that cudalm.cu's
  * call sites keep compiling against it: the Qlm / QSpanD types (qlm.cuh:30-58), qlm_add_span,
- * qlm_gpu_init, qlm_gpu_render, qlm_render_layer, qlm_step_launch, qlm_gpu_update, qlm_save /
- * qlm_load (qlm.cuh:448-541, 577-591, 377-397, 702-788; cudalm.cu:6082-6103) and the grouped expert
+ * qlm_gpu_init, qlm_gpu_render, qlm_render_layer, qlm_step_launch, qlm_gpu_update, qlm_fused_layer /
+ * qlm_fused_tail, qlm_save / qlm_load (qlm.cuh:448-541, 577-591, 377-397, 702-788; cudalm.cu:6082-6103,
+ * 6110-6187) and the grouped expert
  * GEMM queue mg_ab / mg_abt / mg_abt_b / mg_atb / mg_flush (cudalm.cu:3204-3256). Failures print
  * and exit(1) like ck()/ckb() (cudalm.cu:147-152).
  *
@@ -59,6 +60,18 @@ void  qlm_step_launch(float *P, const float *G, signed char *d, signed char *r, 
                       int gi_base, int ng);                             /* qlm.cuh:377 */
 void  qlm_gpu_update(Qlm *q, float *P, float *G, float lr, float b1, float b2, float wd,
                      float bc1, float bc2, int t, const float *gs);     /* cudalm.cu:6082 */
+/* Fused per-layer update (cudalm.cu:6110-6135): step exactly spans [span0, span0+nspans) -- a layer is the 7
+ * spans 7l..7l+6 (qlm.cuh:479-489) -- while their gradients are live, clipped by the PREVIOUS step's norm
+ * (gscale = 1/prev_gn above 1), and leave the 64 partial sums of squares of G[g0 .. g0+gn) in part64.
+ * qlm_fused_tail (cudalm.cu:6176-6186) closes the step: the norm over L slices of 64 layer partials plus
+ * `nextra` further slices (embedding, final norm, ... summed by the caller with qlmx_sqsum), added up on
+ * the host in double; it clips the next step. The float spans' AdamW in both reference functions is the
+ * caller's. */
+void  qlm_fused_spans(Qlm *q, float *P, float *G, int span0, int nspans, size_t g0, size_t gn, float *part64,
+                      float lr, float wd, int t, float prev_gn);
+void  qlm_fused_layer(Qlm *q, float *P, float *G, size_t layer_g0, size_t layer_gn, float *gnpart, int l,
+                      float lr, float wd, int t, float prev_gn);
+float qlm_fused_tail(const float *gnpart, int L, const float *extra, int nextra);
 double qlm_persist_bytes(const Qlm *q);                                 /* qlm.cuh:678 */
 int   qlm_save(const Qlm *q, const char *path, int iter, float prev_gn); /* qlm.cuh:702 */
 int   qlm_load(Qlm *q, const char *path, int *iter, float *prev_gn);    /* qlm.cuh:740 */

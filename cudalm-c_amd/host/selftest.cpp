@@ -91,6 +91,30 @@ int main(){
     int iter = 0; float pg = 0; okio = okio && qlm_load(&q, path, &iter, &pg);
     std::vector<signed char> gd2(nd); qlmx_memcpy_d2h(gd2.data(), q.d, nd);
     check("qlm save/load round trip", (okio && iter == 77 && pg == 1.25f && !memcmp(gd.data(), gd2.data(), nd)) ? 0 : 1, 0);
+
+    /* (c2) fused per-layer update: stepping span by span while "its gradients are live", clipped by the
+     * previous step's norm, must leave the same state as one step over all groups with that multiplier;
+     * the partial sums collected on the way give this step's norm */
+    {
+        const int T2 = 4; const float prev_gn = 2.5f;
+        const float c1 = 1.0f - powf(b1, (float)T2), c2 = 1.0f - powf(b2, (float)T2);
+        int okf = qlm_save(&q, path, 78, prev_gn);
+        qlm_step_launch(Pd, Gd, q.d, q.r, q.s, q.m8, q.m8s, q.v8, q.v8s, q.spanD, q.nspan, q.group, q.dmax, lr, b1, b2, wd,
+                        1.0f / prev_gn, NULL, 1.0f / c1, 1.0f / sqrtf(c2), q.lrmode, (unsigned long long)T2, q.adam, NULL, q.packed, 0, (int)q.ngrp);
+        qlmx_sync(NULL);
+        std::vector<signed char> wd_(nd), wr(nq), wm(nq), fd(nd), fr(nq), fm(nq);
+        qlmx_memcpy_d2h(wd_.data(), q.d, nd); qlmx_memcpy_d2h(wr.data(), q.r, nq); qlmx_memcpy_d2h(wm.data(), q.m8, nq);
+        int it2 = 0; float pg2 = 0; okf = okf && qlm_load(&q, path, &it2, &pg2);
+        float *part = (float *)dmalloc(64 * 3 * 4);
+        for(int si = 0; si < q.nspan; si++)
+            qlm_fused_spans(&q, Pd, Gd, si, 1, (size_t)q.spanH[si].gof, (size_t)q.spanH[si].n, part + 64 * si, lr, wd, T2, pg2);
+        qlmx_sync(NULL);
+        qlmx_memcpy_d2h(fd.data(), q.d, nd); qlmx_memcpy_d2h(fr.data(), q.r, nq); qlmx_memcpy_d2h(fm.data(), q.m8, nq);
+        check("qlm fused per-span step == whole step", (okf && !memcmp(wd_.data(), fd.data(), nd) && !memcmp(wr.data(), fr.data(), nq) && !memcmp(wm.data(), fm.data(), nq)) ? 0 : 1, 0);
+        double ss = 0; for(int si = 0; si < q.nspan; si++) for(unsigned long long i = 0; i < q.spanH[si].n; i++){ double g = Gh[q.spanH[si].gof + i]; ss += g * g; }
+        const float gn = qlm_fused_tail(part, 3, NULL, 0);
+        check("qlm fused grad norm rel-err", fabs((double)gn - sqrt(ss)) / sqrt(ss), 1e-6);
+    }
     remove(path);
 
     /* (d) expert forward through the grouped queue, weights addressed as P + offset */

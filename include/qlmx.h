@@ -104,6 +104,17 @@ int qlmx_step_touched(float *P, const float *Gc, signed char *d, signed char *r,
                       float inv_bc1, float inv_sqrt_bc2, unsigned long long t, unsigned long long nt,
                       const float *gs, int v4, void *stream);
 
+/* ---- gradient-norm clipping around the step: k_sqsum and k_gnorm (cudalm.cu:2794-2816; CPU twins
+ * cpu_kern.h:533-546), called from qlm_fused_layer / qlm_fused_tail (cudalm.cu:6122, 6181) and the
+ * unfused update (6435-6444). qlmx_sqsum writes 64 partial sums of squares, partial c over
+ * G[n*c/64 .. n*(c+1)/64), accumulated in double and rounded to float once (the CPU path's
+ * definition). qlmx_gnorm reduces them (plus `nside` further slices of 64) on the device to
+ * gs[0] = clip multiplier (1 when the norm is <= 1) and gs[1] = the norm, which qlmx_step reads
+ * through its `gsp` argument. ---- */
+int qlmx_sqsum(const float *G, unsigned long long n, float *part64, void *stream);
+int qlmx_gnorm(const float *part, int nside, int clip_side, float *gs, void *stream);
+
+
 /* ---- k_qlm_servo (qlm.cuh:404-441; launched from cudalm.cu:6099): rail-fraction scale servo
  * and re-encode of (d, r) for the groups whose scale moved. ---- */
 int qlmx_servo(signed char *d, signed char *r, float *s,

@@ -105,6 +105,8 @@ class Oracle(_Lib):
         self._swiglu = s("orc_swiglu", None, [c_vp, c_vp, c_vp, c_sz])
         self._swiglu_bwd = s("orc_swiglu_bwd", None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz])
         self._recip = s("orc_recip_div_mismatches", c_sz, [C.c_uint64, c_sz])
+        self._sqsum = s("orc_sqsum", None, [c_vp, C.c_uint64, c_vp])
+        self._gnorm = s("orc_gnorm", None, [c_vp, c_i, c_i, c_vp])
         self._step_touched = s("orc_step_touched", None, [c_vp] * 10 + [c_i, c_i, c_i, c_f, c_f, c_f, c_f, c_f, c_f, c_f,
                                                                        C.c_uint64, C.c_uint64, c_vp, c_i])
         self._q4n_q = s("orc_q4n_quantize", c_sz, [c_vp, c_sz, c_i, c_vp, c_sz, c_vp])
@@ -214,6 +216,16 @@ class Oracle(_Lib):
                            touched.size, group, dmax, lr, b1, b2, wd, sref, inv_bc1, inv_sqrt_bc2, t, nt,
                            _p(gs) if gs is not None else None, v4)
 
+    def sqsum(self, G):
+        part = np.zeros(64, np.float32)
+        self._sqsum(_p(G), G.size, _p(part))
+        return part
+
+    def gnorm(self, part, nside, clip_side):
+        gs = np.zeros(2, np.float32)
+        self._gnorm(_p(part), nside, clip_side, _p(gs))
+        return gs
+
     def recip_div_mismatches(self, seed, n):
         return int(self._recip(seed, n))
 
@@ -318,6 +330,8 @@ class Ref(_Lib):
                                                                  C.c_uint64, C.c_uint64, c_vp])
         self._q4n_d = s("ref_q4n_dequantize", c_i, [c_vp, c_sz, c_vp, c_sz, c_i])
         self._relerr = s("ref_relerr", c_f, [c_vp, c_vp, c_sz])
+        self._sqsum = s("ref_sqsum", None, [c_vp, C.c_uint64, c_vp])
+        self._gnorm = s("ref_gnorm", None, [c_vp, c_i, c_i, c_vp])
 
     def qd_get(self, d, i, packed):
         return self._qd_get(_p(d), i, packed)
@@ -399,6 +413,20 @@ def _ref_step_touched(self, P, Gc, d, r, s, m8, m8s, v8, v8s, touched, group, dm
                   _p(gs) if gs is not None else None)
 
 
+def _ref_sqsum(self, G):
+    part = np.zeros(64, np.float32)
+    self._sqsum(_p(G), G.size, _p(part))
+    return part
+
+
+def _ref_gnorm(self, part, nside, clip_side):
+    gs = np.zeros(2, np.float32)
+    self._gnorm(_p(part), nside, clip_side, _p(gs))
+    return gs
+
+
+Ref.sqsum = _ref_sqsum
+Ref.gnorm = _ref_gnorm
 Ref.step_touched = _ref_step_touched
 Ref.q4n_quantize = _ref_q4n_quantize
 Ref.q4n_dequantize = _ref_q4n_dequantize

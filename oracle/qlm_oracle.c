@@ -798,3 +798,22 @@ void orc_bf16_round_n(float *x, size_t n){
     #pragma omp parallel for schedule(static) if(n >= 65536)
     for(long i = 0; i < (long)n; i++) x[i] = orc_bf16_round(x[i]);
 }
+
+/* ---- gradient-norm clipping: k_sqsum and k_gnorm, cpu_kern.h:533-546 (GPU forms cudalm.cu:2794-2816) ---- */
+void orc_sqsum(const float *G, uint64_t n, float *part64){
+    for(int c = 0; c < 64; c++){
+        const uint64_t i0 = n * (uint64_t)c / 64, i1 = n * (uint64_t)(c + 1) / 64;
+        double s = 0.0;
+        for(uint64_t i = i0; i < i1; i++) s += (double)G[i] * G[i];
+        part64[c] = (float)s;
+    }
+}
+void orc_gnorm(const float *part, int nside, int clip_side, float *gs){
+    double ss = 0.0, sd = 0.0;
+    for(int i = 0; i < 64; i++) ss += part[i];
+    for(int i = 64; i < 64 * (1 + nside); i++) sd += part[i];
+    float gn = (float)sqrt(clip_side ? ss + sd : ss);
+    if(!isfinite(sd)) gn = NAN;
+    gs[0] = gn > 1.0f ? 1.0f / gn : 1.0f;
+    gs[1] = gn;
+}

@@ -55,6 +55,11 @@ void orc_step_touched(float *P, const float *Gc, int8_t *d, int8_t *r, const flo
                       uint8_t *v8, float *v8s, const int *touched_gi, int ntouched, int group, int dmax,
                       float lr, float b1, float b2, float wd, float sref, float inv_bc1, float inv_sqrt_bc2,
                       uint64_t t, uint64_t nt, const float *gs, int v4);
+/* cpu_kern.h:533-546: 64 chunk sums of squares (double accumulation, one rounding to float), and the clip
+ * multiplier / norm pair derived from them */
+void orc_sqsum(const float *G, uint64_t n, float *part64);
+void orc_gnorm(const float *part, int nside, int clip_side, float *gs);
+
 void orc_servo(int8_t *d, int8_t *r, float *s, const orc_span *sp, int nspan, int group, int dmax,
                float f_hi, float f_lo, int packed, int ngrp);
 

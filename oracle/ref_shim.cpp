@@ -70,6 +70,9 @@ void ref_ng_q4_step(float*P,const float*Gc,signed char*d,signed char*r,float*s,s
     KL(k_ng_q4_step,(unsigned)ntouched,group,group)(P,Gc,d,r,s,m8,m8s,v8,v8s,touched,group,dmax,
         lr,b1,b2,wd,sref,inv_bc1,inv_sqrt_bc2,t,nt,gs);
 }
+/* cudalm.cu:2794, 2811 through their CPU twins cpu_kern.h:533-546 */
+void ref_sqsum(const float*G,unsigned long long n,float*part){ KL(k_sqsum,64,TPB)(G,(size_t)n,part); }
+void ref_gnorm(const float*part,int nside,int clip_side,float*gs){ KL(k_gnorm,1,1)(part,nside,clip_side,gs); }
 void ref_servo(signed char*d,signed char*r,float*s,const QSpanD*sp,int nspan,int group,int dmax,
                float f_hi,float f_lo,int packed,int ngrp){
     KL(k_qlm_servo,(unsigned)ngrp,group,group)(d,r,s,sp,nspan,group,dmax,f_hi,f_lo,packed);

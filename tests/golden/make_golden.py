@@ -256,6 +256,24 @@ def golden_step_touched():
     save("step_touched", **out)
 
 
+def golden_gnorm():
+    """k_sqsum and k_gnorm (cpu_kern.h:533-546): the 64 partial sums of squares of three gradient
+    vectors (one shorter than 64, one not a multiple of 64, one large enough for a norm above 1) and
+    the clip multiplier / norm pairs with and without side slices."""
+    out = {}
+    for k, (n, scale) in enumerate([(50, 1e-3), (1000 * 3 + 7, 1e-2), (1 << 18, 3e-3)]):
+        G = gen.normal(n, 0, 970 + k, scale)
+        out["n%d" % k] = np.array([n]); out["seed%d" % k] = np.array([970 + k]); out["scale%d" % k] = np.array([scale], np.float64)
+        out["part%d" % k] = ref.sqsum(G)
+    side = np.concatenate([out["part2"], out["part1"], out["part0"]])
+    for cs in (0, 1):
+        out["gs_side%d" % cs] = ref.gnorm(side, 2, cs)
+    out["gs_small"] = ref.gnorm(out["part0"], 0, 0)
+    bad = side.copy(); bad[70] = np.inf
+    out["gs_inf"] = ref.gnorm(bad, 2, 0)
+    save("gnorm", **out)
+
+
 def golden_q4n():
     """q4n wire format (cudalm.cu:638-656): groups on the 4-bit grid (rendered QLM view), groups off
     the grid (stored raw), an all-zero group, a one-hot group and a short tail."""
@@ -279,6 +297,7 @@ def golden_q4n():
 
 
 if __name__ == "__main__":
+    golden_gnorm()
     golden_q4n()
     golden_step_touched()
     golden_hash()

@@ -186,6 +186,50 @@ def test_step_touched_vs_oracle_sparse_table(q, orc, v4):
         assert beq(got, want)
 
 
+def test_sqsum_gnorm_and_clipped_step(q, orc, golden):
+    """k_sqsum / k_gnorm (cudalm.cu:2794-2816 with the CPU kernels' definition, cpu_kern.h:533-546): the 64
+    partial sums against the reference fixture and the oracle (the double additions run in another
+    order on the GPU: at most one float ulp), the clip pair from the same partials bit for bit, and a step
+    that reads its clip multiplier from the device equal to the oracle's step with that multiplier."""
+    import torch
+    g = golden("gnorm")
+    parts = []
+    for k in range(3):
+        G = orc.normal(int(g["n%d" % k][0]), 0, int(g["seed%d" % k][0]), float(g["scale%d" % k][0]))
+        part = torch.zeros(64, device="cuda")
+        q.sqsum(dev(G), G.size, part)
+        got = host(part)
+        ulps = np.abs(got.view(np.int32).astype(np.int64) - g["part%d" % k].view(np.int32).astype(np.int64)).max()
+        assert ulps <= 1, (k, ulps)
+        parts.append(got)
+    side = np.concatenate([parts[2], parts[1], parts[0]])
+    gs = torch.zeros(2, device="cuda")
+    for cs in (0, 1):
+        q.gnorm(dev(side), 2, cs, gs)
+        assert np.array_equal(host(gs).view(np.uint32), orc.gnorm(side, 2, cs).view(np.uint32))
+    bad = side.copy(); bad[70] = np.inf
+    q.gnorm(dev(bad), 2, 0, gs)
+    assert np.isnan(host(gs)[1]) and host(gs)[0] == 1.0
+    # a step clipped through the device scalar
+    group, dmax = 128, 7
+    tab, nq, ng = make_spans([128 * 300 + 40], group)
+    tab["sref"] = [0.0088]
+    hd = orc.digits(nq, 5, 20); hr = orc.int8(nq, 5, 21, -64, 64); hm8 = orc.int8(nq, 5, 22, -127, 127); hv8 = orc.u8(nq, 5, 23, 0, 255)
+    hs = orc.uniform(ng, 5, 24, 0.5, 1.5) * f32(0.02 * 3 / 7)
+    hm8s = orc.uniform(ng, 5, 25, 0.5, 1.5) * f32(3e-3 / 127); hv8s = orc.uniform(ng, 5, 26, 0.5, 1.5) * f32(3e-3 / 255)
+    hG = orc.normal(nq, 5, 27, 0.05)                                   # norm well above 1
+    d, r, m8, v8, s, m8s, v8s, G = (dev(x) for x in (hd, hr, hm8, hv8, hs, hm8s, hv8s, hG))
+    part = torch.zeros(64, device="cuda")
+    q.sqsum(G, nq, part); q.gnorm(part, 0, 0, gs)
+    hgs = host(gs)
+    assert hgs[1] > 1.0 and hgs[0] == f32(1.0) / hgs[1]
+    hp = lambda gsp: (3e-4, 0.9, 0.95, 0.1, 1.0, gsp, 10.0, 4.4721, 0, 1, 1, None, 1, 0, ng)
+    q.step(None, G, d, r, s, m8, m8s, v8, v8s, dev(tab), 1, group, dmax, *hp(gs))
+    orc.step(None, hG, hd, hr, hs, hm8, hm8s, hv8, hv8s, tab, group, dmax, *hp(hgs[:1].copy()))
+    for got, want, nm in [(d, hd, "d"), (r, hr, "r"), (m8, hm8, "m8"), (v8, hv8, "v8"), (m8s, hm8s, "m8s"), (v8s, hv8s, "v8s")]:
+        assert beq(got, want), nm
+
+
 def test_argument_errors(q):
     import torch
     x = torch.zeros(256, device="cuda")

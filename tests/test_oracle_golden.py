@@ -475,3 +475,38 @@ def test_step_touched_equals_full_step_on_the_touched_groups(orc):
     for gi in untouched:
         sl = slice(gi * group, (gi + 1) * group)
         assert np.array_equal(a[1][sl], base[1][sl]) and np.array_equal(a[2][sl], base[2][sl])
+
+
+def _ulps(a, b):
+    return int(np.abs(a.view(np.int32).astype(np.int64) - b.view(np.int32).astype(np.int64)).max())
+
+
+def test_gnorm_vs_reference_fixture(orc, golden):
+    """k_sqsum / k_gnorm (cpu_kern.h:533-546): partial sums bit for bit (both sum a chunk in double in
+    index order and round once), clip multiplier and norm bit for bit, NaN norm for a non-finite side sum."""
+    g = golden("gnorm")
+    for k in range(3):
+        G = orc.normal(int(g["n%d" % k][0]), 0, int(g["seed%d" % k][0]), float(g["scale%d" % k][0]))
+        assert np.array_equal(orc.sqsum(G).view(np.uint32), g["part%d" % k].view(np.uint32)), k
+    side = np.concatenate([g["part2"], g["part1"], g["part0"]])
+    for cs in (0, 1):
+        assert np.array_equal(orc.gnorm(side, 2, cs).view(np.uint32), g["gs_side%d" % cs].view(np.uint32))
+    assert g["gs_side1"][1] > g["gs_side0"][1] > 1.0 and g["gs_side0"][0] < 1.0      # the fixture clips
+    assert np.array_equal(orc.gnorm(g["part0"], 0, 0), g["gs_small"]) and g["gs_small"][0] == 1.0
+    bad = side.copy(); bad[70] = np.inf
+    got = orc.gnorm(bad, 2, 0)
+    assert np.isnan(got[1]) and np.isnan(g["gs_inf"][1]) and got[0] == g["gs_inf"][0] == 1.0
+
+
+def test_sqsum_closed_forms(orc):
+    """Chunk c covers [n*c/64, n*(c+1)/64): with all ones the partials are the chunk lengths and add up
+    to n; with one non-zero element only its chunk is non-zero; the norm of (3, 4) is 5, clipped by 1/5."""
+    for n in (1, 63, 64, 65, 1000, 4097):
+        part = orc.sqsum(np.ones(n, f32))
+        want = np.array([n * (c + 1) // 64 - n * c // 64 for c in range(64)], f32)
+        assert np.array_equal(part, want) and part.sum() == n
+    G = np.zeros(640, f32); G[137] = 3.0; G[500] = -4.0
+    part = orc.sqsum(G)
+    assert part[13] == 9.0 and part[50] == 16.0 and part.sum() == 25.0
+    gs = orc.gnorm(part, 0, 0)
+    assert gs[1] == 5.0 and gs[0] == f32(1.0) / f32(5.0)

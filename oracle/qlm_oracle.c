@@ -17,6 +17,9 @@
  *                                             explicit FMA, so tolerance rather than bits) + ref lib
  *   q4n quantize/dequantize                   fixtures (byte-exact: grid groups, off-grid raw groups, an
  *                                             all-zero group, a short tail) + round trip + ref lib
+ *   sqsum / gnorm                             fixture written by the reference's k_sqsum / k_gnorm (bit-exact: chunk
+ *                                             sums in double, a clipping and a non-clipping norm, a non-finite
+ *                                             side sum) + closed forms (all ones, a 3-4-5 vector) + ref lib
  *   moe_forward/backward                      double-precision scalar expert FFN in the tests
  *                                             (cudalm.cu:10366-10387 style) + composition of ref lib calls
  * No function here is "parity unpinned".

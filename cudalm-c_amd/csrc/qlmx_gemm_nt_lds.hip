@@ -244,8 +244,9 @@ static int nt3_schedule(DevProb *pr, int n, int K, int N, int cus, DevUnit *unit
     for(int p = 0; p < n; p++){
         int nc = 1;
         if(pr[p].M > mean + mean / 4){ nc = (int)((pr[p].M + mean - 1) / mean); if(nc > 15) nc = 15; }
-        nchunk[p] = nc;
         chunk[p] = ((pr[p].M + nc - 1) / nc + NT3_BK - 1) / NT3_BK * NT3_BK;
+        nc = (pr[p].M + chunk[p] - 1) / chunk[p];                       /* rounding the slice up can make the last one empty */
+        nchunk[p] = nc;
         nunits += (long long)nc * rp * g;
     }
     if(nunits + 8LL * (long long)(rp * g * 15) > QLMX_MAX_UNITS) return 0;

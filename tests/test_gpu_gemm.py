@@ -200,6 +200,9 @@ def test_mfma_nt_split_contraction(q, orc, beta):
     # twice in a row: the flags of the first launch must not satisfy the second
     got2, want2 = run_case(q, orc, "nt", 4, [1700, 40, 0, 333], 256, 256, pkg.ACT_BF16, pkg.MATH_MFMA, seed=7, nt_beta=beta)
     assert orc.relerr(got2, want2) < TOL_MFMA
+    # as many slices as a chain holds (15), of a length that rounding up to whole steps changes
+    got3, want3 = run_case(q, orc, "nt", 2, [3841, 10], 64, 128, pkg.ACT_BF16, pkg.MATH_MFMA, seed=8, nt_beta=beta)
+    assert orc.relerr(got3, want3) < TOL_MFMA
 
 
 @pytest.mark.parametrize("mode", ["nn", "tn"])

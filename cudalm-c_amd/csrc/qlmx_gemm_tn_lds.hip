@@ -190,11 +190,12 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, int
         const uint32_t sbuf = lds_base + (uint32_t)(st & 1) * TN3_B_BYTES;
         const uint32_t wbuf = lds_base + (uint32_t)((st + 1) & 1) * TN3_B_BYTES;
         const int tile2 = st + 2 < steps ? st + 2 : steps - 1, stage2 = (st + 2) % TN3_A_STAGES;   /* past the end: the last one again, never used */
+        const bool fresh = st % spg == 0, last = (st + 1) % spg == 0;
         i32x4 wnext; float fn[2];
         i32x4 wv[4];
         auto item = [&](int k){
             if(k == 0)      wnext = tn3_gld16(pw + (size_t)tile2 * (TN3_BK / 2));
-            else if(k < 3)  fn[k - 1] = load_scale(st + 1, k - 1);
+            else if(k < 3){ if(last) fn[k - 1] = load_scale(st + 1, k - 1); else fn[k - 1] = fs_cur[k - 1]; }   /* a new scale only where a group ends */
             else if(k < 3 + 2 * NI)
                 __builtin_amdgcn_global_load_lds((glb_void *)(srcA[k - 3] + (size_t)tile2 * (TN3_BK * 2)),
                                                  (lds_void *)(lds + stage2 * TN3_A_BYTES + wave_off + (k - 3) * 4096), 16, 0, 0);
@@ -208,7 +209,6 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, int
                 } else tn3_wr(wbuf + wr_off[j], wv[j]);
             }
         };
-        const bool fresh = st % spg == 0, last = (st + 1) % spg == 0;
         Tn3Ops o[2];
         if(NI < 2){ o[0].a[1] = (i32x4)(0); o[1].a[1] = (i32x4)(0); }   /* the wait names both */
         o[0].a[0] = tn3_rd<0>(sa + ra[0]); if(NI > 1) o[0].a[1] = tn3_rd<32 * 128>(sa + ra[0]);

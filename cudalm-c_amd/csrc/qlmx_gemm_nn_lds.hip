@@ -12,9 +12,9 @@
  *     touching a register (lane l of a wave instruction lands at base + 16*l). Rows keep their order,
  *     4 pieces per row, piece ko of row r stored at position ko ^ ((r >> 2) & 3): conflict-free
  *     128-bit operand reads.
- *   Weights: a thread dequantises 8 columns of two contraction rows per step and writes each row's
- *     hi and lo halves as one 16-byte unit; the unit u of row k sits at u ^ 4*(k & 3) of that row's 16
- *     units. The rows stay in the matrix's own order (contraction index = row), and the MFMA operand
+ *   Weights: a thread loads 16 columns of one contraction row per step (8 bytes of digits, one scale),
+ *     dequantises them and writes the hi and lo halves as two 16-byte units each; the unit u of row k
+ *     sits at u ^ 4*(k & 3) of that row's 16 units. The rows stay in the matrix's own order (contraction index = row), and the MFMA operand
  *     -- 8 consecutive contraction elements of one column -- is two ds_read_b64_tr_b16 (within 16 lanes,
  *     lane i receives element i & 3 of the 8-byte pieces addressed by lanes 4v + (i >> 2), v = 0..3).
  *     The general kernel needs eight conflicting 4-byte stores per plane for the same transposition.
@@ -68,6 +68,11 @@ __device__ __forceinline__ int nn3_gld4(const void *p){
     asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
     return v;
 }
+__device__ __forceinline__ i32x2 nn3_gld8(const void *p){
+    i32x2 v;
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
 struct Nn3Ops { i32x4 a[4]; i32x2 bh[2][2], bl[2][2]; };
 __device__ __forceinline__ void nn3_wait(Nn3Ops &o){
     asm volatile("s_waitcnt lgkmcnt(0)"
@@ -110,24 +115,30 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int
             __builtin_amdgcn_global_load_lds((glb_void *)(srcA[h] + (size_t)tl * (NN3_BK * 2)), (lds_void *)(base + h * 4096), 16, 0, 0);
     };
 
-    /* ---- weights: thread = (contraction rows 2kp, 2kp+1; columns oc*8 .. +7) ---- */
-    const int oc = tid & 15, kp = tid >> 4;
-    const size_t e0 = (size_t)(2 * kp) * a.N + j0 + oc * 8;
-    const signed char *pw0 = a.d + ((P.wq + e0) >> 1), *pw1 = pw0 + (a.N >> 1);
-    const float *ps0 = a.s + P.wg + (e0 >> a.gshift), *ps1 = a.s + P.wg + ((e0 + a.N) >> a.gshift);
+    /* ---- weights: thread = (contraction row kr, columns oc*16 .. +15): one 8-byte load of digits and
+     * one scale per step. The two 16-byte units it writes per plane are taken in opposite order by even
+     * and odd rows, so that the 16 lanes of a write phase (two rows) hit 16 different units. ---- */
+    const int oc = tid & 7, kr = tid >> 3, odd = kr & 1;
+    const size_t e0 = (size_t)kr * a.N + j0 + oc * 16;
+    const signed char *pw = a.d + ((P.wq + e0) >> 1);
+    const float *ps = a.s + P.wg + (e0 >> a.gshift);
     const size_t wstep = (size_t)NN3_BK * a.N >> 1, sstep = (size_t)NN3_BK * a.N >> a.gshift;
-    /* unit oc of row k at oc ^ 4*(k & 3); rows 2kp and 2kp+1 */
-    const uint32_t wr0 = NN3_B_OFF + (uint32_t)((2 * kp) * 256 + ((oc ^ (((2 * kp) & 3) << 2)) << 4));
-    const uint32_t wr1 = NN3_B_OFF + (uint32_t)((2 * kp + 1) * 256 + ((oc ^ (((2 * kp + 1) & 3) << 2)) << 4));
-    struct WLoad { int d0, d1, s0, s1; };
+    /* unit u of row k at u ^ 4*(k & 3) */
+    const int sw = (kr & 3) << 2;
+    const uint32_t wr0 = NN3_B_OFF + (uint32_t)(kr * 256 + (((2 * oc + odd) ^ sw) << 4));        /* written first  */
+    const uint32_t wr1 = NN3_B_OFF + (uint32_t)(kr * 256 + (((2 * oc + 1 - odd) ^ sw) << 4));    /* written second */
+    struct WLoad { i32x2 d; int s; };
     auto load_w = [&](int tile) -> WLoad {
         const size_t tl = (size_t)(tile < steps ? tile : steps - 1);      /* past the end: re-read the last one, never used */
         WLoad w;
-        w.d0 = nn3_gld4(pw0 + tl * wstep); w.d1 = nn3_gld4(pw1 + tl * wstep);
-        w.s0 = nn3_gld4(ps0 + tl * sstep); w.s1 = nn3_gld4(ps1 + tl * sstep);
+        w.d = nn3_gld8(pw + tl * wstep); w.s = nn3_gld4(ps + tl * sstep);
         return w;
     };
-    auto dequant_row = [&](uint32_t digits, float sc, i32x4 &hi, i32x4 &lo){
+    /* digits of the unit written first / second */
+    auto unit_digits = [&](const WLoad &w, int which) -> uint32_t {
+        return (uint32_t)((which ^ odd) ? w.d[1] : w.d[0]);
+    };
+    auto dequant_unit = [&](uint32_t digits, float sc, i32x4 &hi, i32x4 &lo){
         float w[8];
 #pragma unroll
         for(int j = 0; j < 8; j++) w[j] = sc * (float)qx_nib(digits, j);
@@ -141,9 +152,9 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int
     auto store_w = [&](const WLoad &w, int buf){
         const uint32_t bb = lds_base + buf * NN3_B_BYTES;
         i32x4 hi, lo;
-        dequant_row((uint32_t)w.d0, __int_as_float(w.s0), hi, lo);
+        dequant_unit(unit_digits(w, 0), __int_as_float(w.s), hi, lo);
         nn3_wr128<0>(bb + wr0, hi); nn3_wr128<NN3_P_BYTES>(bb + wr0, lo);
-        dequant_row((uint32_t)w.d1, __int_as_float(w.s1), hi, lo);
+        dequant_unit(unit_digits(w, 1), __int_as_float(w.s), hi, lo);
         nn3_wr128<0>(bb + wr1, hi); nn3_wr128<NN3_P_BYTES>(bb + wr1, lo);
     };
 
@@ -180,8 +191,7 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int
         wcur = load_w(1);
         issue_a(0, 0);
         issue_a(1, 1);
-        asm volatile("s_waitcnt vmcnt(%8)" : "+v"(w0.d0), "+v"(w0.d1), "+v"(w0.s0), "+v"(w0.s1),
-                                              "+v"(wcur.d0), "+v"(wcur.d1), "+v"(wcur.s0), "+v"(wcur.s1) : "n"(2 * NI) : "memory");
+        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(w0.d), "+v"(w0.s), "+v"(wcur.d), "+v"(wcur.s) : "n"(2 * NI) : "memory");
         store_w(w0, 0);
     }
 
@@ -191,12 +201,12 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int
      * MFMA of a step runs alone. Everything else of a step is therefore cut into small items and
      * dealt evenly into the gaps after the MFMAs of both slices, fences keeping the compiler
      * from gathering them again:
-     *   the four loads of the weights of step st+2 (into wnext, waited for at the end of the step,
+     *   the two loads of the weights of step st+2 (into wnext, waited for at the end of the step,
      *     when they have long arrived: an asynchronously loaded register must not be carried round
      *     the loop before its wait), the activation requests of tile st+2,
      *   the dequantisation of the weights of step st+1 (wcur), two weights per pair of items,
      *   their four LDS writes into the buffer last read in step st-1. */
-    constexpr int SLOTS = NI * 8, ITEMS = 4 + NI + 16 + 4;
+    constexpr int SLOTS = NI * 8, ITEMS = 2 + NI + 16 + 4;
     for(int st = 0; st < steps; st++){
         /* tile st is in, own LDS writes are done; tile st+1 may still be on its way */
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"(NI) : "memory");
@@ -209,27 +219,26 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int
         WLoad wnext;
         i32x4 whi[2], wlo[2];
         float wf[8][2];
+        uint32_t dg[2];
+        const float sc = __int_as_float(wcur.s);
         auto item = [&](int k){
-            if(k == 0)      wnext.d0 = nn3_gld4(pw0 + (size_t)tile2 * wstep);
-            else if(k == 1) wnext.d1 = nn3_gld4(pw1 + (size_t)tile2 * wstep);
-            else if(k == 2) wnext.s0 = nn3_gld4(ps0 + (size_t)tile2 * sstep);
-            else if(k == 3) wnext.s1 = nn3_gld4(ps1 + (size_t)tile2 * sstep);
-            else if(k < 4 + NI)
-                __builtin_amdgcn_global_load_lds((glb_void *)(srcA[k - 4] + (size_t)tile2 * (NN3_BK * 2)),
-                                                 (lds_void *)(lds + stage2 * NN3_A_BYTES + wave_off + (k - 4) * 4096), 16, 0, 0);
-            else if(k < 4 + NI + 16){
-                const int q = k - 4 - NI, p = q >> 1, r = p >> 2, j = p & 3;
+            if(k == 0)      wnext.d = nn3_gld8(pw + (size_t)tile2 * wstep);
+            else if(k == 1) wnext.s = nn3_gld4(ps + (size_t)tile2 * sstep);
+            else if(k < 2 + NI)
+                __builtin_amdgcn_global_load_lds((glb_void *)(srcA[k - 2] + (size_t)tile2 * (NN3_BK * 2)),
+                                                 (lds_void *)(lds + stage2 * NN3_A_BYTES + wave_off + (k - 2) * 4096), 16, 0, 0);
+            else if(k < 2 + NI + 16){
+                const int q = k - 2 - NI, p = q >> 1, r = p >> 2, j = p & 3;
+                if(q == 0){ dg[0] = unit_digits(wcur, 0); dg[1] = unit_digits(wcur, 1); }
                 if((q & 1) == 0){
-                    const uint32_t dg = (uint32_t)(r ? wcur.d1 : wcur.d0);
-                    const float sc = __int_as_float(r ? wcur.s1 : wcur.s0);
-                    wf[p][0] = sc * (float)qx_nib(dg, 2 * j); wf[p][1] = sc * (float)qx_nib(dg, 2 * j + 1);
+                    wf[p][0] = sc * (float)qx_nib(dg[r], 2 * j); wf[p][1] = sc * (float)qx_nib(dg[r], 2 * j + 1);
                 } else {
                     const uint32_t h = nn3_pk(wf[p][0], wf[p][1]);
                     whi[r][j] = (int)h;
                     wlo[r][j] = (int)nn3_pk(wf[p][0] - __uint_as_float(h << 16), wf[p][1] - __uint_as_float(h & 0xFFFF0000u));
                 }
             } else {
-                const int w = k - 4 - NI - 16;
+                const int w = k - 2 - NI - 16;
                 if(w == 0)      nn3_wr128<0>(wbuf + wr0, whi[0]);
                 else if(w == 1) nn3_wr128<NN3_P_BYTES>(wbuf + wr0, wlo[0]);
                 else if(w == 2) nn3_wr128<0>(wbuf + wr1, whi[1]);
@@ -274,7 +283,7 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int
 #undef NN3_READ
 #undef NN3_MMA
         /* the weights of step st+2 have arrived (only the activation requests are younger) */
-        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(wnext.d0), "+v"(wnext.d1), "+v"(wnext.s0), "+v"(wnext.s1) : "n"(NI) : "memory");
+        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(wnext.d), "+v"(wnext.s) : "n"(NI) : "memory");
         wcur = wnext;
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);                    /* vmcnt(0), as a builtin so that the compiler knows it: no request may outlive the workgroup's LDS */

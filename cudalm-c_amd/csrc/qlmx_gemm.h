@@ -174,14 +174,14 @@ __device__ __forceinline__ void qx_store_tiles(const qx_f32x16 (&acc)[NI][NJ], f
     else                           qx_store_tiles_edge<NI, NJ, SYS>(acc, (qx_gfloat *)c, row, rows, ld, accumulate);
 }
 
-/* ---- scheduled launches: instead of deriving its tile from its index, workgroup b reads unit b of a
- * table the host has laid out -- which problem, which output tile, which slice of the contraction
- * (a table of up to 16 KB together with the problems travels about 12 us faster than a larger one,
- * hence the packing). Slices of one output tile form a chain: slice seq waits until flag holds
+/* ---- scheduled launches: instead of deriving its tile from its index, a workgroup reads an entry of
+ * a table the host has laid out -- which problem, which row of output tiles, which slice of the
+ * contraction; the workgroups that share an entry take one column tile each (a table of up to 16 KB
+ * together with the problems travels about 12 us faster than a larger one, hence the packing). Slices of one output tile form a chain: slice seq waits until flag holds
  * (epoch << 4 | seq), adds its product to what is there and publishes seq + 1. A slice always sits at
  * a higher workgroup index than its predecessor, and workgroups start in index order, so whatever a
  * resident workgroup waits for is resident or done; the wait is bounded all the same. ---- */
-typedef uint32_t DevUnit;                 /* prob:10 | tile row:6 | tile column:8 | seq:4 | nseq:4; all ones = nothing to do */
+typedef uint32_t DevUnit;                 /* prob:10 | tile row:6 | (8 spare) | seq:4 | nseq:4; all ones = nothing to do */
 #define QX_UNIT_NONE 0xFFFFFFFFu
 #define QX_UNIT(prob, ti, tj, seq, nseq) ((uint32_t)(prob) << 22 | (uint32_t)(ti) << 16 | (uint32_t)(tj) << 8 | (uint32_t)(seq) << 4 | (uint32_t)(nseq))
 #define QLMX_MAX_UNITS 16384

@@ -87,7 +87,9 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
     int pi, i0, j0, k0 = 0, depth = -1, seq = 0, nseq = 1, flag = 0;
     DevUnit u = QX_UNIT_NONE;
     if(a.units){
-        u = a.units[blockIdx.x];
+        /* one table entry per strip of tiles_n column tiles: workgroup 8k + x is column tile k % tiles_n
+         * of entry k / tiles_n of XCD x */
+        u = a.units[((blockIdx.x >> 3) / a.tiles_n) * 8 + (blockIdx.x & 7)];
         if(u == QX_UNIT_NONE) return;
         pi = (int)(u >> 22);
     } else {
@@ -97,7 +99,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
     }
     const DevProb P = a.pr[pi];
     if(a.units){
-        const int ti = (u >> 16) & 63, tj = (u >> 8) & 255;
+        const int ti = (u >> 16) & 63, tj = (int)(blockIdx.x >> 3) % a.tiles_n;
         seq = (u >> 4) & 15; nseq = u & 15;
         i0 = ti * NT3_BM; j0 = tj * NT3_BN; k0 = seq * P.chunk;
         depth = P.M - k0 < P.chunk ? P.M - k0 : P.chunk;
@@ -228,12 +230,13 @@ static void *g_nt3_zeros = nullptr;
  * cost is its row count, so a Zipf-loaded layer has a few tiles that outlast all others: contractions
  * longer than about the mean load of a workgroup slot are cut into slices that add up through a
  * chain. Groups (problem, tile row) -- the tiles that share the activation slab -- are dealt to the
- * XCDs heaviest first, each to the XCD with the least work so far; workgroup 8k + x is the k-th unit
- * of XCD x. Returns the grid size, or 0 when the launch does not fit the table. */
+ * XCDs heaviest first, each to the XCD with the least work so far. A table entry stands for the g
+ * column tiles of one (problem, tile row, slice); XCD x runs its entries in order, g workgroups each.
+ * Returns the grid size, or 0 when the launch does not fit the table. */
 struct Nt3Group { int prob, ti, cost; };
-static int nt3_schedule(DevProb *pr, int n, int K, int N, int cus, DevUnit *units, int *nflags_out){
+static int nt3_schedule(DevProb *pr, int n, int K, int N, int cus, DevUnit *units, int *nflags_out, int *nent_out){
     const int g = N / NT3_BN, rp = (K + NT3_BM - 1) / NT3_BM;
-    if(g > 256 || rp > 64) return 0;                                   /* the packed unit has 8 and 6 bits for them */
+    if(rp > 64) return 0;                                              /* the packed entry has 6 bits for the tile row */
     long long work = 0;
     for(int p = 0; p < n; p++) work += (long long)pr[p].M * rp * g;
     const long long slots = 2LL * cus;
@@ -247,9 +250,9 @@ static int nt3_schedule(DevProb *pr, int n, int K, int N, int cus, DevUnit *unit
         chunk[p] = ((pr[p].M + nc - 1) / nc + NT3_BK - 1) / NT3_BK * NT3_BK;
         nc = (pr[p].M + chunk[p] - 1) / chunk[p];                       /* rounding the slice up can make the last one empty */
         nchunk[p] = nc;
-        nunits += (long long)nc * rp * g;
+        nunits += (long long)nc * rp;
     }
-    if(nunits + 8LL * (long long)(rp * g * 15) > QLMX_MAX_UNITS) return 0;
+    if(nunits + 8LL * 15 > QLMX_MAX_UNITS) return 0;
     static Nt3Group groups[QLMX_MAX_UNITS];
     int ng = 0;
     for(int p = 0; p < n; p++) for(int ti = 0; ti < rp; ti++) groups[ng++] = {p, ti, pr[p].M};
@@ -259,13 +262,13 @@ static int nt3_schedule(DevProb *pr, int n, int K, int N, int cus, DevUnit *unit
     for(int i = 0; i < ng; i++){
         int x = 0;
         for(int y = 1; y < 8; y++) if(load[y] < load[x]) x = y;
-        gx[i] = x; load[x] += (long long)groups[i].cost * g; len[x] += nchunk[groups[i].prob] * g;
+        gx[i] = x; load[x] += (long long)groups[i].cost * g; len[x] += nchunk[groups[i].prob];
     }
     int longest = 0;
     for(int x = 0; x < 8; x++) if(len[x] > longest) longest = len[x];
-    const int grid = 8 * longest;
-    if(grid > QLMX_MAX_UNITS) return 0;
-    for(int b = 0; b < grid; b++) units[b] = QX_UNIT_NONE;
+    const int nent = 8 * longest;                                      /* table entries; each stands for g workgroups */
+    if(nent > QLMX_MAX_UNITS || (long long)nent * g >= (1LL << 30)) return 0;
+    for(int b = 0; b < nent; b++) units[b] = QX_UNIT_NONE;
     int nflags = 0;
     for(int p = 0; p < n; p++){
         pr[p].chunk = chunk[p]; pr[p].flag0 = nflags;
@@ -274,11 +277,11 @@ static int nt3_schedule(DevProb *pr, int n, int K, int N, int cus, DevUnit *unit
     int pos[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     for(int i = 0; i < ng; i++){
         const int p = groups[i].prob, x = gx[i], nc = nchunk[p];
-        for(int tj = 0; tj < g; tj++)
-            for(int c = 0; c < nc; c++) units[8 * pos[x]++ + x] = QX_UNIT(p, groups[i].ti, tj, c, nc);
+        for(int c = 0; c < nc; c++) units[8 * pos[x]++ + x] = QX_UNIT(p, groups[i].ti, 0, c, nc);
     }
     *nflags_out = nflags;
-    return grid;
+    *nent_out = nent;
+    return nent * g;
 }
 
 /* bf16 operands only; N % 128 == 0, K % 8 == 0, operands 16-byte aligned (checked by the caller) */
@@ -305,15 +308,15 @@ int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N
                 DevProb &q = uu.hprob[n++];
                 q.A = p.A; q.B = p.B; q.C = p.C; q.wq = 0; q.wg = 0; q.M = p.M; q.beta = p.beta; q.tile0 = 0; q.tiles_n = N / NT3_BN;
             }
-            int nflags = 0;
-            const int grid = nt3_schedule(uu.hprob, n, K, N, qlmx_cu_count(), uu.hunit, &nflags);
+            int nflags = 0, nent = 0;
+            const int grid = nt3_schedule(uu.hprob, n, K, N, qlmx_cu_count(), uu.hunit, &nflags, &nent);
             if(grid > 0){
                 Nt3Args a; a.pr = uu.dprob; a.units = uu.dunit; a.flags = uu.flags; a.status = uu.status;
                 a.nprob = n; a.ntiles = grid; a.tiles_n = N / NT3_BN; a.rows_p = 1; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
                 int first = 0; a.epoch = 0;
                 if(nflags){ rc = qlmx_chain_reserve(nflags, &first, &a.epoch); if(rc) return rc; }
                 for(int p = 0; p < n; p++) uu.hprob[p].flag0 += first;
-                rc = qlmx_unit_commit(uslot, n, grid, st); if(rc) return rc;
+                rc = qlmx_unit_commit(uslot, n, nent, st); if(rc) return rc;
                 hipLaunchKernelGGL(k_gemm_nt_lds, dim3(grid), dim3(256), 0, st, a);
                 QLMX_LAUNCH_CHECK("grouped gemm nt (scheduled) launch");
                 return qlmx_unit_done(uslot, st);

@@ -1,5 +1,5 @@
 /* qlmx_gemm.h -- shared plumbing of the grouped expert GEMMs: the device problem record, the
- * pinned upload ring (the counterpart of the reference's mg_h/mg_d ring, cudalm.cu:3220-3241) and
+ * pinned table ring (the counterpart of the reference's mg_h/mg_d ring, cudalm.cu:3220-3241) and
  * the weight-tile readers. */
 #ifndef QLMX_GEMM_H
 #define QLMX_GEMM_H
@@ -17,9 +17,9 @@ struct DevProb {
     int flag0;              /*   and the chain flag of the problem's first tile      */
 };
 
-/* Copies `nprob` problems into the next ring slot, fills tile0/tiles_n with the given tile shape
- * over an output of rows_of(p) x ncols, uploads the slot asynchronously on `stream`, and returns
- * the device pointer and the total tile count. Slots are guarded by events, so a slot is never
+/* Writes `nprob` problems into the next slot of a ring in pinned host memory, fills tile0/tiles_n with
+ * the given tile shape over an output of rows_of(p) x ncols, and returns the pointer the kernel reads
+ * the table through and the total tile count. Slots are guarded by events, so a slot is never
  * rewritten while a kernel launched with it may still read it. */
 struct ProbUpload { const DevProb *dev; int ntiles; int nprob; };
 int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K, int N,
@@ -94,7 +94,7 @@ template<bool SYS> __device__ __forceinline__ float qx_gld_f32(const qx_gfloat *
 }
 template<bool SYS> __device__ __forceinline__ void qx_gst_f32(qx_gfloat *p, float v){
     if(SYS) asm volatile("global_store_dword %0, %1, off sc0 sc1" :: "v"(p), "v"(v) : "memory");
-    else    *p = v;
+    else    __builtin_nontemporal_store(v, p);
 }
 /* at most N younger memory operations may still be in flight; names the 16 values it guards */
 template<int N> __device__ __forceinline__ void qx_wait_old(float (&o)[16]){
@@ -176,8 +176,8 @@ __device__ __forceinline__ void qx_store_tiles(const qx_f32x16 (&acc)[NI][NJ], f
 
 /* ---- scheduled launches: instead of deriving its tile from its index, a workgroup reads an entry of
  * a table the host has laid out -- which problem, which row of output tiles, which slice of the
- * contraction; the workgroups that share an entry take one column tile each (a table of up to 16 KB
- * together with the problems travels about 12 us faster than a larger one, hence the packing). Slices of one output tile form a chain: slice seq waits until flag holds
+ * contraction; the workgroups that share an entry take one column tile each, which keeps the table
+ * to a few hundred bytes. Slices of one output tile form a chain: slice seq waits until flag holds
  * (epoch << 4 | seq), adds its product to what is there and publishes seq + 1. A slice always sits at
  * a higher workgroup index than its predecessor, and workgroups start in index order, so whatever a
  * resident workgroup waits for is resident or done; the wait is bounded all the same. ---- */
@@ -187,8 +187,7 @@ typedef uint32_t DevUnit;                 /* prob:10 | tile row:6 | (8 spare) | 
 #define QLMX_MAX_UNITS 16384
 #define QX_CHAIN_SPINS (1 << 22)
 struct UnitUpload { DevProb *hprob; DevUnit *hunit; const DevProb *dprob; const DevUnit *dunit; int *flags; unsigned *status; };
-int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot);                         /* host tables to fill; waits for the slot's last user */
-int qlmx_unit_commit(int slot, int nprob, int nunits, hipStream_t stream);         /* copies them to the device, asynchronously */
+int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot);                         /* tables to fill (pinned, read by the kernel); waits for the slot's last user */
 int qlmx_unit_done(int slot, hipStream_t stream);                                  /* after the kernel launch */
 int qlmx_chain_reserve(int nflags, int *first, unsigned *epoch);                   /* flags for one launch */
 

@@ -1,10 +1,17 @@
-/* qlmx_gemm_common.hip -- problem-table upload ring and argument checks of the grouped GEMMs. */
+/* qlmx_gemm_common.hip -- problem-table rings and argument checks of the grouped GEMMs.
+ *
+ * The tables of a launch (problems, and for scheduled launches the unit table) are written into a slot
+ * of a ring in pinned host memory and the kernels read them from there: a few KB, fetched once per
+ * XCD and served from cache afterwards. Copying them to device memory first put a 4 us copy kernel
+ * and its dependency in front of every launch (20 us of a 1 ms training step). A slot is handed out
+ * again only after the host has waited for the event recorded behind the kernel that last read it.
+ * Because the slots are rewritten, launches that use them must not be captured into a HIP graph. */
 #include "qlmx_gemm.h"
 #include <string.h>
 #include <algorithm>
 
 #define RING_SLOTS 64
-static DevProb   *g_ring_h = nullptr, *g_ring_d = nullptr;
+static DevProb   *g_ring_h = nullptr;
 static hipEvent_t g_ring_ev[RING_SLOTS];
 static bool       g_ring_used[RING_SLOTS];
 static int        g_ring_next = 0;
@@ -13,7 +20,6 @@ static int ring_init(void){
     if(g_ring_h) return QLMX_OK;
     const size_t bytes = (size_t)RING_SLOTS * QLMX_MAX_PROBLEMS * sizeof(DevProb);
     QLMX_HIP(hipHostMalloc((void **)&g_ring_h, bytes, hipHostMallocDefault), "problem ring (pinned)");
-    QLMX_HIP(hipMalloc((void **)&g_ring_d, bytes), "problem ring (device)");
     for(int i = 0; i < RING_SLOTS; i++){
         QLMX_HIP(hipEventCreateWithFlags(&g_ring_ev[i], hipEventDisableTiming), "problem ring event");
         g_ring_used[i] = false;
@@ -32,7 +38,6 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
     const int slot = g_ring_next; g_ring_next = (g_ring_next + 1) % RING_SLOTS;
     if(g_ring_used[slot]) QLMX_HIP(hipEventSynchronize(g_ring_ev[slot]), "problem ring wait");
     DevProb *h = g_ring_h + (size_t)slot * QLMX_MAX_PROBLEMS;
-    DevProb *dv = g_ring_d + (size_t)slot * QLMX_MAX_PROBLEMS;
     const int tiles_n = (N + tile_cols - 1) / tile_cols;
     long long tiles = 0; int n = 0;
     /* Weight gradients: every problem has the same number of tiles but a cost proportional to its
@@ -67,8 +72,8 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
         tiles += (long long)((rows + tile_rows - 1) / tile_rows) * tiles_n;
         QLMX_REQUIRE(tiles < (1LL << 30), "grouped gemm: too many tiles");
     }
-    if(n) QLMX_HIP(hipMemcpyAsync(dv, h, (size_t)n * sizeof(DevProb), hipMemcpyHostToDevice, stream), "problem table h2d");
-    out->dev = dv; out->ntiles = (int)tiles; out->nprob = n;
+    (void)stream;
+    out->dev = h; out->ntiles = (int)tiles; out->nprob = n;
     *slot_out = slot;
     return QLMX_OK;
 }
@@ -79,12 +84,12 @@ int qlmx_upload_done(int slot, hipStream_t stream){
     return QLMX_OK;
 }
 
-/* ---- unit tables of scheduled launches: a ring of pinned/device slot pairs like the one above, each
- * holding a problem table and a unit table; chain flags handed out round the ring of a fixed array
+/* ---- unit tables of scheduled launches: a ring of pinned slots like the one above, each holding a
+ * problem table and a unit table; chain flags handed out round the ring of a fixed array
  * (a launch's flags carry its epoch, so nothing is ever cleared). ---- */
 #define UNIT_SLOTS 32
 #define CHAIN_FLAGS (1 << 18)
-static char      *g_unit_h = nullptr, *g_unit_d = nullptr;
+static char      *g_unit_h = nullptr;
 static hipEvent_t g_unit_ev[UNIT_SLOTS];
 static bool       g_unit_used[UNIT_SLOTS];
 static int        g_unit_next = 0;
@@ -94,13 +99,12 @@ static int        g_chain_cursor = 0;
 static unsigned   g_chain_epoch = 0;
 static const size_t UNIT_SLOT_BYTES = (size_t)QLMX_MAX_PROBLEMS * sizeof(DevProb) + (size_t)QLMX_MAX_UNITS * sizeof(DevUnit);
 
-/* the unit table follows the problem table, so that one copy moves both */
+/* the unit table follows the problem table */
 static size_t unit_offset(int nprob){ return ((size_t)nprob * sizeof(DevProb) + 63) & ~(size_t)63; }
 
 static int unit_init(void){
     if(g_unit_h) return QLMX_OK;
     QLMX_HIP(hipHostMalloc((void **)&g_unit_h, UNIT_SLOTS * UNIT_SLOT_BYTES, hipHostMallocDefault), "unit ring (pinned)");
-    QLMX_HIP(hipMalloc((void **)&g_unit_d, UNIT_SLOTS * UNIT_SLOT_BYTES), "unit ring (device)");
     QLMX_HIP(hipMalloc((void **)&g_chain_flags, CHAIN_FLAGS * sizeof(int)), "chain flags");
     QLMX_HIP(hipMemset(g_chain_flags, 0, CHAIN_FLAGS * sizeof(int)), "chain flags clear");
     QLMX_HIP(hipHostMalloc((void **)&g_chain_status, sizeof(unsigned), hipHostMallocDefault), "chain status (pinned)");
@@ -120,18 +124,12 @@ int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot_out){
     }
     const int slot = g_unit_next; g_unit_next = (g_unit_next + 1) % UNIT_SLOTS;
     if(g_unit_used[slot]) QLMX_HIP(hipEventSynchronize(g_unit_ev[slot]), "unit ring wait");
-    char *h = g_unit_h + slot * UNIT_SLOT_BYTES, *d = g_unit_d + slot * UNIT_SLOT_BYTES;
+    char *h = g_unit_h + slot * UNIT_SLOT_BYTES;
     const size_t uoff = unit_offset(nprob);
     out->hprob = (DevProb *)h; out->hunit = (DevUnit *)(h + uoff);
-    out->dprob = (const DevProb *)d; out->dunit = (const DevUnit *)(d + uoff);
+    out->dprob = (const DevProb *)h; out->dunit = (const DevUnit *)(h + uoff);
     out->flags = g_chain_flags; out->status = g_chain_status;
     *slot_out = slot;
-    return QLMX_OK;
-}
-
-int qlmx_unit_commit(int slot, int nprob, int nunits, hipStream_t stream){
-    char *h = g_unit_h + slot * UNIT_SLOT_BYTES, *d = g_unit_d + slot * UNIT_SLOT_BYTES;
-    QLMX_HIP(hipMemcpyAsync(d, h, unit_offset(nprob) + (size_t)nunits * sizeof(DevUnit), hipMemcpyHostToDevice, stream), "problem and unit tables h2d");
     return QLMX_OK;
 }
 

@@ -316,7 +316,6 @@ int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N
                 int first = 0; a.epoch = 0;
                 if(nflags){ rc = qlmx_chain_reserve(nflags, &first, &a.epoch); if(rc) return rc; }
                 for(int p = 0; p < n; p++) uu.hprob[p].flag0 += first;
-                rc = qlmx_unit_commit(uslot, n, nent, st); if(rc) return rc;
                 hipLaunchKernelGGL(k_gemm_nt_lds, dim3(grid), dim3(256), 0, st, a);
                 QLMX_LAUNCH_CHECK("grouped gemm nt (scheduled) launch");
                 return qlmx_unit_done(uslot, st);

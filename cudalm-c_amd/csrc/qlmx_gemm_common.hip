@@ -4,26 +4,62 @@
  * of a ring in pinned host memory and the kernels read them from there: a few KB, fetched once per
  * XCD and served from cache afterwards. Copying them to device memory first put a 4 us copy kernel
  * and its dependency in front of every launch (20 us of a 1 ms training step). A slot is handed out
- * again only after the host has waited for the event recorded behind the kernel that last read it.
+ * again only after the host has waited for an event recorded behind the kernel that last read it.
  * Because the slots are rewritten, launches that use them must not be captured into a HIP graph. */
 #include "qlmx_gemm.h"
 #include <string.h>
 #include <algorithm>
 
+/* Reuse guard of a ring: an event behind every launch costs about 6 us of idle GPU between that kernel
+ * and the next (the record makes the end of the kernel visible to the host), so the slots are guarded
+ * by segments instead: when the last slot of a segment has been launched, one event is recorded on
+ * each stream the segment's launches went to, and those events are waited for when the ring comes
+ * round to the segment's first slot again -- three segments' worth of launches later. */
+#define GUARD_STREAMS 4
+struct RingSeg { hipStream_t st[GUARD_STREAMS]; hipEvent_t ev[GUARD_STREAMS]; int nst, nrec; bool made; };
+struct RingGuard { int nslots, per_seg, next; RingSeg seg[8]; };
+
+static int guard_take(RingGuard &g, int *slot_out){
+    const int slot = g.next; g.next = (g.next + 1) % g.nslots;
+    RingSeg &sg = g.seg[slot / g.per_seg];
+    if(slot % g.per_seg == 0){
+        for(int i = 0; i < sg.nrec; i++) QLMX_HIP(hipEventSynchronize(sg.ev[i]), "table ring wait");
+        sg.nrec = 0; sg.nst = 0;
+    }
+    *slot_out = slot;
+    return QLMX_OK;
+}
+static int guard_launched(RingGuard &g, int slot, hipStream_t stream){
+    RingSeg &sg = g.seg[slot / g.per_seg];
+    if(!sg.made){
+        for(int i = 0; i < GUARD_STREAMS; i++) QLMX_HIP(hipEventCreateWithFlags(&sg.ev[i], hipEventDisableTiming), "table ring event");
+        sg.made = true;
+    }
+    int k = 0;
+    while(k < sg.nst && sg.st[k] != stream) k++;
+    if(k == sg.nst){
+        if(sg.nst == GUARD_STREAMS){
+            /* more streams than events in one segment: wait for this one now */
+            QLMX_HIP(hipStreamSynchronize(stream), "table ring stream wait");
+            return QLMX_OK;
+        }
+        sg.st[sg.nst++] = stream;
+    }
+    if(slot % g.per_seg == g.per_seg - 1){
+        for(int i = 0; i < sg.nst; i++) QLMX_HIP(hipEventRecord(sg.ev[i], sg.st[i]), "table ring record");
+        sg.nrec = sg.nst;
+    }
+    return QLMX_OK;
+}
+
 #define RING_SLOTS 64
 static DevProb   *g_ring_h = nullptr;
-static hipEvent_t g_ring_ev[RING_SLOTS];
-static bool       g_ring_used[RING_SLOTS];
-static int        g_ring_next = 0;
+static RingGuard  g_ring_guard = {RING_SLOTS, 16, 0, {}};
 
 static int ring_init(void){
     if(g_ring_h) return QLMX_OK;
     const size_t bytes = (size_t)RING_SLOTS * QLMX_MAX_PROBLEMS * sizeof(DevProb);
     QLMX_HIP(hipHostMalloc((void **)&g_ring_h, bytes, hipHostMallocDefault), "problem ring (pinned)");
-    for(int i = 0; i < RING_SLOTS; i++){
-        QLMX_HIP(hipEventCreateWithFlags(&g_ring_ev[i], hipEventDisableTiming), "problem ring event");
-        g_ring_used[i] = false;
-    }
     return QLMX_OK;
 }
 
@@ -35,8 +71,7 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
         return QLMX_E_LIMIT;
     }
     int rc = ring_init(); if(rc) return rc;
-    const int slot = g_ring_next; g_ring_next = (g_ring_next + 1) % RING_SLOTS;
-    if(g_ring_used[slot]) QLMX_HIP(hipEventSynchronize(g_ring_ev[slot]), "problem ring wait");
+    int slot; rc = guard_take(g_ring_guard, &slot); if(rc) return rc;
     DevProb *h = g_ring_h + (size_t)slot * QLMX_MAX_PROBLEMS;
     const int tiles_n = (N + tile_cols - 1) / tile_cols;
     long long tiles = 0; int n = 0;
@@ -78,11 +113,7 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
     return QLMX_OK;
 }
 
-int qlmx_upload_done(int slot, hipStream_t stream){
-    QLMX_HIP(hipEventRecord(g_ring_ev[slot], stream), "problem ring record");
-    g_ring_used[slot] = true;
-    return QLMX_OK;
-}
+int qlmx_upload_done(int slot, hipStream_t stream){ return guard_launched(g_ring_guard, slot, stream); }
 
 /* ---- unit tables of scheduled launches: a ring of pinned slots like the one above, each holding a
  * problem table and a unit table; chain flags handed out round the ring of a fixed array
@@ -90,9 +121,7 @@ int qlmx_upload_done(int slot, hipStream_t stream){
 #define UNIT_SLOTS 32
 #define CHAIN_FLAGS (1 << 18)
 static char      *g_unit_h = nullptr;
-static hipEvent_t g_unit_ev[UNIT_SLOTS];
-static bool       g_unit_used[UNIT_SLOTS];
-static int        g_unit_next = 0;
+static RingGuard  g_unit_guard = {UNIT_SLOTS, 8, 0, {}};
 static int       *g_chain_flags = nullptr;
 static unsigned  *g_chain_status = nullptr;      /* pinned: a kernel whose wait ran out sets it */
 static int        g_chain_cursor = 0;
@@ -109,10 +138,6 @@ static int unit_init(void){
     QLMX_HIP(hipMemset(g_chain_flags, 0, CHAIN_FLAGS * sizeof(int)), "chain flags clear");
     QLMX_HIP(hipHostMalloc((void **)&g_chain_status, sizeof(unsigned), hipHostMallocDefault), "chain status (pinned)");
     *g_chain_status = 0;
-    for(int i = 0; i < UNIT_SLOTS; i++){
-        QLMX_HIP(hipEventCreateWithFlags(&g_unit_ev[i], hipEventDisableTiming), "unit ring event");
-        g_unit_used[i] = false;
-    }
     return QLMX_OK;
 }
 
@@ -122,8 +147,7 @@ int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot_out){
         qlmx_set_error("grouped gemm: an earlier launch gave up waiting for a partial sum of a split contraction; its output is incomplete");
         return QLMX_E_HIP;
     }
-    const int slot = g_unit_next; g_unit_next = (g_unit_next + 1) % UNIT_SLOTS;
-    if(g_unit_used[slot]) QLMX_HIP(hipEventSynchronize(g_unit_ev[slot]), "unit ring wait");
+    int slot; rc = guard_take(g_unit_guard, &slot); if(rc) return rc;
     char *h = g_unit_h + slot * UNIT_SLOT_BYTES;
     const size_t uoff = unit_offset(nprob);
     out->hprob = (DevProb *)h; out->hunit = (DevUnit *)(h + uoff);
@@ -133,11 +157,7 @@ int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot_out){
     return QLMX_OK;
 }
 
-int qlmx_unit_done(int slot, hipStream_t stream){
-    QLMX_HIP(hipEventRecord(g_unit_ev[slot], stream), "unit ring record");
-    g_unit_used[slot] = true;
-    return QLMX_OK;
-}
+int qlmx_unit_done(int slot, hipStream_t stream){ return guard_launched(g_unit_guard, slot, stream); }
 
 int qlmx_chain_reserve(int nflags, int *first, unsigned *epoch){
     QLMX_REQUIRE(nflags <= CHAIN_FLAGS / 4, "grouped gemm: %d chained tiles in one launch", nflags);

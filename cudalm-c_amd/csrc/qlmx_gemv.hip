@@ -231,13 +231,22 @@ int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const
                           int K, int N, hipStream_t st){
     QLMX_REQUIRE(N % 32 == 0 && group % 32 == 0, "gemv: N and group must be multiples of 32");
     QLMX_REQUIRE(((uintptr_t)d & 15) == 0, "gemv: digit array must be 16-byte aligned");
-    static GvProb *h_tab = nullptr, *d_tab = nullptr; static hipEvent_t ev; static bool used = false;
-    if(!h_tab){
-        QLMX_HIP(hipHostMalloc((void **)&h_tab, QLMX_MAX_PROBLEMS * sizeof(GvProb), hipHostMallocDefault), "gemv table (pinned)");
-        QLMX_HIP(hipMalloc((void **)&d_tab, QLMX_MAX_PROBLEMS * sizeof(GvProb)), "gemv table (device)");
-        QLMX_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "gemv table event");
+    /* The problem table is written into one of 16 slots of pinned host memory and read by the kernels
+     * from there. The slots are guarded in two halves: an event is recorded behind the launch that
+     * uses the last slot of a half and waited for when the ring re-enters that half (an event behind
+     * every launch would leave the GPU idle for some microseconds each time). */
+    enum { GV_SLOTS = 16, GV_HALF = 8 };
+    static GvProb *ring = nullptr; static hipEvent_t ev[2]; static bool recorded[2] = {false, false};
+    static hipStream_t ev_stream[2] = {nullptr, nullptr}; static int next_slot = 0;
+    if(!ring){
+        QLMX_HIP(hipHostMalloc((void **)&ring, (size_t)GV_SLOTS * QLMX_MAX_PROBLEMS * sizeof(GvProb), hipHostMallocDefault), "gemv table ring (pinned)");
+        for(int i = 0; i < 2; i++) QLMX_HIP(hipEventCreateWithFlags(&ev[i], hipEventDisableTiming), "gemv table event");
     }
-    if(used) QLMX_HIP(hipEventSynchronize(ev), "gemv table wait");
+    const int slot = next_slot, half = slot / GV_HALF;
+    if(slot % GV_HALF == 0 && recorded[half]){ QLMX_HIP(hipEventSynchronize(ev[half]), "gemv table wait"); recorded[half] = false; }
+    /* a half whose launches went to more than one stream is closed by waiting for the odd stream at once */
+    if(slot % GV_HALF == 0) ev_stream[half] = st;
+    GvProb *h_tab = ring + (size_t)slot * QLMX_MAX_PROBLEMS, *d_tab = h_tab;
     int n = 0;
     for(int i = 0; i < nprob; i++){
         if(probs[i].M == 0) continue;
@@ -252,11 +261,12 @@ int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const
     choose_split(K, N, n, &a.S, &a.rps);
     int rc = ws_reserve(0, (size_t)n * a.S * GV_MAXROWS * N, st); if(rc) return rc;
     a.part = g_ws.part[0];
-    QLMX_HIP(hipMemcpyAsync(d_tab, h_tab, (size_t)n * sizeof(GvProb), hipMemcpyHostToDevice, st), "gemv table h2d");
     rc = launch_gemv<GV_MAXROWS>(a, n, st); if(rc) return rc;
     hipLaunchKernelGGL(k_qlmx_gemv_finish<GV_MAXROWS>, dim3((N + 255) / 256, n), dim3(256), 0, st, d_tab, g_ws.part[0], a.S, N);
     QLMX_LAUNCH_CHECK("gemv finish launch");
-    QLMX_HIP(hipEventRecord(ev, st), "gemv table record"); used = true;
+    next_slot = (slot + 1) % GV_SLOTS;
+    if(st != ev_stream[half]) QLMX_HIP(hipStreamSynchronize(st), "gemv table stream wait");
+    if(slot % GV_HALF == GV_HALF - 1){ QLMX_HIP(hipEventRecord(ev[half], ev_stream[half]), "gemv table record"); recorded[half] = true; }
     return QLMX_OK;
 }
 

@@ -65,6 +65,18 @@ def test_gemv_small_rows_vs_oracle(q, orc, K, N):
     q.gemm_nn(dd, ds, 128, q.problems(items), E, K, N, pkg.ACT_F32, pkg.MATH_F32)
     torch.cuda.synchronize()
     assert orc.relerr(dC.cpu().numpy(), want) < 1e-5
+    # forty calls without a synchronisation between them go twice round the ring of problem tables,
+    # each call with its own output (and a different problem order): every one must come out right
+    outs = [torch.zeros(int(off[-1]) * N, device="cuda") for _ in range(40)]
+    for it, o in enumerate(outs):
+        its = [(dA.data_ptr() + int(off[e]) * K * 4, None, o.data_ptr() + int(off[e]) * N * 4, e * K * N, e * K * N // 128, rows[e], 0.0)
+               for e in range(E)]
+        if it & 1:
+            its.reverse()
+        q.gemm_nn(dd, ds, 128, q.problems(its), E, K, N, pkg.ACT_F32, pkg.MATH_F32)
+    torch.cuda.synchronize()
+    for o in outs:
+        assert orc.relerr(o.cpu().numpy(), want) < 1e-5
 
 
 @pytest.mark.parametrize("T,E,D,F,K", [(1, 32, 768, 2048, 2), (4, 8, 768, 2048, 2), (16, 8, 768, 2048, 2),

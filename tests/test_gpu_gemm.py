@@ -227,6 +227,36 @@ def test_mfma_more_problems_than_lanes(q, orc, mode):
     assert orc.relerr(got, want) < TOL_MFMA
 
 
+def test_mfma_table_ring_wraps(q, orc):
+    """150 grouped launches without a synchronisation between them go more than twice round the ring of
+    problem tables (and four times round the unit-table ring of the weight gradient); a launch whose
+    table had been overwritten too early would compute on the wrong pointers."""
+    import torch
+    E, rows, K, N = 3, [70, 0, 33], 64, 128
+    tot = sum(rows)
+    off = np.concatenate([[0], np.cumsum(rows)]).astype(int)
+    d, s, P = make_weights(orc, 21, E, K, N)
+    A = orc.bf16_round(orc.normal(tot * K, 21, 10)); B = orc.bf16_round(orc.normal(tot * N, 21, 11))
+    dA, dB, dd, ds = dev(A), dev(B), dev(d), dev(s)
+    pa, pb = to_bf16_bits(dA), to_bf16_bits(dB)
+    want_nn = np.zeros(tot * N, f32); want_nt = np.zeros(E * K * N, f32)
+    for e in range(E):
+        if rows[e]:
+            orc.gemm_nn(A[off[e] * K:], P[e * K * N:(e + 1) * K * N], want_nn[off[e] * N:off[e + 1] * N], rows[e], K, N)
+            orc.gemm_nt(A[off[e] * K:], B[off[e] * N:], want_nt[e * K * N:(e + 1) * K * N], rows[e], K, N)
+    outs = []
+    for it in range(75):
+        c1 = torch.zeros(tot * N, device="cuda"); c2 = torch.zeros(E * K * N, device="cuda")
+        q.gemm_nn(dd, ds, 128, q.problems([(pa.data_ptr() + off[e] * K * 2, None, c1.data_ptr() + off[e] * N * 4, e * K * N, e * K * N // 128,
+                                            rows[e], 0.0) for e in range(E)]), E, K, N, pkg.ACT_BF16, pkg.MATH_MFMA)
+        q.gemm_nt(q.problems([(pa.data_ptr() + off[e] * K * 2, pb.data_ptr() + off[e] * N * 2, c2.data_ptr() + e * K * N * 4, 0, 0,
+                               rows[e], 0.0) for e in range(E)]), E, K, N, pkg.ACT_BF16, pkg.MATH_MFMA)
+        outs.append((c1, c2))
+    torch.cuda.synchronize()
+    for c1, c2 in outs:
+        assert orc.relerr(c1.cpu().numpy(), want_nn) < TOL_MFMA and orc.relerr(c2.cpu().numpy(), want_nt) < TOL_MFMA
+
+
 def test_mfma_rejects_unsupported_shapes(q):
     import torch
     x = torch.zeros(4096, device="cuda")

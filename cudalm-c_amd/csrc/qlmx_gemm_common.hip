@@ -46,8 +46,15 @@ static int guard_launched(RingGuard &g, int slot, hipStream_t stream){
         sg.st[sg.nst++] = stream;
     }
     if(slot % g.per_seg == g.per_seg - 1){
-        for(int i = 0; i < sg.nst; i++) QLMX_HIP(hipEventRecord(sg.ev[i], sg.st[i]), "table ring record");
-        sg.nrec = sg.nst;
+        sg.nrec = 0;
+        for(int i = 0; i < sg.nst; i++){
+            if(hipEventRecord(sg.ev[sg.nrec], sg.st[i]) == hipSuccess) sg.nrec++;
+            else {
+                /* e.g. a stream destroyed since its launch: fall back to waiting for the whole device */
+                (void)hipGetLastError();
+                QLMX_HIP(hipDeviceSynchronize(), "table ring device wait");
+            }
+        }
     }
     return QLMX_OK;
 }

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the QLM 4-bit hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|adamw|decode|train]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|adamw|decode|train|train5|codec|glue]
 
 Prints ONE JSON line. A "step" is one pass of a hot-path kernel set over one batch of synthetic
 input that is already resident in HBM. Workloads (shapes from BASELINE.json `configs`):
@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train", "copy"])
+    ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train", "train5", "codec", "glue", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--adamw-weights", type=int, default=120 * 2 ** 20)
     ap.add_argument("--render-p", type=int, default=0, help="adamw: also write the fp32 view P (4 B/weight more)")
@@ -71,7 +71,7 @@ def zipf_counts(E, tokens, topk, seed=0):
     return np.bincount(top.ravel(), minlength=E).astype(int)
 
 
-def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2):
+def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label="C3 train layer"):
     from cudalm_c_amd.binding import ACT_BF16, MATH_MFMA
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev); g.manual_seed(0)
@@ -146,8 +146,8 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2):
     tf = flops / (tm["event_ms_avg"] * 1e-3) / 1e12
     dom = max(per, key=lambda k: per[k]["ms"])
     return {
-        "workload": "C3 train layer: E=%d top-%d D=%d F=%d, %d bf16 tokens -> %d expert rows, Zipf(1.1) load (max %d, min %d rows); "
-                    "fwd+dgrad+wgrad = 9 grouped GEMMs in 7 launches" % (E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min())),
+        "workload": "%s: E=%d top-%d D=%d F=%d, %d bf16 tokens -> %d expert rows, Zipf(1.1) load (max %d, min %d rows); "
+                    "fwd+dgrad+wgrad = 9 grouped GEMMs in 7 launches" % (label, E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min())),
         "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tm["wall_ms"], "dtype": "bf16",
         "kernel_ms": tm, "per_launch": per, "gflop_per_step": flops / 1e9,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
@@ -308,6 +308,89 @@ def cpu_adamw(args):
             "weights_per_s": nq * reps / t_used}
 
 
+# --------------------------------------------------------------------------------------- codec, glue
+def _stream_result(name, kernel, entries, note):
+    """entries: list of (label, algorithmic bytes per launch, timing). The reported value is the slowest-rated entry's GB/s."""
+    per = {lab: {"ms": tm["event_ms_avg"], "bytes": b, "gbs": b / (tm["event_ms_avg"] * 1e-3) / 1e9} for lab, b, tm in entries}
+    tot_b = sum(b for _, b, _ in entries); tot_ms = sum(tm["event_ms_avg"] for _, _, tm in entries)
+    gbs = tot_b / (tot_ms * 1e-3) / 1e9
+    return {"workload": name, "metric": "streaming GB/s (algorithmic bytes of all listed launches / their summed time)", "value": gbs,
+            "unit": "GB/s", "ms_per_step": tot_ms, "dtype": "u8+f32", "per_launch": per,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                         "traffic": None, "kernel": kernel, "note": note}}
+
+
+def bench_codec(torch, q, args):
+    """Encode, render and servo over one span of the AdamW sweep's size (init / resume / every 100th step)."""
+    import numpy as np
+    from cudalm_c_amd.binding import SPAN_DTYPE
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev); g.manual_seed(0)
+    nq = (args.adamw_weights // 128) * 128
+    ng = nq // 128
+    P = 0.02 * torch.randn(nq, device=dev, generator=g)
+    d = torch.zeros(nq // 2, dtype=torch.int8, device=dev); r = torch.zeros(nq, dtype=torch.int8, device=dev)
+    s = torch.zeros(ng, device=dev)
+    tab = np.zeros(1, dtype=SPAN_DTYPE)
+    tab[0] = (0, 0, 0, nq, 0, ng, 0.0, 0)
+    sp = torch.from_numpy(tab.view(np.uint8)).to(dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    te = timed(torch, lambda: q.encode(P, d, r, s, sp, 1, 128, 7, 1, ng, stream), args.steps, args.warmup)
+    tr = timed(torch, lambda: q.render(P, d, s, sp, 1, 128, 1, 0, ng, stream), args.steps, args.warmup)
+    # servo thresholds that leave the scales alone (the usual case) and ones that rescale every group
+    ts0 = timed(torch, lambda: q.servo(d, r, s, sp, 1, 128, 7, 2.0, -1.0, 1, ng, stream), args.steps, args.warmup)
+    state = {"k": 0}
+
+    def servo_all():
+        state["k"] ^= 1          # up, down, up, ...: the scales stay in range over any number of calls
+        q.servo(d, r, s, sp, 1, 128, 7, (-1.0 if state["k"] else 2.0), (-1.0 if state["k"] else 2.0), 1, ng, stream)
+    ts1 = timed(torch, servo_all, args.steps, args.warmup)
+    gb = 4.0 / 128
+    return _stream_result(
+        "encode / render / servo over %d weights, group 128, 4-bit packed" % nq, "k_qlmx_encode, k_qlmx_render, k_qlmx_servo",
+        [("encode", nq * (4 + 0.5 + 1 + gb), te), ("render", nq * (0.5 + gb + 4), tr),
+         ("servo, no group rescaled", nq * (0.5 + gb), ts0), ("servo, every group rescaled", nq * (2 * 0.5 + 2 * 1 + 2 * gb), ts1)],
+        "bytes per weight: encode 4 read + 1.5 written, render 0.5 + 4, servo 0.5 read (+ 1 read + 1.5 written where a group is rescaled)")
+
+
+def bench_glue(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2):
+    """The MoE glue kernels at the training layer's shape, each timed on its own."""
+    from cudalm_c_amd.binding import ACT_BF16
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev); g.manual_seed(0)
+    N, K = tokens, topk
+    stream = torch.cuda.current_stream().cuda_stream
+    rt = torch.randn(N * E, device=dev, generator=g)
+    rprobs = torch.empty(N * E, device=dev); assign = torch.empty(K * N, dtype=torch.int32, device=dev); gate = torch.empty(K * N, device=dev)
+    perm = torch.empty(K * N, dtype=torch.int32, device=dev); off = torch.empty(K * (E + 1), dtype=torch.int32, device=dev)
+    ws = torch.empty(q.moe_perm_workspace(N, E, K), dtype=torch.uint8, device=dev)
+    x = torch.randn(N * D, device=dev, generator=g)
+    Xp = torch.empty(N * D, dtype=torch.bfloat16, device=dev)
+    gp = torch.randn(N * F, device=dev, generator=g); up = torch.randn(N * F, device=dev, generator=g)
+    act = torch.empty(N * F, dtype=torch.bfloat16, device=dev)
+    dact = torch.randn(N * F, device=dev, generator=g)
+    dg = torch.empty(N * F, dtype=torch.bfloat16, device=dev); du = torch.empty(N * F, dtype=torch.bfloat16, device=dev)
+    yp = torch.randn(N * D, device=dev, generator=g); out = torch.zeros(N * D, device=dev)
+    dout = torch.randn(N * D, device=dev, generator=g); dgate = torch.empty(N, device=dev)
+    dyp = torch.empty(N * D, dtype=torch.bfloat16, device=dev); dx = torch.zeros(N * D, device=dev)
+    q.router_topk(rt, rprobs, assign, gate, N, E, K, None, 0, stream)
+    q.moe_perm(assign, N, E, K, perm, off, ws, stream)
+    T = lambda fn: timed(torch, fn, args.steps, args.warmup)
+    ent = [
+        ("router_topk", N * E * 8 + K * N * 8, T(lambda: q.router_topk(rt, rprobs, assign, gate, N, E, K, None, 0, stream))),
+        ("moe_perm (both passes)", K * N * 8, T(lambda: q.moe_perm(assign, N, E, K, perm, off, ws, stream))),
+        ("gather -> bf16 (one pass)", N * D * 6 + N * 4, T(lambda: q.moe_gather(x, perm, Xp, N, D, ACT_BF16, stream))),
+        ("swiglu -> bf16 (one pass)", N * F * 10, T(lambda: q.swiglu(gp, up, act, N * F, ACT_BF16, stream))),
+        ("scatter_gate (one pass)", N * D * 12 + N * 8, T(lambda: q.moe_scatter_gate(yp, perm, gate, out, N, D, stream))),
+        ("dgate -> bf16 (one pass)", N * D * 10 + N * 12, T(lambda: q.moe_dgate(dout, yp, perm, gate, dgate, dyp, N, D, ACT_BF16, stream))),
+        ("swiglu_bwd -> bf16 (one pass)", N * F * 16, T(lambda: q.swiglu_bwd(gp, up, dact, dg, du, N * F, ACT_BF16, stream))),
+        ("scatter_add (one pass)", N * D * 12 + N * 4, T(lambda: q.moe_scatter_add(yp, perm, dx, N, D, stream))),
+    ]
+    return _stream_result("MoE glue at E=%d top-%d D=%d F=%d, %d tokens (per pass of %d rows)" % (E, K, D, F, N, N),
+                          "qlmx_glue.hip kernels", ent,
+                          "bytes: every operand read once and every output written once (scatter kernels read-modify-write their destination)")
+
+
 def bench_copy(torch, q, args):
     """Plain 1 GiB device copy: the known-size kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
     n = 2 ** 28
@@ -368,12 +451,13 @@ def main():
     q = pkg.load()           # raises if libqlmx.so is missing or no gfx950 device
     torch.cuda.set_device(0)
     want = ["train", "decode", "adamw"] if args.workload == "all" else [args.workload]
-    runners = {"adamw": bench_adamw, "train": bench_train, "decode": bench_decode, "copy": bench_copy}
+    runners = {"adamw": bench_adamw, "train": bench_train, "decode": bench_decode, "copy": bench_copy, "codec": bench_codec, "glue": bench_glue,
+               "train5": lambda t, qq, a: bench_train(t, qq, a, E=64, D=2048, F=1408, tokens=32768, topk=4, label="C5 train layer (one of 8)")}
     results = {}
     for w in want:
         if w in runners:
             results[w] = runners[w](torch, q, args)
-    first = next(results[w] for w in ["train", "decode", "adamw", "copy"] if w in results)
+    first = next(results[w] for w in ["train", "train5", "decode", "adamw", "codec", "glue", "copy"] if w in results)
     line = {
         "metric": "QLM expert dequant-GEMM TFLOP/s & GB/s (% roofline); int-AdamW GB/s",
         "value": first["value"], "unit": first["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -112,11 +112,41 @@ __global__ void __launch_bounds__(256) k_qlmx_render(float *P, const signed char
 
 __global__ void __launch_bounds__(256) k_qlmx_servo(signed char *d, signed char *r, float *s,
                                                     const qlmx_span *sp, int nspan, int group, int dmax,
-                                                    float f_hi, float f_lo, int packed, int ngrp){
+                                                    float f_hi, float f_lo, int packed, int ngrp, int vec_ok){
     const int lane16 = threadIdx.x & 15;
     const int gi = (int)((blockIdx.x * (unsigned)blockDim.x + threadIdx.x) >> 4);
     if(gi >= ngrp) return;
     const GroupLoc L = group_loc(sp, nspan, gi, group);
+    if(vec_ok && group == 128 && packed && L.n == 128 && (L.qi0 & 7ULL) == 0){
+        /* 8 consecutive elements per lane: one 32-bit word of digits, and 8 residual bytes only where the
+         * group is rescaled */
+        const uint64_t e0 = L.qi0 + (uint64_t)lane16 * 8;
+        const uint32_t dw = *(const uint32_t *)(d + (e0 >> 1));
+        int dv[8], railed = 0;
+#pragma unroll
+        for(int k = 0; k < 8; k++){ dv[k] = qx_nib(dw, k); railed += (dv[k] == dmax) | (dv[k] == -dmax); }
+        railed = qx_row16_sum(railed);
+        const float f = (float)railed / 128.0f, sg = s[gi];
+        float sn;
+        if(f > f_hi)      sn = sg * 1.09051f;
+        else if(f < f_lo) sn = sg / 1.09051f;
+        else return;
+        const float conv = sg / sn;
+        if(lane16 == 0) s[gi] = sn;
+        const uint2 rw = *(const uint2 *)(r + e0);
+        uint32_t dn = 0, r0 = 0, r1 = 0;
+#pragma unroll
+        for(int k = 0; k < 8; k++){
+            const int rb = (int)(signed char)(((k < 4 ? rw.x : rw.y) >> (8 * (k & 3))) & 0xFFu);
+            const float t = ((float)dv[k] + (float)rb * (1.0f / 128.0f)) * conv;
+            int dd, rr; quantize(t, dmax, dd, rr);
+            dn |= ((uint32_t)dd & 15u) << (4 * k);
+            if(k < 4) r0 |= ((uint32_t)rr & 0xFFu) << (8 * k); else r1 |= ((uint32_t)rr & 0xFFu) << (8 * (k - 4));
+        }
+        *(uint32_t *)(d + (e0 >> 1)) = dn;
+        *(uint2 *)(r + e0) = make_uint2(r0, r1);
+        return;
+    }
     int railed = 0;
     for(int jb = 2 * lane16; jb < L.n; jb += 32)
         for(int h = 0; h < 2; h++){
@@ -192,8 +222,9 @@ extern "C" int qlmx_servo(signed char *d, signed char *r, float *s,
     QLMX_REQUIRE(d && r && s && sp, "qlmx_servo: NULL buffer");
     rc = codec_args_ok("qlmx_servo", nspan, group, dmax, packed); if(rc) return rc;
     if(ngrp <= 0) return QLMX_OK;
+    const int vec_ok = ((uintptr_t)r & 7) == 0 && ((uintptr_t)d & 3) == 0;
     hipLaunchKernelGGL(k_qlmx_servo, dim3((unsigned)((ngrp + 15) / 16)), dim3(256), 0, (hipStream_t)stream,
-                       d, r, s, sp, nspan, group, dmax, f_hi, f_lo, packed, ngrp);
+                       d, r, s, sp, nspan, group, dmax, f_hi, f_lo, packed, ngrp, vec_ok);
     QLMX_LAUNCH_CHECK("qlmx_servo launch");
     return QLMX_OK;
 }

@@ -30,13 +30,10 @@ __device__ __forceinline__ float qx_fexp(float x){
 __device__ __forceinline__ float qx_fsig(float x){ return 1.0f / (1.0f + qx_fexp(-x)); }
 
 /* ---- router: one thread per token, experts visited in order so the softmax sum rounds exactly as
- * the reference's loop does ---- */
-__global__ void __launch_bounds__(256) k_router_topk(const float *rt, float *rprobs, int *assign, float *gate,
-                                                     int N, int E, int K, const float *bias, int bs){
-    const int n = blockIdx.x * 256 + threadIdx.x;
-    if(n >= N) return;
-    const float *logit = rt + (size_t)n * E;
-    float *pr = rprobs + (size_t)n * E;
+ * the reference's loop does. `logit` points at the token's E logits and `pr` at E floats for its
+ * probabilities (the two may be the same place). ---- */
+__device__ __forceinline__ void route_token(const float *logit, float *pr, int n, int *assign, float *gate,
+                                            int N, int E, int K, const float *bias, int bs){
     float mx = -1e30f;
     for(int e = 0; e < E; e++) if(logit[e] > mx) mx = logit[e];
     float sum = 0.0f;
@@ -60,6 +57,93 @@ __global__ void __launch_bounds__(256) k_router_topk(const float *rt, float *rpr
         assign[(size_t)k * N + n] = best;
         gate[(size_t)k * N + n] = pr[best];
     }
+}
+
+/* rows straight from memory: consecutive threads are E floats apart, for any E */
+__global__ void __launch_bounds__(256) k_router_topk(const float *rt, float *rprobs, int *assign, float *gate,
+                                                     int N, int E, int K, const float *bias, int bs){
+    const int n = blockIdx.x * 256 + threadIdx.x;
+    if(n >= N) return;
+    route_token(rt + (size_t)n * E, rprobs + (size_t)n * E, n, assign, gate, N, E, K, bias, bs);
+}
+
+/* The rows of RT_TOK consecutive tokens are one contiguous piece of `rt`: it is copied to LDS with
+ * consecutive threads on consecutive floats, each thread then routes its token out of LDS (rows an odd
+ * number of floats apart, so the lanes of a wavefront hit different banks), and the probabilities go
+ * back the way the logits came. Same arithmetic in the same order as the kernel above. */
+#define RT_TOK 64
+#define RT_MAXE 96
+__global__ void __launch_bounds__(RT_TOK) k_router_topk_lds(const float *rt, float *rprobs, int *assign, float *gate,
+                                                            int N, int E, int K, const float *bias, int bs){
+    extern __shared__ float rows[];
+    const int n0 = blockIdx.x * RT_TOK, tid = threadIdx.x;
+    const int ld = E | 1;
+    const int cnt = min(RT_TOK, N - n0) * E;
+    const float *src = rt + (size_t)n0 * E;
+    int t = tid / E, e = tid - t * E;
+    const int dt = RT_TOK / E, de = RT_TOK - dt * E;
+    for(int i = tid; i < cnt; i += RT_TOK){
+        rows[t * ld + e] = src[i];
+        t += dt; e += de; if(e >= E){ e -= E; t++; }
+    }
+    __syncthreads();
+    if(n0 + tid < N) route_token(rows + tid * ld, rows + tid * ld, n0 + tid, assign, gate, N, E, K, bias, bs);
+    __syncthreads();
+    float *dst = rprobs + (size_t)n0 * E;
+    t = tid / E; e = tid - t * E;
+    for(int i = tid; i < cnt; i += RT_TOK){
+        dst[i] = rows[t * ld + e];
+        t += dt; e += de; if(e >= E){ e -= E; t++; }
+    }
+}
+
+/* Expert count known at compile time (at most 64): the token's row lives in registers between the
+ * staged load and the staged store, the chosen experts in a bit mask. Same operations in the same
+ * order as route_token. */
+template<int EE>
+__global__ void __launch_bounds__(RT_TOK) k_router_topk_reg(const float *rt, float *rprobs, int *assign, float *gate,
+                                                            int N, int K, const float *bias, int bs){
+    __shared__ float rows[RT_TOK * (EE | 1)];
+    constexpr int ld = EE | 1;
+    const int n0 = blockIdx.x * RT_TOK, tid = threadIdx.x;
+    const int cnt = min(RT_TOK, N - n0) * EE;
+    const float *src = rt + (size_t)n0 * EE;
+    for(int i = tid; i < cnt; i += RT_TOK) rows[(i / EE) * ld + (i % EE)] = src[i];
+    __syncthreads();
+    const int n = n0 + tid;
+    if(n < N){
+        float p[EE];
+#pragma unroll
+        for(int e = 0; e < EE; e++) p[e] = rows[tid * ld + e];
+        float mx = -1e30f;
+#pragma unroll
+        for(int e = 0; e < EE; e++) if(p[e] > mx) mx = p[e];
+        float sum = 0.0f;
+#pragma unroll
+        for(int e = 0; e < EE; e++){ p[e] = qx_fexp(p[e] - mx); sum += p[e]; }
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for(int e = 0; e < EE; e++){ p[e] *= inv; rows[tid * ld + e] = p[e]; }
+        unsigned long long taken = 0ULL;
+        for(int k = 0; k < K; k++){
+            int best = -1; float bestp = -1e30f;
+#pragma unroll
+            for(int e = 0; e < EE; e++){
+                const float sc = p[e] + (bias ? bias[k * bs + e] : 0.0f);
+                if(!((taken >> e) & 1ULL) && sc > bestp){ bestp = sc; best = e; }
+            }
+            if(best < 0) best = k;
+            taken |= 1ULL << best;
+            float gv = 0.0f;
+#pragma unroll
+            for(int e = 0; e < EE; e++) if(e == best) gv = p[e];
+            assign[(size_t)k * N + n] = best;
+            gate[(size_t)k * N + n] = gv;
+        }
+    }
+    __syncthreads();
+    float *dst = rprobs + (size_t)n0 * EE;
+    for(int i = tid; i < cnt; i += RT_TOK) dst[i] = rows[(i / EE) * ld + (i % EE)];
 }
 
 /* ---- grouping permutation of one pass: perm lists the tokens expert by expert, tokens of one
@@ -252,7 +336,18 @@ extern "C" int qlmx_router_topk(const float *rt, float *rprobs, int *assign, flo
     QLMX_REQUIRE(rt && rprobs && assign && gate, "qlmx_router_topk: NULL buffer");
     QLMX_REQUIRE(N >= 0 && E > 0 && K > 0 && K <= 8 && K <= E, "qlmx_router_topk: N=%d E=%d K=%d (K at most 8 and at most E)", N, E, K);
     if(N == 0) return QLMX_OK;
-    hipLaunchKernelGGL(k_router_topk, dim3((N + 255) / 256), dim3(256), 0, (hipStream_t)stream, rt, rprobs, assign, gate, N, E, K, bias, bs);
+    const dim3 rgrid((N + RT_TOK - 1) / RT_TOK);
+#define ROUTE_REG(EE) hipLaunchKernelGGL(k_router_topk_reg<EE>, rgrid, dim3(RT_TOK), 0, (hipStream_t)stream, rt, rprobs, assign, gate, N, K, bias, bs)
+    if(E == 8) ROUTE_REG(8);
+    else if(E == 16) ROUTE_REG(16);
+    else if(E == 32) ROUTE_REG(32);
+    else if(E == 64) ROUTE_REG(64);
+#undef ROUTE_REG
+    else if(E <= RT_MAXE)
+        hipLaunchKernelGGL(k_router_topk_lds, dim3((N + RT_TOK - 1) / RT_TOK), dim3(RT_TOK), (size_t)RT_TOK * (E | 1) * sizeof(float),
+                           (hipStream_t)stream, rt, rprobs, assign, gate, N, E, K, bias, bs);
+    else
+        hipLaunchKernelGGL(k_router_topk, dim3((N + 255) / 256), dim3(256), 0, (hipStream_t)stream, rt, rprobs, assign, gate, N, E, K, bias, bs);
     QLMX_LAUNCH_CHECK("router launch");
     return QLMX_OK;
 }

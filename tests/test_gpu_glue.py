@@ -79,6 +79,25 @@ def test_router_training_size_vs_oracle(q, orc):
     assert np.array_equal(pr.cpu().numpy().view(np.uint32), want_pr.view(np.uint32))
 
 
+@pytest.mark.parametrize("N,E,K,with_bias", [(1000, 64, 4, False), (77, 5, 2, True), (130, 96, 8, False), (65, 97, 3, True),
+                                              (300, 7, 7, False), (1, 32, 2, False), (515, 32, 8, True), (200, 16, 3, False), (129, 8, 8, True)])
+def test_router_shapes_vs_oracle(q, orc, N, E, K, with_bias):
+    """Expert counts served by the register kernel (8, 16, 32, 64), by the LDS-staged one and beyond its
+    limit, odd counts, token counts off the workgroup size, K up to its maximum, per-pass bias:
+    bit-identical to the CPU oracle."""
+    import torch
+    rt = np.round(orc.normal(N * E, 5, N + E, 2.0) * 16).astype(f32) / 16
+    bias = (orc.normal(K * E, 5, 7, 0.01) if with_bias else None)
+    want_pr = np.zeros(N * E, f32); want_asn = np.zeros(K * N, np.int32); want_gate = np.zeros(K * N, f32)
+    orc.router_topk(rt, want_pr, want_asn, want_gate, N, E, K, bias, E if with_bias else 0)
+    pr, asn, gate = zeros(N * E), zeros(K * N, torch.int32), zeros(K * N)
+    q.router_topk(dev(rt), pr, asn, gate, N, E, K, dev(bias) if with_bias else None, E if with_bias else 0)
+    torch.cuda.synchronize()
+    assert np.array_equal(asn.cpu().numpy(), want_asn)
+    assert np.array_equal(gate.cpu().numpy().view(np.uint32), want_gate.view(np.uint32))
+    assert np.array_equal(pr.cpu().numpy().view(np.uint32), want_pr.view(np.uint32))
+
+
 def test_router_limits(q):
     z = zeros(64)
     with pytest.raises(pkg.QlmxError, match="K"):

@@ -79,6 +79,24 @@ def test_golden_encode_render_step_servo(q, golden, name):
     assert beq(d2, g["sv_d"]) and beq(r2, g["sv_r"]) and beq(s2, g["sv_s"])
 
 
+def test_servo_vs_oracle_seeded(q, orc):
+    """Servo over 1M weights in two spans (the second ends in a short group): thresholds chosen so that
+    groups go up, down and stay; digits, residuals and scales byte-identical to the CPU oracle."""
+    group, dmax = 128, 7
+    tab, nq, ng = make_spans([128 * 5000, 128 * 3000 + 40], group)
+    hd = orc.digits(nq, 3, 1); hr = orc.int8(nq, 3, 2, -64, 64)
+    hs = orc.uniform(ng, 3, 3, 0.5, 1.5) * f32(0.02 * 3 / 7)
+    # uniform digits rail 2/15 of the elements on average: thresholds either side of that
+    f_hi, f_lo = 0.15, 0.11
+    d, r, s = dev(hd), dev(hr), dev(hs)
+    q.servo(d, r, s, dev(tab), len(tab), group, dmax, f_hi, f_lo, 1, ng)
+    s0 = hs.copy()
+    orc.servo(hd, hr, hs, tab, group, dmax, f_hi, f_lo, 1, ng)
+    assert beq(d, hd) and beq(r, hr) and beq(s, hs)
+    up, down = int((hs > s0).sum()), int((hs < s0).sum())
+    assert up > 100 and down > 100 and ng - up - down > 100
+
+
 @pytest.mark.parametrize("nopview", [False, True])
 def test_step_vs_oracle_seeded_2m(q, orc, nopview):
     """Three consecutive steps over 2M weights in two spans (one with a short tail group and a

@@ -96,15 +96,19 @@ __global__ void __launch_bounds__(256) k_qlmx_render(float *P, const signed char
     const float sg = s[gi];
     const bool fast = vec_ok && group == 128 && packed && L.n == 128 && ((L.pof | L.qi0) & 7ULL) == 0;
     if(fast){
-        const uint64_t e0 = (uint64_t)lane16 * 8;
-        const uint32_t dw = *(const uint32_t *)(d + ((L.qi0 + e0) >> 1));
-        float4 o0, o1;
-        o0.x = sg * (float)qx_nib(dw, 0); o0.y = sg * (float)qx_nib(dw, 1);
-        o0.z = sg * (float)qx_nib(dw, 2); o0.w = sg * (float)qx_nib(dw, 3);
-        o1.x = sg * (float)qx_nib(dw, 4); o1.y = sg * (float)qx_nib(dw, 5);
-        o1.z = sg * (float)qx_nib(dw, 6); o1.w = sg * (float)qx_nib(dw, 7);
-        *(float4 *)(P + L.pof + e0) = o0;
-        *(float4 *)(P + L.pof + e0 + 4) = o1;
+        /* a lane renders elements 4*lane16 .. +3 and the same 64 further on: each of the two stores of
+         * a 16-lane row covers 256 contiguous bytes of P, written past the caches */
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        const uint64_t e0 = (uint64_t)lane16 * 4;
+        const unsigned short *dh = (const unsigned short *)(d + (L.qi0 >> 1));
+        const uint32_t w0 = dh[lane16], w1 = dh[16 + lane16];
+        f4 o0, o1;
+        o0.x = sg * (float)qx_nib(w0, 0); o0.y = sg * (float)qx_nib(w0, 1);
+        o0.z = sg * (float)qx_nib(w0, 2); o0.w = sg * (float)qx_nib(w0, 3);
+        o1.x = sg * (float)qx_nib(w1, 0); o1.y = sg * (float)qx_nib(w1, 1);
+        o1.z = sg * (float)qx_nib(w1, 2); o1.w = sg * (float)qx_nib(w1, 3);
+        __builtin_nontemporal_store(o0, (f4 *)(P + L.pof + e0));
+        __builtin_nontemporal_store(o1, (f4 *)(P + L.pof + e0 + 64));
     } else {
         for(int j = lane16; j < L.n; j += 16) P[L.pof + j] = sg * (float)load_digit(d, L.qi0 + j, packed);
     }

@@ -148,12 +148,17 @@ __global__ void __launch_bounds__(RT_TOK) k_router_topk_reg(const float *rt, flo
 
 /* ---- grouping permutation of one pass: perm lists the tokens expert by expert, tokens of one
  * expert in ascending order; off[e] is the first row of expert e, off[E] = N.
- * Three launches: per-chunk histograms, one scan per pass, stable placement. ---- */
+ * Launches: clear, per-chunk histograms (which also add up the experts' totals), scan, stable placement. ---- */
 #define GP_CHUNK 256
-__global__ void k_gp_clear(int *bad){ if(threadIdx.x == 0) *bad = 0; }
+/* workspace: ch[K][NC][E] chunk histograms, then 4 ints (the first is the out-of-range flag), then
+ * tot[K][E] per-expert totals */
+__global__ void __launch_bounds__(256) k_gp_clear(int *bad, int ntot){
+    for(int i = threadIdx.x; i < 4 + ntot; i += 256) bad[i] = 0;
+}
 __global__ void __launch_bounds__(GP_CHUNK) k_gp_hist(const int *asn, int N, int E, int NC, int *ch, int *bad){
     extern __shared__ int hist[];
     const int c = blockIdx.x, k = blockIdx.y, n = c * GP_CHUNK + threadIdx.x;
+    int *tot = bad + 4;
     for(int e = threadIdx.x; e < E; e += GP_CHUNK) hist[e] = 0;
     __syncthreads();
     if(n < N){
@@ -161,28 +166,40 @@ __global__ void __launch_bounds__(GP_CHUNK) k_gp_hist(const int *asn, int N, int
         if((unsigned)e >= (unsigned)E) atomicExch(bad, -1 - e); else atomicAdd(&hist[e], 1);
     }
     __syncthreads();
-    for(int e = threadIdx.x; e < E; e += GP_CHUNK) ch[((size_t)k * NC + c) * E + e] = hist[e];
+    for(int e = threadIdx.x; e < E; e += GP_CHUNK){
+        const int h = hist[e];
+        ch[((size_t)k * NC + c) * E + e] = h;
+        if(h) atomicAdd(&tot[(size_t)k * E + e], h);
+    }
 }
-/* one workgroup per pass: ch[k][c][e] becomes the first output row of (chunk c, expert e) */
-__global__ void __launch_bounds__(256) k_gp_scan(int *ch, int E, int NC, int *off){
-    extern __shared__ int tot[];
-    const int k = blockIdx.x;
-    int *chk = ch + (size_t)k * NC * E;
-    for(int e = threadIdx.x; e < E; e += 256){
-        int t = 0;
-        for(int c = 0; c < NC; c++) t += chk[(size_t)c * E + e];
-        tot[e] = t;
+__device__ __forceinline__ int wave_incl_scan(int v, int lane){
+#pragma unroll
+    for(int d = 1; d < 64; d <<= 1){ const int u = __shfl_up(v, d, 64); if(lane >= d) v += u; }
+    return v;
+}
+/* one wavefront per (pass, expert), and one more per pass for off[E]: the expert's first row is the
+ * sum of the totals of the experts before it; ch[k][c][e] becomes the first output row of
+ * (chunk c, expert e), 64 chunks per scan step */
+__global__ void __launch_bounds__(256) k_gp_scan(int *ch, const int *tot, int E, int NC, int *off){
+    const int k = blockIdx.y, lane = threadIdx.x & 63, e = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if(e > E) return;
+    int base = 0;
+    for(int j0 = 0; j0 < e; j0 += 64){
+        const int j = j0 + lane;
+        base += j < e ? tot[(size_t)k * E + j] : 0;
     }
-    __syncthreads();
-    if(threadIdx.x == 0){
-        int run = 0;
-        for(int e = 0; e < E; e++){ const int t = tot[e]; tot[e] = run; off[(size_t)k * (E + 1) + e] = run; run += t; }
-        off[(size_t)k * (E + 1) + E] = run;
-    }
-    __syncthreads();
-    for(int e = threadIdx.x; e < E; e += 256){
-        int run = tot[e];
-        for(int c = 0; c < NC; c++){ const int t = chk[(size_t)c * E + e]; chk[(size_t)c * E + e] = run; run += t; }
+#pragma unroll
+    for(int d = 32; d >= 1; d >>= 1) base += __shfl_xor(base, d, 64);
+    if(lane == 0) off[(size_t)k * (E + 1) + e] = base;
+    if(e == E) return;
+    int *col = ch + (size_t)k * NC * E + e;
+    int run = base;
+    for(int c0 = 0; c0 < NC; c0 += 64){
+        const int c = c0 + lane;
+        const int t = c < NC ? col[(size_t)c * E] : 0;
+        const int incl = wave_incl_scan(t, lane);
+        if(c < NC) col[(size_t)c * E] = run + incl - t;
+        run += __shfl(incl, 63, 64);
     }
 }
 /* stable placement: a token's row = start of (its chunk, its expert) + the number of earlier
@@ -354,7 +371,7 @@ extern "C" int qlmx_router_topk(const float *rt, float *rprobs, int *assign, flo
 
 extern "C" size_t qlmx_moe_perm_workspace(int N, int E, int K){
     const size_t NC = (size_t)(N + GP_CHUNK - 1) / GP_CHUNK;
-    return ((size_t)K * NC * E + 4) * sizeof(int);
+    return ((size_t)K * NC * E + 4 + (size_t)K * E) * sizeof(int);
 }
 
 extern "C" int qlmx_moe_perm(const int *assign, int N, int E, int K, int *perm, int *off, void *workspace, void *stream){
@@ -364,11 +381,11 @@ extern "C" int qlmx_moe_perm(const int *assign, int N, int E, int K, int *perm, 
     QLMX_REQUIRE(N > 0 && E > 0 && E <= 4096 && K > 0, "qlmx_moe_perm: N=%d E=%d K=%d", N, E, K);
     const int NC = (N + GP_CHUNK - 1) / GP_CHUNK;
     int *ch = (int *)workspace, *bad = ch + (size_t)K * NC * E;
-    hipLaunchKernelGGL(k_gp_clear, dim3(1), dim3(64), 0, st, bad);       /* a kernel, not a memset: callers may capture this into a graph */
+    hipLaunchKernelGGL(k_gp_clear, dim3(1), dim3(256), 0, st, bad, K * E);       /* a kernel, not a memset: callers may capture this into a graph */
     QLMX_LAUNCH_CHECK("perm flag clear");
     hipLaunchKernelGGL(k_gp_hist, dim3(NC, K), dim3(GP_CHUNK), E * sizeof(int), st, assign, N, E, NC, ch, bad);
     QLMX_LAUNCH_CHECK("perm histogram launch");
-    hipLaunchKernelGGL(k_gp_scan, dim3(K), dim3(256), E * sizeof(int), st, ch, E, NC, off);
+    hipLaunchKernelGGL(k_gp_scan, dim3((E + 1 + 3) / 4, K), dim3(256), 0, st, ch, (const int *)(bad + 4), E, NC, off);
     QLMX_LAUNCH_CHECK("perm scan launch");
     hipLaunchKernelGGL(k_gp_scatter, dim3(NC, K), dim3(GP_CHUNK), 4 * E * sizeof(int), st, assign, N, E, NC, (const int *)ch, perm);
     QLMX_LAUNCH_CHECK("perm scatter launch");

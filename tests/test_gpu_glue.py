@@ -114,7 +114,7 @@ def gpu_perm(q, asn, N, E, K):
     return perm.cpu().numpy(), off.cpu().numpy(), ws
 
 
-@pytest.mark.parametrize("N,E,K", [(1, 1, 1), (50, 3, 2), (256, 8, 1), (257, 8, 3), (1000, 64, 4), (8192, 32, 2), (5000, 300, 2)])
+@pytest.mark.parametrize("N,E,K", [(1, 1, 1), (50, 3, 2), (256, 8, 1), (257, 8, 3), (1000, 64, 4), (8192, 32, 2), (5000, 300, 2), (40000, 70, 2)])
 def test_perm_vs_oracle(q, orc, N, E, K):
     rng = np.random.default_rng(N * 31 + E)
     p = (np.arange(E) + 1.0) ** -1.1; p /= p.sum()
@@ -127,6 +127,23 @@ def test_perm_vs_oracle(q, orc, N, E, K):
         assert orc.moe_perm(asn[k * N:(k + 1) * N], N, E, wp, wo) == 0
         assert np.array_equal(off[k * (E + 1):(k + 1) * (E + 1)], wo)
         assert np.array_equal(perm[k * N:(k + 1) * N], wp)
+
+
+def test_perm_workspace_reused(q, orc):
+    """The same workspace serves one call after another (its counters are cleared by each call)."""
+    import torch
+    N, E, K = 3000, 16, 2
+    ws = torch.zeros(q.moe_perm_workspace(N, E, K), dtype=torch.uint8, device="cuda")
+    for seed in (1, 2, 3):
+        asn = np.random.default_rng(seed).integers(0, E, K * N).astype(np.int32)
+        perm, off = zeros(K * N, torch.int32), zeros(K * (E + 1), torch.int32)
+        q.moe_perm(dev(asn), N, E, K, perm, off, ws)
+        q.moe_perm_status(ws, N, E, K)
+        for k in range(K):
+            wp = np.zeros(N, np.int32); wo = np.zeros(E + 1, np.int32)
+            assert orc.moe_perm(asn[k * N:(k + 1) * N], N, E, wp, wo) == 0
+            assert np.array_equal(off.cpu().numpy()[k * (E + 1):(k + 1) * (E + 1)], wo)
+            assert np.array_equal(perm.cpu().numpy()[k * N:(k + 1) * N], wp)
 
 
 def test_perm_reports_bad_expert(q):

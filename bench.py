@@ -126,8 +126,7 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
         ("fwd w1,w3 (nn)", lambda: q.gemm_nn(d, s, group, p_w13, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream), 2),
         ("fwd w2 (nn)", lambda: q.gemm_nn(d, s, group, p_w2, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
         ("dgrad w2 (tn)", lambda: q.gemm_tn(d, s, group, p_d2, E, D, F, ACT_BF16, MATH_MFMA, stream), 1),
-        ("dgrad w1 (tn)", lambda: q.gemm_tn(d, s, group, p_d1, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
-        ("dgrad w3 (tn,+=)", lambda: q.gemm_tn(d, s, group, p_d3, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
+        ("dgrad w1,w3 (tn pair)", lambda: q.gemm_tn_pair(d, s, group, p_d1, p_d3, E, F, D, ACT_BF16, MATH_MFMA, stream), 2),
         ("wgrad w2 (nt)", lambda: q.gemm_nt(p_g2, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
         ("wgrad w1,w3 (nt)", lambda: q.gemm_nt(p_g13, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream), 2),
     ]
@@ -147,11 +146,11 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
     dom = max(per, key=lambda k: per[k]["ms"])
     return {
         "workload": "%s: E=%d top-%d D=%d F=%d, %d bf16 tokens -> %d expert rows, Zipf(1.1) load (max %d, min %d rows); "
-                    "fwd+dgrad+wgrad = 9 grouped GEMMs in 7 launches" % (label, E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min())),
+                    "fwd+dgrad+wgrad = 9 grouped GEMMs in 6 launches" % (label, E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min())),
         "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tm["wall_ms"], "dtype": "bf16",
         "kernel_ms": tm, "per_launch": per, "gflop_per_step": flops / 1e9,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "kernel": "k_gemm_nn_lds, k_gemm_tn_lds, k_gemm_nt_lds (all 7 launches; slowest: %s)" % dom,
+                     "traffic": None, "kernel": "k_gemm_nn_lds, k_gemm_tn_lds, k_gemm_nt_lds (all 6 launches; slowest: %s)" % dom,
                      "note": "algorithmic flops only; the forward issues two MFMAs per product (bf16 hi+lo weight split)"},
     }
 

@@ -1,16 +1,18 @@
 /* qlmx_gemm_api.hip -- C entry points of the grouped expert GEMMs: argument checks and the choice
  * between the fp32 vector-ALU kernels and the bf16 MFMA kernels. */
 #include "qlmx_gemm.h"
+#include <stdlib.h>
 
 int qlmx_gemm_f32_dispatch(int mode, const signed char *d, const float *s, int group,
                            const qlmx_gemm_prob *probs, int nprob, int K, int N, int act_dtype, hipStream_t st);
 int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob,
                           int K, int N, hipStream_t st);
 int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int group,
-                            const qlmx_gemm_prob *probs, int nprob, int K, int N, int act_dtype, hipStream_t st);
+                            const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second, int nprob, int K, int N, int act_dtype, hipStream_t st);
 
 static int gemm_entry(const char *who, int mode, const signed char *d, const float *s, int group,
-                      const qlmx_gemm_prob *probs, int nprob, int K, int N, int act_dtype, int math, void *stream){
+                      const qlmx_gemm_prob *probs, int nprob, int K, int N, int act_dtype, int math, void *stream,
+                      const qlmx_gemm_prob *second = nullptr){
     int rc = qlmx_check_ready(); if(rc) return rc;
     QLMX_REQUIRE(K > 0 && N > 0, "%s: K=%d N=%d", who, K, N);
     QLMX_REQUIRE(act_dtype == QLMX_ACT_F32 || act_dtype == QLMX_ACT_BF16, "%s: act_dtype %d", who, act_dtype);
@@ -21,10 +23,12 @@ static int gemm_entry(const char *who, int mode, const signed char *d, const flo
         const int along = mode == GEMM_NN ? N : K;
         QLMX_REQUIRE(along % group == 0, "%s: the grouped dimension (%d) is not a multiple of the group (%d)", who, along, group);
         for(int i = 0; i < nprob; i++)
-            QLMX_REQUIRE(probs[i].wq % (unsigned long long)group == 0, "%s: problem %d weight offset is not group aligned", who, i);
+            QLMX_REQUIRE(probs[i].wq % (unsigned long long)group == 0 && (!second || second[i].wq % (unsigned long long)group == 0),
+                         "%s: problem %d weight offset is not group aligned", who, i);
     }
     if(math == QLMX_MATH_MFMA)
-        return qlmx_gemm_mfma_dispatch(mode, d, s, group, probs, nprob, K, N, act_dtype, (hipStream_t)stream);
+        return qlmx_gemm_mfma_dispatch(mode, d, s, group, probs, second, nprob, K, N, act_dtype, (hipStream_t)stream);
+    QLMX_REQUIRE(!second, "%s: continued contractions need the MFMA path", who);
     if(mode == GEMM_NN && act_dtype == QLMX_ACT_F32 && N % 32 == 0 && group % 32 == 0 && ((uintptr_t)d & 15) == 0){
         /* every problem has a few rows only: stream the weights once (decode shape) */
         bool small = nprob > 0;
@@ -45,6 +49,28 @@ extern "C" int qlmx_moe_gemm_tn(const signed char *d, const float *s, int group,
                                 const qlmx_gemm_prob *probs, int nprob, int K, int N,
                                 int act_dtype, int math, void *stream){
     return gemm_entry("qlmx_moe_gemm_tn", GEMM_TN, d, s, group, probs, nprob, K, N, act_dtype, math, stream);
+}
+/* The pair of mg_abt_b calls on one output (cudalm.cu:4365-4366: dXp = dgp . w1^T, then dXp += dup . w3^T)
+ * as one launch: problem i computes C = first[i].A . W(first[i])^T + second[i].A . W(second[i])^T
+ * (+ C when first[i].beta = 1); second[i] supplies A, wq, wg and must repeat M. On bf16 activations
+ * with MFMA math the two contractions run as one, the sum never leaving the accumulators; every other
+ * combination runs the two launches the reference would. */
+extern "C" int qlmx_moe_gemm_tn_pair(const signed char *d, const float *s, int group,
+                                     const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int K, int N,
+                                     int act_dtype, int math, void *stream){
+    QLMX_REQUIRE(first && second && nprob >= 0, "qlmx_moe_gemm_tn_pair: NULL problem list");
+    for(int i = 0; i < nprob; i++)
+        QLMX_REQUIRE(second[i].M == first[i].M, "qlmx_moe_gemm_tn_pair: problem %d has %d and %d rows", i, first[i].M, second[i].M);
+    if(act_dtype == QLMX_ACT_BF16 && math == QLMX_MATH_MFMA)
+        return gemm_entry("qlmx_moe_gemm_tn_pair", GEMM_TN, d, s, group, first, nprob, K, N, act_dtype, math, stream, second);
+    int rc = gemm_entry("qlmx_moe_gemm_tn_pair", GEMM_TN, d, s, group, first, nprob, K, N, act_dtype, math, stream);
+    if(rc) return rc;
+    qlmx_gemm_prob *tmp = (qlmx_gemm_prob *)malloc(sizeof(qlmx_gemm_prob) * (size_t)(nprob > 0 ? nprob : 1));
+    QLMX_REQUIRE(tmp, "qlmx_moe_gemm_tn_pair: out of host memory");
+    for(int i = 0; i < nprob; i++){ tmp[i] = second[i]; tmp[i].C = first[i].C; tmp[i].B = nullptr; tmp[i].beta = 1.0f; }
+    rc = gemm_entry("qlmx_moe_gemm_tn_pair", GEMM_TN, d, s, group, tmp, nprob, K, N, act_dtype, math, stream);
+    free(tmp);
+    return rc;
 }
 /* mg_atb + mg_flush (cudalm.cu:3254-3256) */
 extern "C" int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs, int nprob, int K, int N,

@@ -70,11 +70,14 @@ static int ring_init(void){
     return QLMX_OK;
 }
 
-int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K, int N,
-                         int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot_out){
+/* `second` (tn only, else NULL): problem i continues its contraction over second[i].A and the weight
+ * matrix at second[i].wq / wg. Such a problem is followed in the table by an entry that carries those
+ * three fields and owns no tile (its tile0 is the next problem's), and has `chunk` set to 1. */
+static int upload_problems(const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second, int nprob, int mode, int K, int N,
+                           int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot_out){
     QLMX_REQUIRE(probs && nprob >= 0, "grouped gemm: NULL problem list");
-    if(nprob > QLMX_MAX_PROBLEMS){
-        qlmx_set_error("grouped gemm: %d problems exceed the limit of %d", nprob, QLMX_MAX_PROBLEMS);
+    if(nprob * (second ? 2 : 1) > QLMX_MAX_PROBLEMS){
+        qlmx_set_error("grouped gemm: %d problems exceed the limit of %d", nprob, QLMX_MAX_PROBLEMS / (second ? 2 : 1));
         return QLMX_E_LIMIT;
     }
     int rc = ring_init(); if(rc) return rc;
@@ -110,14 +113,30 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
         DevProb &q = h[n++];
         q.A = p.A; q.B = p.B; q.C = p.C; q.wq = p.wq; q.wg = p.wg; q.M = p.M;
         q.beta = mode == GEMM_NN ? 0.0f : p.beta;
-        q.tile0 = (int)tiles; q.tiles_n = tiles_n; q.chunk = 0; q.flag0 = 0;
+        q.tile0 = (int)tiles; q.tiles_n = tiles_n; q.chunk = second ? 1 : 0; q.flag0 = 0;
         tiles += (long long)((rows + tile_rows - 1) / tile_rows) * tiles_n;
         QLMX_REQUIRE(tiles < (1LL << 30), "grouped gemm: too many tiles");
+        if(second){
+            const qlmx_gemm_prob &p2 = second[i];
+            QLMX_REQUIRE(p2.A && p2.M == p.M, "grouped gemm: problem %d and its continuation differ in rows (%d, %d) or the continuation has no input", i, p.M, p2.M);
+            DevProb &c = h[n++];
+            c = q; c.A = p2.A; c.wq = p2.wq; c.wg = p2.wg; c.tile0 = (int)tiles; c.chunk = 0;
+        }
     }
     (void)stream;
     out->dev = h; out->ntiles = (int)tiles; out->nprob = n;
     *slot_out = slot;
     return QLMX_OK;
+}
+
+int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K, int N,
+                         int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot_out){
+    return upload_problems(probs, nullptr, nprob, mode, K, N, tile_rows, tile_cols, stream, out, slot_out);
+}
+int qlmx_upload_problem_pairs(const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int K, int N,
+                              int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot_out){
+    QLMX_REQUIRE(second, "grouped gemm: NULL continuation list");
+    return upload_problems(first, second, nprob, GEMM_TN, K, N, tile_rows, tile_cols, stream, out, slot_out);
 }
 
 int qlmx_upload_done(int slot, hipStream_t stream){ return guard_launched(g_ring_guard, slot, stream); }

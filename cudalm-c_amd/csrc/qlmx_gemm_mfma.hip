@@ -30,7 +30,8 @@
  * every expert of the call through a flattened (problem, row tile, column tile) list.
  */
 #include "qlmx_gemm.h"
-int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
+int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second,
+                            int nprob, int K, int N, hipStream_t st);
 int qlmx_gemm_nn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
 int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
 
@@ -389,8 +390,10 @@ static int launch_mfma(const signed char *d, const float *s, int group, const ql
     return qlmx_upload_done(slot, st);
 }
 
+/* `second`: tn on bf16 activations only, the continuation of every problem's contraction (else NULL) */
 int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int group,
-                            const qlmx_gemm_prob *probs, int nprob, int K, int N, int act_dtype, hipStream_t st){
+                            const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second, int nprob, int K, int N, int act_dtype, hipStream_t st){
+    QLMX_REQUIRE(!second || (mode == GEMM_TN && act_dtype == QLMX_ACT_BF16), "mfma gemm: continued contractions exist for tn on bf16 activations only");
     /* shapes the tiling assumes; anything else must use QLMX_MATH_F32 */
     QLMX_REQUIRE(N % BN == 0, "mfma gemm: N=%d is not a multiple of %d (use QLMX_MATH_F32)", N, BN);
     if(mode == GEMM_NT) QLMX_REQUIRE(K % 8 == 0, "mfma gemm nt: K=%d is not a multiple of 8 (use QLMX_MATH_F32)", K);
@@ -403,10 +406,14 @@ int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int 
         QLMX_REQUIRE(((uintptr_t)probs[i].A & 15) == 0 && (mode != GEMM_NT || ((uintptr_t)probs[i].B & 15) == 0),
                      "mfma gemm: problem %d operand is not 16-byte aligned", i);
         QLMX_REQUIRE(mode == GEMM_NT || (probs[i].wq & 31ULL) == 0, "mfma gemm: problem %d weight offset not a multiple of 32", i);
+        if(second && probs[i].M != 0){
+            QLMX_REQUIRE(((uintptr_t)second[i].A & 15) == 0, "mfma gemm: problem %d continuation operand is not 16-byte aligned", i);
+            QLMX_REQUIRE((second[i].wq & 31ULL) == 0, "mfma gemm: problem %d continuation weight offset not a multiple of 32", i);
+        }
     }
     QLMX_REQUIRE(mode == GEMM_NT || ((uintptr_t)d & 15) == 0, "mfma gemm: digit array is not 16-byte aligned");
     /* bf16 operands take the direct-to-LDS kernels; fp32 activations need the converting ones */
-    if(mode == GEMM_TN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_tn_lds_launch(d, s, group, probs, nprob, K, N, st);
+    if(mode == GEMM_TN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_tn_lds_launch(d, s, group, probs, second, nprob, K, N, st);
     if(mode == GEMM_NT && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nt_lds_launch(probs, nprob, K, N, st);
     if(mode == GEMM_NN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nn_lds_launch(d, s, group, probs, nprob, K, N, st);
     if(mode == GEMM_NN) return launch_mfma<GEMM_NN, 4, true>(d, s, group, probs, nprob, K, N, act_dtype, st);

@@ -32,6 +32,9 @@ typedef int    i32x4  __attribute__((ext_vector_type(4)));
 #define TN3_A_STAGES 3
 #define TN3_B_OFF (TN3_A_STAGES * TN3_A_BYTES)
 
+/* a continued problem: number of operand pairs (1 or 2) and where the second pair's activations (bytes),
+ * digits (bytes) and scales (floats) lie relative to the first's */
+struct Tn3Seg { int nseg; long long dA, dW, dS; };
 struct Tn3Args { const DevProb *pr; int nprob, ntiles; const signed char *d; const float *s; int gshift; int K, N; };
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -71,7 +74,7 @@ __device__ __forceinline__ void tn3_wait(Tn3Ops &o){
 /* One output tile of NI*64 rows: the four wavefronts 2x2, each NI x 2 accumulators. NI = 2 is the
  * full tile; a last tile with at most 64 rows does half the work. */
 template<int NI>
-__device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, int i0, int j0, unsigned char *lds){
+__device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, const Tn3Seg &sg, int i0, int j0, unsigned char *lds){
     const int rows = P.M;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wi = (wave >> 1) * (NI * 32), wj = (wave & 1) * 64;
@@ -88,13 +91,18 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, int
         srcA[h] = (const char *)P.A + ((size_t)rr * a.K + ko * 8) * 2;
     }
     const int wave_off = __builtin_amdgcn_readfirstlane(wave * 1024);
-    const int steps = a.K / TN3_BK;
+    /* steps of one operand pair, and of the whole contraction; step T of a continued problem reads the
+     * second pair's operands, which lie a constant distance from the first's */
+    const int steps1 = a.K / TN3_BK, steps = steps1 * sg.nseg;
+    auto off_a = [&](int T) -> long long { return T < steps1 ? (long long)T * (TN3_BK * 2) : (long long)(T - steps1) * (TN3_BK * 2) + sg.dA; };
+    auto off_w = [&](int T) -> long long { return T < steps1 ? (long long)T * (TN3_BK / 2) : (long long)(T - steps1) * (TN3_BK / 2) + sg.dW; };
     auto issue_a = [&](int tile, int stage){
         const int tl = tile < steps ? tile : steps - 1;                   /* past the end: the last tile again, into a stage nobody reads */
+        const long long oa = off_a(tl);
         unsigned char *base = lds + stage * TN3_A_BYTES + wave_off;
 #pragma unroll
         for(int h = 0; h < 2 * NI; h++)
-            __builtin_amdgcn_global_load_lds((glb_void *)(srcA[h] + (size_t)tl * (TN3_BK * 2)), (lds_void *)(base + h * 4096), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((glb_void *)(srcA[h] + oa), (lds_void *)(base + h * 4096), 16, 0, 0);
     };
 
     /* ---- weights: thread = (row n, half of the step's 64 digits) ---- */
@@ -108,7 +116,7 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, int
     }
     auto load_w = [&](int tile) -> i32x4 {
         const int tl = tile < steps ? tile : steps - 1;                   /* past the end: re-read the last one, never used */
-        return tn3_gld16(pw + (size_t)tl * (TN3_BK / 2));
+        return tn3_gld16(pw + off_w(tl));
     };
     auto store_w = [&](const i32x4 w, int buf){
         const uint32_t wd[4] = {(uint32_t)w[0], (uint32_t)w[1], (uint32_t)w[2], (uint32_t)w[3]};
@@ -143,8 +151,9 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, int
 #pragma unroll
     for(int j = 0; j < 2; j++) pfold[j] = a.s + P.wg + (size_t)(j0 + wj + j * 32 + fr) * ngroups;
     auto load_scale = [&](int step, int j) -> float {
-        int g = step / spg; g = g < ngroups ? g : ngroups - 1;
-        return tn3_gld4(pfold[j] + g);
+        int g = step / spg; g = g < ngroups * sg.nseg ? g : ngroups * sg.nseg - 1;
+        const long long og = g < ngroups ? (long long)g : (long long)(g - ngroups) + sg.dS;
+        return tn3_gld4(pfold[j] + og);
     };
 
     f32x16 acc[NI][2], part[NI][2];
@@ -191,13 +200,14 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, int
         const uint32_t wbuf = lds_base + (uint32_t)((st + 1) & 1) * TN3_B_BYTES;
         const int tile2 = st + 2 < steps ? st + 2 : steps - 1, stage2 = (st + 2) % TN3_A_STAGES;   /* past the end: the last one again, never used */
         const bool fresh = st % spg == 0, last = (st + 1) % spg == 0;
+        const long long oa2 = off_a(tile2);
         i32x4 wnext; float fn[2];
         i32x4 wv[4];
         auto item = [&](int k){
-            if(k == 0)      wnext = tn3_gld16(pw + (size_t)tile2 * (TN3_BK / 2));
+            if(k == 0)      wnext = tn3_gld16(pw + off_w(tile2));
             else if(k < 3){ if(last) fn[k - 1] = load_scale(st + 1, k - 1); else fn[k - 1] = fs_cur[k - 1]; }   /* a new scale only where a group ends */
             else if(k < 3 + 2 * NI)
-                __builtin_amdgcn_global_load_lds((glb_void *)(srcA[k - 3] + (size_t)tile2 * (TN3_BK * 2)),
+                __builtin_amdgcn_global_load_lds((glb_void *)(srcA[k - 3] + oa2),
                                                  (lds_void *)(lds + stage2 * TN3_A_BYTES + wave_off + (k - 3) * 4096), 16, 0, 0);
             else {
                 /* per 16-byte unit: two conversion items, then its write */
@@ -264,19 +274,30 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
     __shared__ __attribute__((aligned(16))) unsigned char lds[TN3_A_STAGES * TN3_A_BYTES + 2 * TN3_B_BYTES];
     const int t = qx_xcd_tile(blockIdx.x, gridDim.x);
     if(t >= a.ntiles) return;
-    const DevProb P = a.pr[qx_find_problem(a.pr, a.nprob, t)];
+    const int pi = qx_find_problem(a.pr, a.nprob, t);
+    const DevProb P = a.pr[pi];
+    Tn3Seg sg; sg.nseg = 1; sg.dA = 0; sg.dW = 0; sg.dS = 0;
+    if(P.chunk){
+        const DevProb Q = a.pr[pi + 1];
+        sg.nseg = 2;
+        sg.dA = (long long)((const char *)Q.A - (const char *)P.A);
+        sg.dW = ((long long)Q.wq - (long long)P.wq) / 2;
+        sg.dS = (long long)Q.wg - (long long)P.wg;
+    }
     const int lt = t - P.tile0;
     const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
     const int i0 = ti * TN3_BM, j0 = tj * TN3_BN;
-    if(P.M - i0 > 64) tn3_tile<2>(a, P, i0, j0, lds);
-    else              tn3_tile<1>(a, P, i0, j0, lds);
+    if(P.M - i0 > 64) tn3_tile<2>(a, P, sg, i0, j0, lds);
+    else              tn3_tile<1>(a, P, sg, i0, j0, lds);
 }
 
 /* bf16 activations only; N % 128 == 0, K % 64 == 0, group a power of two >= 64 (checked by the caller) */
-int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob,
-                            int K, int N, hipStream_t st){
+int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs,
+                            const qlmx_gemm_prob *second, int nprob, int K, int N, hipStream_t st){
     ProbUpload up; int slot;
-    int rc = qlmx_upload_problems(probs, nprob, GEMM_TN, K, N, TN3_BM, TN3_BN, st, &up, &slot); if(rc) return rc;
+    int rc = second ? qlmx_upload_problem_pairs(probs, second, nprob, K, N, TN3_BM, TN3_BN, st, &up, &slot)
+                    : qlmx_upload_problems(probs, nprob, GEMM_TN, K, N, TN3_BM, TN3_BN, st, &up, &slot);
+    if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;
     Tn3Args a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.d = d; a.s = s; a.K = K; a.N = N;
     a.gshift = 0; while((1 << a.gshift) < group) a.gshift++;

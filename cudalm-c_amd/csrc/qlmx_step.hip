@@ -172,8 +172,11 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
         *(uint32_t *)(a.d + (q >> 1)) = dnew;
         *(uint2 *)(a.r + q) = make_uint2(rn0, rn1);
         if(a.P){
-            *(float4 *)(a.P + pof + e0)     = make_float4(pv[0], pv[1], pv[2], pv[3]);
-            *(float4 *)(a.P + pof + e0 + 4) = make_float4(pv[4], pv[5], pv[6], pv[7]);
+            /* the rendered view is not read again by this launch: written past the caches */
+            typedef float f4 __attribute__((ext_vector_type(4)));
+            f4 p0 = {pv[0], pv[1], pv[2], pv[3]}, p1 = {pv[4], pv[5], pv[6], pv[7]};
+            __builtin_nontemporal_store(p0, (f4 *)(a.P + pof + e0));
+            __builtin_nontemporal_store(p1, (f4 *)(a.P + pof + e0 + 4));
         }
         am = qx_row16_max(am); vm = qx_row16_max(vm);
         const float ms = am > 0.0f ? am / 127.0f : 1e-12f;

@@ -305,4 +305,36 @@ static void mg_run(std::vector<MgItem> &v){
     }
     v.clear();
 }
-void mg_flush(void){ mg_run(g_q[0]); mg_run(g_q[1]); mg_run(g_q[2]); }
+/* A queue-1 problem (tn, beta = 1) whose output a queue-0 tn problem of the same shape writes is that
+ * problem's second half (cudalm.cu:4365-4366): on the MFMA path the two run as one continued
+ * contraction per (K, N) instead of two launches with the output stored and read back in between. */
+static void mg_run_pairs(void){
+    if(g_mg_act != QLMX_ACT_BF16 || g_mg_math != QLMX_MATH_MFMA) return;
+    std::vector<MgItem> &v0 = g_q[0], &v1 = g_q[1];
+    std::vector<int> mate(v1.size(), -1);
+    std::vector<char> used(v0.size(), 0);
+    bool any = false;
+    for(size_t j = 0; j < v1.size(); j++){
+        if(v1[j].mode != 1 || v1[j].p.beta != 1.0f || v1[j].p.M == 0) continue;
+        for(size_t i = 0; i < v0.size(); i++)
+            if(!used[i] && v0[i].mode == 1 && v0[i].p.C == v1[j].p.C && v0[i].p.M == v1[j].p.M && v0[i].K == v1[j].K && v0[i].N == v1[j].N){
+                mate[j] = (int)i; used[i] = 1; any = true; break;
+            }
+    }
+    if(!any) return;
+    std::vector<char> done(v1.size(), 0);
+    for(size_t j = 0; j < v1.size(); j++){
+        if(done[j] || mate[j] < 0) continue;
+        std::vector<qlmx_gemm_prob> first, second;
+        for(size_t k = j; k < v1.size() && first.size() < QLMX_MAX_PROBLEMS / 2; k++)
+            if(!done[k] && mate[k] >= 0 && v1[k].K == v1[j].K && v1[k].N == v1[j].N){ first.push_back(v0[mate[k]].p); second.push_back(v1[k].p); done[k] = 1; }
+        const int rc = qlmx_moe_gemm_tn_pair(g_mg_q->d, g_mg_q->s, g_mg_q->group, first.data(), second.data(), (int)first.size(),
+                                             v1[j].K, v1[j].N, g_mg_act, g_mg_math, NULL);
+        if(rc != QLMX_OK){ fprintf(stderr, "grouped GEMM error %d at mg grouped (pairs): %s\n", rc, qlmx_last_error()); exit(1); }
+    }
+    std::vector<MgItem> r0, r1;
+    for(size_t i = 0; i < v0.size(); i++) if(!used[i]) r0.push_back(v0[i]);
+    for(size_t j = 0; j < v1.size(); j++) if(!done[j]) r1.push_back(v1[j]);
+    v0.swap(r0); v1.swap(r1);
+}
+void mg_flush(void){ mg_run_pairs(); mg_run(g_q[0]); mg_run(g_q[1]); mg_run(g_q[2]); }

@@ -3,7 +3,7 @@
  * 2*dmax+1 levels per group; one Integer AdamW step against a scalar host restatement that reuses
  * the host helpers (digits/residuals must agree bit for bit here because both sides are compiled
  * without FMA contraction); a save/load round trip; an expert FFN forward through the grouped GEMM
- * queue against a host triple loop. Prints one line per check and exits 0 only if all pass. */
+ * queue against a host triple loop, and the paired input-gradient GEMMs of w1 and w3. Prints one line per check and exits 0 only if all pass. */
 #include "qlm_host.h"
 #include <math.h>
 #include <stdio.h>
@@ -135,6 +135,32 @@ int main(){
         Yref[(size_t)m * F + f] = (float)acc; }
     double num = 0, den = 0; for(size_t i = 0; i < Y.size(); i++){ double dlt = (double)Y[i] - Yref[i]; num += dlt * dlt; den += (double)Yref[i] * Yref[i]; }
     check("moe expert fwd (mg_ab) rel-err", sqrt(num / den), 1e-3);
+
+    /* (e) input gradient of w1 and w3 through the queue as the reference issues it (beta 0, then beta 1
+     * on the same output), bf16 activations on the matrix cores: the flush runs each pair as one launch */
+    {
+        auto bf16 = [](float f) -> unsigned short { unsigned u; memcpy(&u, &f, 4); u += 0x7FFFu + ((u >> 16) & 1u); return (unsigned short)(u >> 16); };
+        auto f32 = [](unsigned short h) -> float { unsigned u = (unsigned)h << 16; float f; memcpy(&f, &u, 4); return f; };
+        std::vector<unsigned short> dg((size_t)N * F), du((size_t)N * F);
+        for(auto &v : dg) v = bf16(nrand());
+        for(auto &v : du) v = bf16(nrand());
+        std::vector<float> dX((size_t)N * D, 0.f);
+        void *dgd = dmalloc(dg.size() * 2), *dud = dmalloc(du.size() * 2); float *dXd = (float *)dmalloc(dX.size() * 4);
+        qlmx_memcpy_h2d(dgd, dg.data(), dg.size() * 2); qlmx_memcpy_h2d(dud, du.data(), du.size() * 2);
+        mg_bind(&q, Pd, QLMX_ACT_BF16, QLMX_MATH_MFMA);
+        for(int e = 0; e < E; e++){ int ne = off[e + 1] - off[e]; if(!ne) continue;
+            mg_abt_b((const unsigned short *)dgd + (size_t)off[e] * F, Pd + 16 + (size_t)e * D * F, dXd + (size_t)off[e] * D, ne, F, D, 0.0f);
+            mg_abt_b((const unsigned short *)dud + (size_t)off[e] * F, Pd + 16 + nw + (size_t)e * D * F, dXd + (size_t)off[e] * D, ne, F, D, 1.0f); }
+        mg_flush(); qlmx_sync(NULL);
+        qlmx_memcpy_d2h(dX.data(), dXd, dX.size() * 4);
+        double num2 = 0, den2 = 0;
+        for(int e = 0; e < E; e++) for(int m = off[e]; m < off[e + 1]; m++) for(int k = 0; k < D; k++){
+            double acc = 0;
+            for(int f = 0; f < F; f++) acc += (double)f32(dg[(size_t)m * F + f]) * Pr[16 + (size_t)e * D * F + (size_t)k * F + f]
+                                            + (double)f32(du[(size_t)m * F + f]) * Pr[16 + nw + (size_t)e * D * F + (size_t)k * F + f];
+            const double dlt = (double)dX[(size_t)m * D + k] - acc; num2 += dlt * dlt; den2 += acc * acc; }
+        check("moe dgrad w1+w3 (mg_abt_b pair) rel-err", sqrt(num2 / den2), 1e-3);
+    }
     qlm_free(&q);
     printf(ok_all ? "[selftest] ALL PASS\n" : "[selftest] FAILED\n");
     return ok_all ? 0 : 1;

@@ -159,6 +159,16 @@ int qlmx_moe_gemm_nn(const signed char *d, const float *s, int group,
 int qlmx_moe_gemm_tn(const signed char *d, const float *s, int group,
                      const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
                      int act_dtype, int math, void *stream);
+/* The two mg_abt_b calls on one output (cudalm.cu:4365-4366: dXp = dgp . w1^T with beta 0, then
+ * dXp += dup . w3^T with beta 1) as one call: problem i computes
+ *   C = first[i].A . W(first[i].wq)^T + second[i].A . W(second[i].wq)^T   (+ C when first[i].beta = 1).
+ * second[i] supplies A, wq, wg and must repeat M; its B, C and beta are ignored. On bf16 activations
+ * with QLMX_MATH_MFMA both contractions run in one launch and the sum stays in the accumulators;
+ * every other combination issues the two launches the reference would. At most QLMX_MAX_PROBLEMS / 2
+ * problems. */
+int qlmx_moe_gemm_tn_pair(const signed char *d, const float *s, int group,
+                          const qlmx_gemm_prob *first_host, const qlmx_gemm_prob *second_host, int nprob,
+                          int K, int N, int act_dtype, int math, void *stream);
 /* nt: no weight operand; both inputs are activations, fp32 result. beta = 1 reproduces the
  * reference's accumulation into a zeroed G; beta = 0 saves the read when G is known to be fresh. */
 int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs_host, int nprob, int K, int N,

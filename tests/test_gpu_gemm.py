@@ -188,6 +188,70 @@ def test_mfma_tn_many_rows_per_expert(q, orc, beta):
     assert orc.relerr(got, want) < TOL_MFMA
 
 
+def _pair_case(q, orc, rowsM, K, N, act, math, beta, seed=7, swap=False):
+    """C = A1 . W1^T + A2 . W2^T (+ C) per expert through qlmx_moe_gemm_tn_pair; W1 and W2 are the two halves
+    of one digit array (`swap`: the second operand pair lies before the first in memory)."""
+    import torch
+    E = len(rowsM); tot = sum(rowsM)
+    off = np.concatenate([[0], np.cumsum(rowsM)]).astype(int)
+    bf = act == pkg.ACT_BF16
+    d, s, P = make_weights(orc, seed, 2 * E, N, K)
+    A = [orc.normal(tot * K, seed, 20 + i) for i in range(2)]
+    if bf:
+        A = [orc.bf16_round(a) for a in A]
+    C0 = orc.normal(tot * N, seed, 12)
+    both = dev(np.concatenate(A))
+    pb = to_bf16_bits(both) if bf else both
+    esz = 2 if bf else 4
+    dC, dd, ds = dev(C0.copy()), dev(d), dev(s)
+    wsel = [1, 0] if swap else [0, 1]
+    def items(i, b):
+        w0 = wsel[i] * E
+        return [(pb.data_ptr() + (wsel[i] * tot + off[e]) * K * esz, None, dC.data_ptr() + off[e] * N * 4 if i == 0 else None,
+                 (w0 + e) * N * K, (w0 + e) * N * K // 128, rowsM[e], b) for e in range(E)]
+    q.gemm_tn_pair(dd, ds, 128, q.problems(items(0, beta)), q.problems(items(1, 0.0)), E, K, N, act, math)
+    torch.cuda.synchronize()
+    want = C0.copy()
+    for e in range(E):
+        if not rowsM[e]:
+            continue
+        for i in range(2):
+            w = P[(wsel[i] * E + e) * N * K:(wsel[i] * E + e + 1) * N * K]
+            orc.gemm_tn(A[wsel[i]][off[e] * K:], w, want[off[e] * N:off[e + 1] * N], rowsM[e], K, N, beta if i == 0 else 1.0)
+    return dC.cpu().numpy(), want
+
+
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+@pytest.mark.parametrize("swap", [False, True])
+def test_mfma_tn_pair_one_launch(q, orc, beta, swap):
+    """The two input-gradient GEMMs that share an output, as one continued contraction: ragged experts,
+    an empty one, last tiles of 1..128 rows, either order of the operand pairs in memory."""
+    got, want = _pair_case(q, orc, [300, 0, 64, 1, 129, 517], 256, 384, pkg.ACT_BF16, pkg.MATH_MFMA, beta, swap=swap)
+    assert orc.relerr(got, want) < TOL_MFMA
+
+
+def test_mfma_tn_pair_layer_shape(q, orc):
+    got, want = _pair_case(q, orc, [700, 40, 333], 2048, 768, pkg.ACT_BF16, pkg.MATH_MFMA, 0.0, seed=8)
+    assert orc.relerr(got, want) < TOL_MFMA
+
+
+@pytest.mark.parametrize("act,math", [("f32", "f32"), ("bf16", "f32"), ("f32", "mfma")])
+def test_tn_pair_other_paths_take_two_launches(q, orc, act, math):
+    a = pkg.ACT_BF16 if act == "bf16" else pkg.ACT_F32
+    m = pkg.MATH_MFMA if math == "mfma" else pkg.MATH_F32
+    got, want = _pair_case(q, orc, [70, 0, 130], 256, 128, a, m, 1.0, seed=9)
+    assert orc.relerr(got, want) < (TOL_MFMA if math == "mfma" else TOL_F32)
+
+
+def test_tn_pair_rejects_mismatched_rows(q):
+    import torch
+    z = torch.zeros(1 << 16, device="cuda")
+    zb = torch.zeros(1 << 16, dtype=torch.int8, device="cuda")
+    a = q.problems([(z, None, z, 0, 0, 64, 0.0)]); b = q.problems([(z, None, None, 0, 0, 32, 0.0)])
+    with pytest.raises(pkg.QlmxError, match="rows"):
+        q.gemm_tn_pair(zb, z, 128, a, b, 1, 128, 128, pkg.ACT_BF16, pkg.MATH_MFMA)
+
+
 @pytest.mark.parametrize("beta", [0.0, 1.0])
 def test_mfma_nt_split_contraction(q, orc, beta):
     """One expert with far more rows than the others: its contraction is cut into slices that add up

@@ -433,9 +433,9 @@ def cpu_gemm(args):
 
 # HBM bytes from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the 1 GiB copy calibration); the runs,
 # counter values and scale factors are in profiles/*.txt. adamw: per launch. train: per step, i.e. summed over
-# the step's 7 launches (1221 MiB read + 1134 MiB written). decode: per launch = per layer at T=16
+# the step's 6 launches (1182 MiB read + 1086 MiB written). decode: per launch = per layer at T=16
 # (56.2 MiB read + 4.5 MiB written).
-PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.47e9, "decode": 6.37e7}
+PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.38e9, "decode": 6.37e7}
 
 
 def main():

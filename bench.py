@@ -14,6 +14,8 @@ Each workload reports its own roofline object; the top-level `value`/`roofline` 
 workload that ran in the order train, decode, adamw. `cpu_baseline` times the reference's own CPU
 backend (oracle/_ref, kind "reference") or the repository's C restatement (kind "port") on a bounded
 sample on this host's cores; it is a reported baseline, not the target.
+Defaults: 30 warm-up and 100 timed steps. The device takes some 20 ms of load to reach the clock it then
+holds; with 3 + 20 steps of 1 ms the timed region lies inside that ramp and reads 8 % low.
 """
 import argparse
 import json
@@ -31,8 +33,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train", "train5", "codec", "glue", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--adamw-weights", type=int, default=120 * 2 ** 20)

@@ -124,13 +124,15 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
     p_d3 = P([(a, b, c, wq, wg, m, 1.0) for (a, b, c, wq, wg, m, _) in it3])
     p_g2 = P(probs(ap, F, dyp, D, G, 0, o2, True))
     p_g13 = P(probs(Xp, D, dgp, F, G, 0, o1, True) + probs(Xp, D, dup, F, G, 0, o3, True))
+    # the order of moe_forward / moe_backward (cudalm.cu:4211-4225, 4333-4335, 4362-4366): each backward flush
+    # holds the weight gradient and the input gradient of the same operands
     calls = [
         ("fwd w1,w3 (nn)", lambda: q.gemm_nn(d, s, group, p_w13, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream), 2),
         ("fwd w2 (nn)", lambda: q.gemm_nn(d, s, group, p_w2, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
-        ("dgrad w2 (tn)", lambda: q.gemm_tn(d, s, group, p_d2, E, D, F, ACT_BF16, MATH_MFMA, stream), 1),
-        ("dgrad w1,w3 (tn pair)", lambda: q.gemm_tn_pair(d, s, group, p_d1, p_d3, E, F, D, ACT_BF16, MATH_MFMA, stream), 2),
         ("wgrad w2 (nt)", lambda: q.gemm_nt(p_g2, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
+        ("dgrad w2 (tn)", lambda: q.gemm_tn(d, s, group, p_d2, E, D, F, ACT_BF16, MATH_MFMA, stream), 1),
         ("wgrad w1,w3 (nt)", lambda: q.gemm_nt(p_g13, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream), 2),
+        ("dgrad w1,w3 (tn pair)", lambda: q.gemm_tn_pair(d, s, group, p_d1, p_d3, E, F, D, ACT_BF16, MATH_MFMA, stream), 2),
     ]
     unit = 2.0 * rows * D * F            # flops of one expert GEMM over all rows
 

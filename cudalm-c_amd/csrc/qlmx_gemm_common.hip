@@ -12,19 +12,36 @@
 
 /* Reuse guard of a ring: an event behind every launch costs about 6 us of idle GPU between that kernel
  * and the next (the record makes the end of the kernel visible to the host), so the slots are guarded
- * by segments instead: when the last slot of a segment has been launched, one event is recorded on
- * each stream the segment's launches went to, and those events are waited for when the ring comes
- * round to the segment's first slot again -- three segments' worth of launches later. */
+ * by segments instead: when the ring moves on to the next segment, one event is recorded on each stream
+ * the segment's launches went to, and those events are waited for when the ring comes round to the
+ * segment's first slot again -- three segments' worth of launches later. Closing a segment on the way
+ * out covers every launch made from it, also when a call that took its last slot returned without
+ * launching (an error, or nothing but empty problems). */
 #define GUARD_STREAMS 4
 struct RingSeg { hipStream_t st[GUARD_STREAMS]; hipEvent_t ev[GUARD_STREAMS]; int nst, nrec; bool made; };
 struct RingGuard { int nslots, per_seg, next; RingSeg seg[8]; };
 
+static int guard_close(RingSeg &sg){
+    sg.nrec = 0;
+    for(int i = 0; i < sg.nst; i++){
+        if(hipEventRecord(sg.ev[sg.nrec], sg.st[i]) == hipSuccess) sg.nrec++;
+        else {
+            /* e.g. a stream destroyed since its launch: fall back to waiting for the whole device */
+            (void)hipGetLastError();
+            QLMX_HIP(hipDeviceSynchronize(), "table ring device wait");
+        }
+    }
+    sg.nst = 0;
+    return QLMX_OK;
+}
 static int guard_take(RingGuard &g, int *slot_out){
     const int slot = g.next; g.next = (g.next + 1) % g.nslots;
-    RingSeg &sg = g.seg[slot / g.per_seg];
     if(slot % g.per_seg == 0){
+        const int nseg = g.nslots / g.per_seg, cur = slot / g.per_seg;
+        int rc = guard_close(g.seg[(cur + nseg - 1) % nseg]); if(rc) return rc;
+        RingSeg &sg = g.seg[cur];
         for(int i = 0; i < sg.nrec; i++) QLMX_HIP(hipEventSynchronize(sg.ev[i]), "table ring wait");
-        sg.nrec = 0; sg.nst = 0;
+        sg.nrec = 0;
     }
     *slot_out = slot;
     return QLMX_OK;
@@ -44,17 +61,6 @@ static int guard_launched(RingGuard &g, int slot, hipStream_t stream){
             return QLMX_OK;
         }
         sg.st[sg.nst++] = stream;
-    }
-    if(slot % g.per_seg == g.per_seg - 1){
-        sg.nrec = 0;
-        for(int i = 0; i < sg.nst; i++){
-            if(hipEventRecord(sg.ev[sg.nrec], sg.st[i]) == hipSuccess) sg.nrec++;
-            else {
-                /* e.g. a stream destroyed since its launch: fall back to waiting for the whole device */
-                (void)hipGetLastError();
-                QLMX_HIP(hipDeviceSynchronize(), "table ring device wait");
-            }
-        }
     }
     return QLMX_OK;
 }

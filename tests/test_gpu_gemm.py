@@ -294,7 +294,8 @@ def test_mfma_more_problems_than_lanes(q, orc, mode):
 def test_mfma_table_ring_wraps(q, orc):
     """150 grouped launches without a synchronisation between them go more than twice round the ring of
     problem tables (and four times round the unit-table ring of the weight gradient); a launch whose
-    table had been overwritten too early would compute on the wrong pointers."""
+    table had been overwritten too early would compute on the wrong pointers. Calls that take a slot without
+    launching (nothing but empty problems; an error found while the table is written) are mixed in."""
     import torch
     E, rows, K, N = 3, [70, 0, 33], 64, 128
     tot = sum(rows)
@@ -316,6 +317,12 @@ def test_mfma_table_ring_wraps(q, orc):
         q.gemm_nt(q.problems([(pa.data_ptr() + off[e] * K * 2, pb.data_ptr() + off[e] * N * 2, c2.data_ptr() + e * K * N * 4, 0, 0,
                                rows[e], 0.0) for e in range(E)]), E, K, N, pkg.ACT_BF16, pkg.MATH_MFMA)
         outs.append((c1, c2))
+        if it % 5 == 4:
+            # calls that take a table slot and launch nothing: only empty problems, and an error found after
+            # the slot was taken (a pair whose halves differ in rows is caught earlier, so a NULL input is used)
+            q.gemm_nn(dd, ds, 128, q.problems([(pa, None, c1, 0, 0, 0, 0.0)]), 1, K, N, pkg.ACT_BF16, pkg.MATH_MFMA)
+            with pytest.raises(pkg.QlmxError):
+                q.gemm_nn(dd, ds, 128, q.problems([(pa, None, c1, 0, 0, 8, 0.0), (None, None, c1, 0, 0, 8, 0.0)]), 2, K, N, pkg.ACT_BF16, pkg.MATH_MFMA)
     torch.cuda.synchronize()
     for c1, c2 in outs:
         assert orc.relerr(c1.cpu().numpy(), want_nn) < TOL_MFMA and orc.relerr(c2.cpu().numpy(), want_nt) < TOL_MFMA

@@ -250,6 +250,11 @@ def test_tn_pair_rejects_mismatched_rows(q):
     a = q.problems([(z, None, z, 0, 0, 64, 0.0)]); b = q.problems([(z, None, None, 0, 0, 32, 0.0)])
     with pytest.raises(pkg.QlmxError, match="rows"):
         q.gemm_tn_pair(zb, z, 128, a, b, 1, 128, 128, pkg.ACT_BF16, pkg.MATH_MFMA)
+    # a pair needs two table entries: half as many problems as a plain call
+    many = q.problems([(z, None, z, 0, 0, 1, 0.0)] * 513)
+    with pytest.raises(pkg.QlmxError, match="limit"):
+        q.gemm_tn_pair(zb, z, 128, many, many, 513, 128, 128, pkg.ACT_BF16, pkg.MATH_MFMA)
+    q.gemm_tn_pair(zb, z, 128, a, a, 0, 128, 128, pkg.ACT_BF16, pkg.MATH_MFMA)       # no problems: nothing to do
 
 
 @pytest.mark.parametrize("beta", [0.0, 1.0])

@@ -116,6 +116,15 @@ def test_train_size_mfma_vs_fp32_kernels_and_properties(q, orc, E, D, F, rows):
     q.gemm_tn(d, s, 128, probs(dY, F, None, 0, dX1, D), E, F, D, pkg.ACT_BF16, pkg.MATH_MFMA)
     q.gemm_tn(d, s, 128, probs(dY, F, None, 0, dX2, D), E, F, D, pkg.ACT_BF16, pkg.MATH_F32)
     assert rel(dX1, dX2) < 1e-3
+    # the paired input gradient (one continued contraction) against two calls, the second accumulating
+    dY2 = torch.randn(rows * F, device="cuda", generator=gen).to(torch.bfloat16)
+    dX3 = torch.zeros(rows * D, device="cuda"); dX4 = torch.zeros(rows * D, device="cuda")
+    q.gemm_tn_pair(d, s, 128, probs(dY, F, None, 0, dX3, D), probs(dY2, F, None, 0, dX3, D), E, F, D, pkg.ACT_BF16, pkg.MATH_MFMA)
+    q.gemm_tn(d, s, 128, probs(dY, F, None, 0, dX4, D), E, F, D, pkg.ACT_BF16, pkg.MATH_MFMA)
+    acc = q.problems([(dY2.data_ptr() + int(off[e]) * F * 2, None, dX4.data_ptr() + int(off[e]) * D * 4, e * D * F, e * D * F // 128, int(cnt[e]), 1.0)
+                      for e in range(E)])
+    q.gemm_tn(d, s, 128, acc, E, F, D, pkg.ACT_BF16, pkg.MATH_MFMA)
+    assert rel(dX3, dX4) < 1e-6
     # wgrad nt: G[D, F] += X^T dY per expert
     G1 = torch.zeros(nw, device="cuda"); G2 = torch.zeros(nw, device="cuda")
     q.gemm_nt(probs(X, D, dY, F, G1, 0, True), E, D, F, pkg.ACT_BF16, pkg.MATH_MFMA)

@@ -145,6 +145,15 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
     for name, fn, ng in calls:
         t1 = timed(torch, fn, max(5, args.steps // 2), 2)
         per[name] = {"ms": t1["event_ms_avg"], "tflops": ng * unit / (t1["event_ms_avg"] * 1e-3) / 1e12}
+    # beside the step: the forward's gate|up GEMMs with the SwiGLU in their epilogue, against the two-launch form
+    act = torch.empty(rows * F, dtype=torch.bfloat16, device=dev)
+    g_gate = P(probs(Xp, D, None, 0, gp, F, o1))
+    g_up = P([(None, act.data_ptr() + off[e] * F * 2, up.data_ptr() + off[e] * F * 4, o3 + e * D * F, (o3 + e * D * F) // group, int(cnt[e]), 0.0)
+              for e in range(E)])
+    extra = {}
+    for name, fn in [("fwd w1,w3 + SwiGLU, one launch", lambda: q.gemm_nn_swiglu(d, s, group, g_gate, g_up, E, D, F, ACT_BF16, MATH_MFMA, stream)),
+                     ("SwiGLU kernel alone", lambda: q.swiglu(gp, up, act, rows * F, ACT_BF16, stream))]:
+        extra[name] = {"ms": timed(torch, fn, max(5, args.steps // 2), 2)["event_ms_avg"]}
     flops = 9 * unit
     tf = flops / (tm["event_ms_avg"] * 1e-3) / 1e12
     dom = max(per, key=lambda k: per[k]["ms"])
@@ -152,7 +161,7 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
         "workload": "%s: E=%d top-%d D=%d F=%d, %d bf16 tokens -> %d expert rows, Zipf(1.1) load (max %d, min %d rows); "
                     "fwd+dgrad+wgrad = 9 grouped GEMMs in 6 launches" % (label, E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min())),
         "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tm["wall_ms"], "dtype": "bf16",
-        "kernel_ms": tm, "per_launch": per, "gflop_per_step": flops / 1e9,
+        "kernel_ms": tm, "per_launch": per, "beside_the_step": extra, "gflop_per_step": flops / 1e9,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": None, "kernel": "k_gemm_nn_lds, k_gemm_tn_lds, k_gemm_nt_lds (all 6 launches; slowest: %s)" % dom,
                      "note": "algorithmic flops only; the forward issues two MFMAs per product (bf16 hi+lo weight split)"},

@@ -70,6 +70,7 @@ SIGNATURES = {
     "qlmx_moe_gemm_nn": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_tn": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_tn_pair": (c_i, [c_vp, c_vp, c_i, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_moe_gemm_nn_swiglu": (c_i, [c_vp, c_vp, c_i, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_nt": (c_i, [c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_decode_forward": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_step_touched": (c_i, [c_vp] * 10 + [c_i, c_i, c_i, c_f, c_f, c_f, c_f, c_f, c_f, c_f, c_u64, c_u64, c_vp, c_i, c_vp]),
@@ -153,6 +154,9 @@ class Qlmx:
 
     def gemm_tn_pair(self, d, s, group, first, second, nprob, K, N, act=ACT_F32, math=MATH_F32, stream=None):
         self.call("qlmx_moe_gemm_tn_pair", d, s, group, C.addressof(first), C.addressof(second), nprob, K, N, act, math, stream)
+
+    def gemm_nn_swiglu(self, d, s, group, gate, up, nprob, K, N, act=ACT_F32, math=MATH_F32, stream=None):
+        self.call("qlmx_moe_gemm_nn_swiglu", d, s, group, C.addressof(gate), C.addressof(up), nprob, K, N, act, math, stream)
 
     def gemm_nt(self, probs, nprob, K, N, act=ACT_F32, math=MATH_F32, stream=None):
         self.call("qlmx_moe_gemm_nt", C.addressof(probs), nprob, K, N, act, math, stream)

@@ -24,10 +24,11 @@ struct DevProb {
 struct ProbUpload { const DevProb *dev; int ntiles; int nprob; };
 int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K, int N,
                          int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot);
-/* tn only: problem i continues its contraction over second[i].A and the weights at second[i].wq / wg
- * (same M, K, N). In the table such a problem has chunk = 1 and is followed by an entry holding those
- * fields that owns no tile. */
-int qlmx_upload_problem_pairs(const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int K, int N,
+/* Problems with a second half (same M, K, N). tn: the contraction continues over second[i].A and the
+ * weights at second[i].wq / wg. nn: a tile holds columns of both weight matrices; second[i] gives the other
+ * matrix (wq, wg), its output (C) and the combined output (B). In the table such a problem has chunk = 1 and
+ * is followed by an entry holding the second half's fields that owns no tile. */
+int qlmx_upload_problem_pairs(const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int mode, int K, int N,
                               int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot);
 int qlmx_upload_done(int slot, hipStream_t stream);
 

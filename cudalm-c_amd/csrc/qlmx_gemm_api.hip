@@ -72,6 +72,46 @@ extern "C" int qlmx_moe_gemm_tn_pair(const signed char *d, const float *s, int g
     free(tmp);
     return rc;
 }
+int qlmx_gemm_nn_swiglu_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *gate,
+                                   const qlmx_gemm_prob *up, int nprob, int K, int N, hipStream_t st);
+extern "C" int qlmx_swiglu(const float *G, const float *U, void *O, size_t n, int out_dtype, void *stream);
+
+/* The gate and up GEMMs of moe_forward and the SwiGLU between them and the down GEMM (cudalm.cu:4211-4215:
+ * mg_ab(Xp, w1_e, gp), mg_ab(Xp, w3_e, up), mg_flush, e_swig(gp, up, ap)) as one call. Problem i computes
+ *   gp = A . W(gate[i].wq), up = A . W(up[i].wq), act = bf16(gp * sigmoid(gp) * up)
+ * with A = gate[i].A [M, K] and the outputs at gate[i].C, up[i].C (fp32 [M, N]) and up[i].B (bf16 [M, N]).
+ * On bf16 activations with MFMA math a tile holds 64 columns of both matrices and the SwiGLU is applied to
+ * the accumulators; every other combination runs the two GEMM launches and one SwiGLU launch per problem. */
+extern "C" int qlmx_moe_gemm_nn_swiglu(const signed char *d, const float *s, int group,
+                                       const qlmx_gemm_prob *gate, const qlmx_gemm_prob *up, int nprob, int K, int N,
+                                       int act_dtype, int math, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(gate && up && nprob >= 0, "qlmx_moe_gemm_nn_swiglu: NULL problem list");
+    for(int i = 0; i < nprob; i++){
+        QLMX_REQUIRE(up[i].M == gate[i].M, "qlmx_moe_gemm_nn_swiglu: problem %d has %d and %d rows", i, gate[i].M, up[i].M);
+        QLMX_REQUIRE(gate[i].M == 0 || (gate[i].A && gate[i].C && up[i].C && up[i].B), "qlmx_moe_gemm_nn_swiglu: problem %d has a NULL pointer", i);
+    }
+    if(act_dtype == QLMX_ACT_BF16 && math == QLMX_MATH_MFMA && N % 64 == 0 && K % 32 == 0 && group >= 64 && (group & (group - 1)) == 0 &&
+       nprob * 2 <= QLMX_MAX_PROBLEMS){
+        QLMX_REQUIRE(d && s && ((uintptr_t)d & 15) == 0, "qlmx_moe_gemm_nn_swiglu: digits and scales must be given, digits 16-byte aligned");
+        for(int i = 0; i < nprob; i++){
+            QLMX_REQUIRE(((uintptr_t)gate[i].A & 15) == 0 && ((uintptr_t)up[i].B & 1) == 0, "qlmx_moe_gemm_nn_swiglu: problem %d operand alignment", i);
+            QLMX_REQUIRE(gate[i].wq % (unsigned long long)group == 0 && up[i].wq % (unsigned long long)group == 0 &&
+                         (gate[i].wq & 31ULL) == 0 && (up[i].wq & 31ULL) == 0, "qlmx_moe_gemm_nn_swiglu: problem %d weight offset alignment", i);
+        }
+        return qlmx_gemm_nn_swiglu_lds_launch(d, s, group, gate, up, nprob, K, N, (hipStream_t)stream);
+    }
+    rc = gemm_entry("qlmx_moe_gemm_nn_swiglu", GEMM_NN, d, s, group, gate, nprob, K, N, act_dtype, math, stream); if(rc) return rc;
+    qlmx_gemm_prob *tmp = (qlmx_gemm_prob *)malloc(sizeof(qlmx_gemm_prob) * (size_t)(nprob > 0 ? nprob : 1));
+    QLMX_REQUIRE(tmp, "qlmx_moe_gemm_nn_swiglu: out of host memory");
+    for(int i = 0; i < nprob; i++){ tmp[i] = up[i]; tmp[i].A = gate[i].A; tmp[i].B = nullptr; }
+    rc = gemm_entry("qlmx_moe_gemm_nn_swiglu", GEMM_NN, d, s, group, tmp, nprob, K, N, act_dtype, math, stream);
+    free(tmp);
+    for(int i = 0; i < nprob && !rc; i++)
+        if(gate[i].M > 0) rc = qlmx_swiglu(gate[i].C, up[i].C, (void *)up[i].B, (size_t)gate[i].M * N, QLMX_ACT_BF16, stream);
+    return rc;
+}
+
 /* mg_atb + mg_flush (cudalm.cu:3254-3256) */
 extern "C" int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs, int nprob, int K, int N,
                                 int act_dtype, int math, void *stream){

@@ -76,9 +76,11 @@ static int ring_init(void){
     return QLMX_OK;
 }
 
-/* `second` (tn only, else NULL): problem i continues its contraction over second[i].A and the weight
- * matrix at second[i].wq / wg. Such a problem is followed in the table by an entry that carries those
- * three fields and owns no tile (its tile0 is the next problem's), and has `chunk` set to 1. */
+/* `second` (else NULL): problem i has a second half. tn: it continues its contraction over second[i].A
+ * and the weight matrix at second[i].wq / wg. nn: its tiles hold columns of two weight matrices, the
+ * second at second[i].wq / wg with its output at second[i].C and the combined output at second[i].B.
+ * Such a problem is followed in the table by an entry that carries the second half's fields and owns
+ * no tile (its tile0 is the next problem's), and has `chunk` set to 1. */
 static int upload_problems(const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second, int nprob, int mode, int K, int N,
                            int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot_out){
     QLMX_REQUIRE(probs && nprob >= 0, "grouped gemm: NULL problem list");
@@ -124,9 +126,10 @@ static int upload_problems(const qlmx_gemm_prob *probs, const qlmx_gemm_prob *se
         QLMX_REQUIRE(tiles < (1LL << 30), "grouped gemm: too many tiles");
         if(second){
             const qlmx_gemm_prob &p2 = second[i];
-            QLMX_REQUIRE(p2.A && p2.M == p.M, "grouped gemm: problem %d and its continuation differ in rows (%d, %d) or the continuation has no input", i, p.M, p2.M);
+            QLMX_REQUIRE(p2.M == p.M, "grouped gemm: problem %d and its second half differ in rows (%d, %d)", i, p.M, p2.M);
+            QLMX_REQUIRE(mode == GEMM_TN ? p2.A != nullptr : (p2.B != nullptr && p2.C != nullptr), "grouped gemm: the second half of problem %d lacks a pointer", i);
             DevProb &c = h[n++];
-            c = q; c.A = p2.A; c.wq = p2.wq; c.wg = p2.wg; c.tile0 = (int)tiles; c.chunk = 0;
+            c = q; c.A = p2.A; c.B = p2.B; c.C = p2.C; c.wq = p2.wq; c.wg = p2.wg; c.tile0 = (int)tiles; c.chunk = 0;
         }
     }
     (void)stream;
@@ -139,10 +142,10 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
                          int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot_out){
     return upload_problems(probs, nullptr, nprob, mode, K, N, tile_rows, tile_cols, stream, out, slot_out);
 }
-int qlmx_upload_problem_pairs(const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int K, int N,
+int qlmx_upload_problem_pairs(const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int mode, int K, int N,
                               int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot_out){
-    QLMX_REQUIRE(second, "grouped gemm: NULL continuation list");
-    return upload_problems(first, second, nprob, GEMM_TN, K, N, tile_rows, tile_cols, stream, out, slot_out);
+    QLMX_REQUIRE(second && (mode == GEMM_TN || mode == GEMM_NN), "grouped gemm: NULL list of second halves");
+    return upload_problems(first, second, nprob, mode, K, N, tile_rows, tile_cols, stream, out, slot_out);
 }
 
 int qlmx_upload_done(int slot, hipStream_t stream){ return guard_launched(g_ring_guard, slot, stream); }

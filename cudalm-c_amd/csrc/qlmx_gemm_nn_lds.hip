@@ -88,8 +88,47 @@ __device__ __forceinline__ bf16x8 nn3_pack(const i32x2 lo, const i32x2 hi){
 /* One output tile of NI*64 rows: the four wavefronts 2x2, each NI x 2 accumulators. NI = 4 is the
  * full tile; the last tile of a problem takes the smallest NI that holds its rows, so that an expert
  * with 130 rows does a 192-row tile's work rather than a 256-row tile's. */
+/* The second half of a gate|up problem: the other weight matrix, its output, the SwiGLU output. */
+struct Nn3Dual { unsigned long long wq, wg; float *C; unsigned short *act; };
+
+/* gate, up and bf16(gate * sigmoid(gate) * up) of a gate|up tile. The tile's 128 LDS columns are
+ * [gate 0-31 | up 0-31 | gate 32-63 | up 32-63] of the problem's columns j0 .. j0+63, so a wavefront's first
+ * accumulator column holds gate and its second holds up of the same 32 columns, element for element. */
 template<int NI>
-__device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int i0, int j0, unsigned char *lds){
+__device__ __forceinline__ void nn3_store_swiglu(const f32x16 (&acc)[NI][2], float *gp, float *up, unsigned short *act,
+                                                 int row, int rows, size_t ld){
+    typedef __attribute__((address_space(1))) float gfloat;
+    typedef __attribute__((address_space(1))) uint32_t guint;
+    const bool oddl = threadIdx.x & 1;
+#pragma unroll
+    for(int i = 0; i < NI; i++){
+        uint32_t a[16];
+#pragma unroll
+        for(int e = 0; e < 16; e++){
+            const int ro = i * 32 + (e >> 2) * 8 + (e & 3);
+            const float g = acc[i][0][e], u = acc[i][1][e];
+            a[e] = qx_f32_to_bf16(g * qx_fsig(g) * u);
+            if(row + ro < rows){
+                const size_t o = (size_t)ro * ld;
+                __builtin_nontemporal_store(g, (gfloat *)gp + o);
+                __builtin_nontemporal_store(u, (gfloat *)up + o);
+            }
+        }
+        /* two neighbouring columns per 4-byte store: the even lane of a pair writes the first eight of its
+         * rows for both, the odd lane the other eight */
+#pragma unroll
+        for(int e = 0; e < 8; e++){
+            const uint32_t got = (uint32_t)__shfl_xor((int)(oddl ? a[e] : a[e + 8]), 1, 64);
+            const int e2 = oddl ? e + 8 : e;
+            const int ro = i * 32 + (e2 >> 2) * 8 + (e2 & 3);
+            const uint32_t v = oddl ? (got | (a[e + 8] << 16)) : (a[e] | (got << 16));
+            if(row + ro < rows) *(guint *)(act + (size_t)ro * ld - (oddl ? 1 : 0)) = v;
+        }
+    }
+}
+
+template<int NI, bool DUAL = false>
+__device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, const Nn3Dual &Q, int i0, int j0, unsigned char *lds){
     const int rows = P.M;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wi = (wave >> 1) * (NI * 32), wj = (wave & 1) * 64;
@@ -119,9 +158,11 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int
      * one scale per step. The two 16-byte units it writes per plane are taken in opposite order by even
      * and odd rows, so that the 16 lanes of a write phase (two rows) hit 16 different units. ---- */
     const int oc = tid & 7, kr = tid >> 3, odd = kr & 1;
-    const size_t e0 = (size_t)kr * a.N + j0 + oc * 16;
-    const signed char *pw = a.d + ((P.wq + e0) >> 1);
-    const float *ps = a.s + P.wg + (e0 >> a.gshift);
+    /* gate|up tile: LDS column block oc holds 16 columns of gate (blocks 0, 1, 4, 5) or up (2, 3, 6, 7) */
+    const bool second = DUAL && ((oc >> 1) & 1);
+    const size_t e0 = (size_t)kr * a.N + j0 + (DUAL ? ((oc & 1) + ((oc >> 2) << 1)) * 16 : oc * 16);
+    const signed char *pw = a.d + (((second ? Q.wq : P.wq) + e0) >> 1);
+    const float *ps = a.s + (second ? Q.wg : P.wg) + (e0 >> a.gshift);
     const size_t wstep = (size_t)NN3_BK * a.N >> 1, sstep = (size_t)NN3_BK * a.N >> a.gshift;
     /* unit u of row k at u ^ 4*(k & 3) */
     const int sw = (kr & 3) << 2;
@@ -290,7 +331,11 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, int
 
     /* ---- epilogue: the lane holds column lane%32 of each 32x32 tile, four-row band lane/32 ---- */
     const int row = i0 + wi + hf * 4;
-    qx_store_tiles<NI, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
+    if(DUAL){
+        const size_t o = (size_t)row * a.N + (j0 + (wj >> 1) + fr);
+        nn3_store_swiglu<NI>(acc, P.C + o, Q.C + o, Q.act + o, row, rows, (size_t)a.N);
+    } else
+        qx_store_tiles<NI, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
 }
 
 __global__ void __launch_bounds__(256, 2) k_gemm_nn_lds(Nn3Args a){
@@ -301,10 +346,30 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nn_lds(Nn3Args a){
     const int lt = t - P.tile0;
     const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
     const int i0 = ti * NN3_BM, j0 = tj * NN3_BN, left = P.M - i0;
-    if(left > 192)      nn3_tile<4>(a, P, i0, j0, lds);
-    else if(left > 128) nn3_tile<3>(a, P, i0, j0, lds);
-    else if(left > 64)  nn3_tile<2>(a, P, i0, j0, lds);
-    else                nn3_tile<1>(a, P, i0, j0, lds);
+    const Nn3Dual none = {0, 0, nullptr, nullptr};
+    if(left > 192)      nn3_tile<4>(a, P, none, i0, j0, lds);
+    else if(left > 128) nn3_tile<3>(a, P, none, i0, j0, lds);
+    else if(left > 64)  nn3_tile<2>(a, P, none, i0, j0, lds);
+    else                nn3_tile<1>(a, P, none, i0, j0, lds);
+}
+
+/* gate|up problems: tiles of 256 rows x 64 columns of both matrices; the entry after the problem's holds the
+ * second matrix and the two further outputs */
+__global__ void __launch_bounds__(256, 2) k_gemm_nn_lds_swiglu(Nn3Args a){
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NN3_A_STAGES * NN3_A_BYTES + 2 * NN3_B_BYTES];
+    const int t = qx_xcd_tile(blockIdx.x, gridDim.x);
+    if(t >= a.ntiles) return;
+    const int pi = qx_find_problem(a.pr, a.nprob, t);
+    const DevProb P = a.pr[pi];
+    const DevProb P2 = a.pr[pi + 1];
+    const Nn3Dual Q = {P2.wq, P2.wg, P2.C, (unsigned short *)P2.B};
+    const int lt = t - P.tile0;
+    const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
+    const int i0 = ti * NN3_BM, j0 = tj * (NN3_BN / 2), left = P.M - i0;
+    if(left > 192)      nn3_tile<4, true>(a, P, Q, i0, j0, lds);
+    else if(left > 128) nn3_tile<3, true>(a, P, Q, i0, j0, lds);
+    else if(left > 64)  nn3_tile<2, true>(a, P, Q, i0, j0, lds);
+    else                nn3_tile<1, true>(a, P, Q, i0, j0, lds);
 }
 
 /* bf16 activations only; N % 128 == 0, K % 32 == 0, group a power of two >= 32 (checked by the caller) */
@@ -318,5 +383,20 @@ int qlmx_gemm_nn_lds_launch(const signed char *d, const float *s, int group, con
     const int grid = (up.ntiles + 7) / 8 * 8;
     hipLaunchKernelGGL(k_gemm_nn_lds, dim3(grid), dim3(256), 0, st, a);
     QLMX_LAUNCH_CHECK("grouped gemm nn (direct-to-LDS) launch");
+    return qlmx_upload_done(slot, st);
+}
+
+/* gate|up pairs with the SwiGLU in the epilogue: bf16 activations only; N % 64 == 0, K % 32 == 0, group a
+ * power of two >= 64 (so that a tile's 64 columns of a matrix share a scale per contraction row) */
+int qlmx_gemm_nn_swiglu_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *gate,
+                                   const qlmx_gemm_prob *up_, int nprob, int K, int N, hipStream_t st){
+    ProbUpload up; int slot;
+    int rc = qlmx_upload_problem_pairs(gate, up_, nprob, GEMM_NN, K, N, NN3_BM, NN3_BN / 2, st, &up, &slot); if(rc) return rc;
+    if(up.ntiles == 0) return QLMX_OK;
+    Nn3Args a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.d = d; a.s = s; a.K = K; a.N = N;
+    a.gshift = 0; while((1 << a.gshift) < group) a.gshift++;
+    const int grid = (up.ntiles + 7) / 8 * 8;
+    hipLaunchKernelGGL(k_gemm_nn_lds_swiglu, dim3(grid), dim3(256), 0, st, a);
+    QLMX_LAUNCH_CHECK("grouped gemm nn + swiglu launch");
     return qlmx_upload_done(slot, st);
 }

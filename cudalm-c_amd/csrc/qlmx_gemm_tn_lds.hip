@@ -295,7 +295,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
 int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs,
                             const qlmx_gemm_prob *second, int nprob, int K, int N, hipStream_t st){
     ProbUpload up; int slot;
-    int rc = second ? qlmx_upload_problem_pairs(probs, second, nprob, K, N, TN3_BM, TN3_BN, st, &up, &slot)
+    int rc = second ? qlmx_upload_problem_pairs(probs, second, nprob, GEMM_TN, K, N, TN3_BM, TN3_BN, st, &up, &slot)
                     : qlmx_upload_problems(probs, nprob, GEMM_TN, K, N, TN3_BM, TN3_BN, st, &up, &slot);
     if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;

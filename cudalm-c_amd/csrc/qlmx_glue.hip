@@ -16,19 +16,6 @@
 #include "qlmx_dev.h"
 #include "qlmx_gemm.h"
 
-/* cpu_kern.h:29-34: clamp, Cody-Waite split of ln 2, degree-6 Horner polynomial, exponent built
- * with integer bit arithmetic */
-__device__ __forceinline__ float qx_fexp(float x){
-    x = x < -87.0f ? -87.0f : (x > 88.0f ? 88.0f : x);
-    const float fi = rintf(x * 1.44269504089f);
-    float r = x - fi * 0.693145751953125f;
-    r -= fi * 1.428606765330187e-06f;
-    const float p = 1.0f + r * (1.0f + r * (0.5f + r * (1.0f / 6 + r * (1.0f / 24 + r * (1.0f / 120 + r * (1.0f / 720))))));
-    const float scale = __uint_as_float((uint32_t)((int)fi + 127) << 23);
-    return p * scale;
-}
-__device__ __forceinline__ float qx_fsig(float x){ return 1.0f / (1.0f + qx_fexp(-x)); }
-
 /* ---- router: one thread per token, experts visited in order so the softmax sum rounds exactly as
  * the reference's loop does. `logit` points at the token's E logits and `pr` at E floats for its
  * probabilities (the two may be the same place). ---- */

@@ -290,6 +290,33 @@ void mg_abt_b(const void *A, const float *B, float *C, int M, int K, int N, floa
 void mg_abt(const void *A, const float *B, float *C, int M, int K, int N){ mg_abt_b(A, B, C, M, K, N, 0.0f); }
 void mg_atb(const void *A, const void *B, float *C, int M, int K, int N){ mg_push(2, 2, A, B, C, 0, 0, M, K, N, 1.0f); }
 
+/* gate|up problems with the SwiGLU behind them: queued apart, flushed first as one call per (K, N) */
+struct MgDual { int K, N; qlmx_gemm_prob gate, up; };
+static std::vector<MgDual> g_qdual;
+void mg_ab_swiglu(const void *A, const float *B1, const float *B3, float *gp, float *up, void *ap, int M, int K, int N){
+    if(g_qdual.size() >= QLMX_MAX_PROBLEMS / 2){ fprintf(stderr, "mg queue overflow\n"); exit(1); }
+    MgDual it; it.K = K; it.N = N;
+    unsigned long long wq, wg;
+    weight_of(B1, &wq, &wg);
+    it.gate.A = A; it.gate.B = NULL; it.gate.C = gp; it.gate.wq = wq; it.gate.wg = wg; it.gate.M = M; it.gate.beta = 0.0f;
+    weight_of(B3, &wq, &wg);
+    it.up.A = NULL; it.up.B = ap; it.up.C = up; it.up.wq = wq; it.up.wg = wg; it.up.M = M; it.up.beta = 0.0f;
+    g_qdual.push_back(it);
+}
+static void mg_run_dual(void){
+    std::vector<char> done(g_qdual.size(), 0);
+    for(size_t i = 0; i < g_qdual.size(); i++){
+        if(done[i]) continue;
+        std::vector<qlmx_gemm_prob> gate, up;
+        for(size_t j = i; j < g_qdual.size(); j++)
+            if(!done[j] && g_qdual[j].K == g_qdual[i].K && g_qdual[j].N == g_qdual[i].N){ gate.push_back(g_qdual[j].gate); up.push_back(g_qdual[j].up); done[j] = 1; }
+        const int rc = qlmx_moe_gemm_nn_swiglu(g_mg_q->d, g_mg_q->s, g_mg_q->group, gate.data(), up.data(), (int)gate.size(),
+                                               g_qdual[i].K, g_qdual[i].N, g_mg_act, g_mg_math, NULL);
+        if(rc != QLMX_OK){ fprintf(stderr, "grouped GEMM error %d at mg grouped (gate|up): %s\n", rc, qlmx_last_error()); exit(1); }
+    }
+    g_qdual.clear();
+}
+
 static void mg_run(std::vector<MgItem> &v){
     std::vector<char> done(v.size(), 0);
     for(size_t i = 0; i < v.size(); i++){
@@ -337,4 +364,4 @@ static void mg_run_pairs(void){
     for(size_t j = 0; j < v1.size(); j++) if(!done[j]) r1.push_back(v1[j]);
     v0.swap(r0); v1.swap(r1);
 }
-void mg_flush(void){ mg_run_pairs(); mg_run(g_q[0]); mg_run(g_q[1]); mg_run(g_q[2]); }
+void mg_flush(void){ mg_run_dual(); mg_run_pairs(); mg_run(g_q[0]); mg_run(g_q[1]); mg_run(g_q[2]); }

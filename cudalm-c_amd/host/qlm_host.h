@@ -83,5 +83,8 @@ void mg_ab(const void *A, const float *B, float *C, int M, int K, int N);       
 void mg_abt_b(const void *A, const float *B, float *C, int M, int K, int N, float beta); /* cudalm.cu:3250 */
 void mg_abt(const void *A, const float *B, float *C, int M, int K, int N);               /* cudalm.cu:3253 */
 void mg_atb(const void *A, const void *B, float *C, int M, int K, int N);                /* cudalm.cu:3254 */
+/* mg_ab on w1 and w3 of one expert followed by the reference's e_swig (cudalm.cu:4211-4215) as one queued
+ * item: gp = A.B1, up = A.B3 (fp32, kept for the backward pass), ap = bf16(SwiGLU(gp, up)) */
+void mg_ab_swiglu(const void *A, const float *B1, const float *B3, float *gp, float *up, void *ap, int M, int K, int N);
 void mg_flush(void);                                                                      /* cudalm.cu:3243 */
 #endif

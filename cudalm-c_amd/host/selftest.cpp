@@ -3,7 +3,7 @@
  * 2*dmax+1 levels per group; one Integer AdamW step against a scalar host restatement that reuses
  * the host helpers (digits/residuals must agree bit for bit here because both sides are compiled
  * without FMA contraction); a save/load round trip; an expert FFN forward through the grouped GEMM
- * queue against a host triple loop, and the paired input-gradient GEMMs of w1 and w3. Prints one line per check and exits 0 only if all pass. */
+ * queue against a host triple loop, the paired input-gradient GEMMs of w1 and w3, and the gate|up GEMMs with the SwiGLU behind them. Prints one line per check and exits 0 only if all pass. */
 #include "qlm_host.h"
 #include <math.h>
 #include <stdio.h>
@@ -160,6 +160,26 @@ int main(){
                                             + (double)f32(du[(size_t)m * F + f]) * Pr[16 + nw + (size_t)e * D * F + (size_t)k * F + f];
             const double dlt = (double)dX[(size_t)m * D + k] - acc; num2 += dlt * dlt; den2 += acc * acc; }
         check("moe dgrad w1+w3 (mg_abt_b pair) rel-err", sqrt(num2 / den2), 1e-3);
+
+        /* (f) gate | up | SwiGLU as one queued item per expert, bf16 activations on the matrix cores */
+        std::vector<unsigned short> Xb((size_t)N * D), apb((size_t)N * F, 0);
+        for(size_t i = 0; i < Xb.size(); i++) Xb[i] = bf16(X[i]);
+        void *Xbd = dmalloc(Xb.size() * 2), *apd = dmalloc(apb.size() * 2);
+        float *gpd = (float *)dmalloc((size_t)N * F * 4), *upd = (float *)dmalloc((size_t)N * F * 4);
+        qlmx_memcpy_h2d(Xbd, Xb.data(), Xb.size() * 2);
+        for(int e = 0; e < E; e++){ int ne = off[e + 1] - off[e]; if(!ne) continue;
+            mg_ab_swiglu((const unsigned short *)Xbd + (size_t)off[e] * D, Pd + 16 + (size_t)e * D * F, Pd + 16 + nw + (size_t)e * D * F,
+                         gpd + (size_t)off[e] * F, upd + (size_t)off[e] * F, (unsigned short *)apd + (size_t)off[e] * F, ne, D, F); }
+        mg_flush(); qlmx_sync(NULL);
+        qlmx_memcpy_d2h(apb.data(), apd, apb.size() * 2);
+        double num3 = 0, den3 = 0;
+        for(int e = 0; e < E; e++) for(int m = off[e]; m < off[e + 1]; m++) for(int f = 0; f < F; f++){
+            double g = 0, u = 0;
+            for(int k = 0; k < D; k++){ const double x = f32(Xb[(size_t)m * D + k]);
+                g += x * Pr[16 + (size_t)e * D * F + (size_t)k * F + f]; u += x * Pr[16 + nw + (size_t)e * D * F + (size_t)k * F + f]; }
+            const double want = g / (1.0 + exp(-g)) * u, dlt = (double)f32(apb[(size_t)m * F + f]) - want;
+            num3 += dlt * dlt; den3 += want * want; }
+        check("moe gate|up|swiglu (mg_ab_swiglu) rel-err", sqrt(num3 / den3), 5e-3);   /* bf16 output: 2^-9 per element */
     }
     qlm_free(&q);
     printf(ok_all ? "[selftest] ALL PASS\n" : "[selftest] FAILED\n");

@@ -169,6 +169,17 @@ int qlmx_moe_gemm_tn(const signed char *d, const float *s, int group,
 int qlmx_moe_gemm_tn_pair(const signed char *d, const float *s, int group,
                           const qlmx_gemm_prob *first_host, const qlmx_gemm_prob *second_host, int nprob,
                           int K, int N, int act_dtype, int math, void *stream);
+/* The gate and up GEMMs of moe_forward and the SwiGLU that follows them (cudalm.cu:4211-4215: mg_ab(Xp, w1_e,
+ * gp), mg_ab(Xp, w3_e, up), mg_flush, e_swig(gp, up, ap)) as one call: problem i computes
+ *   gp = A . W(gate[i].wq),  up = A . W(up[i].wq),  ap = bf16(gp * sigmoid(gp) * up)   (k_swiglu, cudalm.cu:2430)
+ * with A = gate[i].A [M, K]; gp goes to gate[i].C and up to up[i].C (fp32 [M, N], kept for the backward pass),
+ * ap to up[i].B (bf16 [M, N], the down GEMM's input). up[i] must repeat M; its A and beta are ignored.
+ * On bf16 activations with QLMX_MATH_MFMA (N % 64 == 0, K % 32 == 0, group a power of two >= 64, at most
+ * QLMX_MAX_PROBLEMS / 2 problems) an output tile holds 64 columns of both matrices and the SwiGLU is applied
+ * to the accumulators; every other combination runs the two GEMM launches and a SwiGLU launch per problem. */
+int qlmx_moe_gemm_nn_swiglu(const signed char *d, const float *s, int group,
+                            const qlmx_gemm_prob *gate_host, const qlmx_gemm_prob *up_host, int nprob,
+                            int K, int N, int act_dtype, int math, void *stream);
 /* nt: no weight operand; both inputs are activations, fp32 result. beta = 1 reproduces the
  * reference's accumulation into a zeroed G; beta = 0 saves the read when G is known to be fresh. */
 int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs_host, int nprob, int K, int N,

@@ -257,6 +257,63 @@ def test_tn_pair_rejects_mismatched_rows(q):
     q.gemm_tn_pair(zb, z, 128, a, a, 0, 128, 128, pkg.ACT_BF16, pkg.MATH_MFMA)       # no problems: nothing to do
 
 
+def _swiglu_case(q, orc, rowsM, K, N, act, math, seed=13):
+    """gate | up | SwiGLU through qlmx_moe_gemm_nn_swiglu against the library's separate calls: returns
+    (gp, up, ap as fp32) of both ways plus the oracle's gp."""
+    import torch
+    E = len(rowsM); tot = sum(rowsM)
+    off = np.concatenate([[0], np.cumsum(rowsM)]).astype(int)
+    bf = act == pkg.ACT_BF16
+    d, s, P = make_weights(orc, seed, 2 * E, K, N)
+    A = orc.normal(tot * K, seed, 10)
+    if bf or math == pkg.MATH_MFMA:
+        A = orc.bf16_round(A)                       # the matrix cores see bf16 activations either way
+    dA, dd, ds = dev(A), dev(d), dev(s)
+    pa = to_bf16_bits(dA) if bf else dA
+    esz = 2 if bf else 4
+    out = []
+    for fused in (True, False):
+        gp = torch.full((tot * N,), 7.0, device="cuda"); up = torch.full((tot * N,), 7.0, device="cuda")
+        ap = torch.zeros(tot * N, dtype=torch.bfloat16, device="cuda")
+        gate = q.problems([(pa.data_ptr() + off[e] * K * esz, None, gp.data_ptr() + off[e] * N * 4, e * K * N, e * K * N // 128, rowsM[e], 0.0) for e in range(E)])
+        upp = q.problems([(None, ap.data_ptr() + off[e] * N * 2, up.data_ptr() + off[e] * N * 4, (E + e) * K * N, (E + e) * K * N // 128, rowsM[e], 0.0) for e in range(E)])
+        if fused:
+            q.gemm_nn_swiglu(dd, ds, 128, gate, upp, E, K, N, act, math)
+        else:
+            up2 = q.problems([(pa.data_ptr() + off[e] * K * esz, None, up.data_ptr() + off[e] * N * 4, (E + e) * K * N, (E + e) * K * N // 128, rowsM[e], 0.0) for e in range(E)])
+            q.gemm_nn(dd, ds, 128, gate, E, K, N, act, math)
+            q.gemm_nn(dd, ds, 128, up2, E, K, N, act, math)
+            q.swiglu(gp, up, ap, tot * N, pkg.ACT_BF16)
+        torch.cuda.synchronize()
+        out.append((gp.cpu().numpy(), up.cpu().numpy(), ap.float().cpu().numpy()))
+    want = np.zeros(tot * N, f32)
+    for e in range(E):
+        if rowsM[e]:
+            orc.gemm_nn(A[off[e] * K:], P[e * K * N:(e + 1) * K * N], want[off[e] * N:off[e + 1] * N], rowsM[e], K, N)
+    return out, want
+
+
+@pytest.mark.parametrize("rowsM,K,N", [([300, 0, 64, 1, 129, 517], 256, 384), ([700, 40, 333], 768, 2048)])
+def test_mfma_nn_swiglu_one_launch(q, orc, rowsM, K, N):
+    """Gate and up columns share a tile and the SwiGLU runs on the accumulators: gp and up bit-identical to the
+    two separate GEMM calls (same MFMA sequence per element), ap bit-identical to the SwiGLU kernel on them;
+    ragged experts, an empty one, last tiles of every height."""
+    (f, sep), want = _swiglu_case(q, orc, rowsM, K, N, pkg.ACT_BF16, pkg.MATH_MFMA)
+    assert orc.relerr(f[0], want) < TOL_MFMA
+    for a, b in zip(f, sep):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+@pytest.mark.parametrize("act,math", [("f32", "f32"), ("bf16", "f32"), ("f32", "mfma")])
+def test_nn_swiglu_other_paths(q, orc, act, math):
+    a = pkg.ACT_BF16 if act == "bf16" else pkg.ACT_F32
+    m = pkg.MATH_MFMA if math == "mfma" else pkg.MATH_F32
+    (f, sep), want = _swiglu_case(q, orc, [70, 0, 132], 256, 128, a, m, seed=14)
+    assert orc.relerr(f[0], want) < (TOL_MFMA if math == "mfma" else TOL_F32)
+    for x, y in zip(f, sep):
+        assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+
+
 @pytest.mark.parametrize("beta", [0.0, 1.0])
 def test_mfma_nt_split_contraction(q, orc, beta):
     """One expert with far more rows than the others: its contraction is cut into slices that add up

@@ -15,7 +15,8 @@ workload that ran in the order train, decode, adamw. `cpu_baseline` times the re
 backend (oracle/_ref, kind "reference") or the repository's C restatement (kind "port") on a bounded
 sample on this host's cores; it is a reported baseline, not the target.
 Defaults: 30 warm-up and 100 timed steps. The device takes some 20 ms of load to reach the clock it then
-holds; with 3 + 20 steps of 1 ms the timed region lies inside that ramp and reads 8 % low.
+holds; with 3 + 20 steps of 1 ms the timed region would lie inside that ramp and read 8 % low, so every
+measurement is preceded by 40 ms of the same calls, untimed, in addition to the W warm-up steps.
 """
 import argparse
 import json
@@ -26,6 +27,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+SETTLE_MS = 40.0               # untimed load in front of every measurement (clock ramp, see the docstring)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
 
@@ -46,6 +48,13 @@ def timed(torch, fn, steps, warmup):
     """W untimed calls, then exactly K timed ones bracketed by synchronize. One pair of HIP events on the
     stream the kernels run on (torch's current stream, handed to the library) spans the K calls: an
     event between two calls would itself leave the GPU idle for some 6 us and be charged to the step."""
+    # the device reaches the clock it then holds only after some 20 ms of load: keep it busy with the same
+    # call for SETTLE_MS first, whatever W is, so that a short run does not time the ramp
+    t_end = time.perf_counter() + SETTLE_MS * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -474,7 +483,7 @@ def main():
         "metric": "QLM expert dequant-GEMM TFLOP/s & GB/s (% roofline); int-AdamW GB/s",
         "value": first["value"], "unit": first["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": first["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": first["dtype"], "data": "synthetic",
+        "dtype": first["dtype"], "data": "synthetic", "settle_ms": SETTLE_MS,
         "config": {"workload": first["workload"]},
         "roofline": first["roofline"],
         "workloads": results,

@@ -317,6 +317,7 @@ struct DfArgs {
     const float *x; const int *assign; const float *gate; float *out;
     const signed char *d; const float *s;
     u64 w1q, w3q, w2q; int group;
+    u64 w1g, w3g, w2g, dfg;   /* the matrices' first scale groups, and scale groups per expert matrix (host-side divisions) */
     int T, K, E, D, F;
     int R1, S1, NC1, R2, S2, NC2;
     u64 *part1, *part2; unsigned epoch; unsigned *status;
@@ -389,7 +390,7 @@ __device__ __forceinline__ uint32_t df_and(uint32_t v){
 }
 
 /* One task: which slice of which matrix, for which problem. list 0 = none. */
-struct DfT { u64 wq; int list, N, k0, rows, chunk, M, prob, mat, sl; };
+struct DfT { u64 wq, wg; int list, N, k0, rows, chunk, M, prob, mat, sl; };
 
 /* first DF_BATCH steps of a task's digits into W (the caller keeps them in flight across the end of
  * the previous task) */
@@ -569,7 +570,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
     const int tpg2 = a.NC2 * a.S2, lim2 = ((nprob + 7) >> 3) * tpg2;
     int list = 1, q = slot0;
     auto fetch = [&]() -> DfT {
-        DfT t; t.list = 0; t.wq = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = 0;
+        DfT t; t.list = 0; t.wq = 0; t.wg = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = 0;
         for(;;){
             if(list == 1){
                 if(q >= lim1){ list = 2; q = slot0; continue; }
@@ -578,6 +579,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
                 t.list = 1; t.prob = g >> 1; t.mat = g & 1; t.chunk = sub / a.S1; t.sl = sub - t.chunk * a.S1;
                 t.N = a.F; t.k0 = t.sl * a.R1; t.rows = min(a.R1, a.D - t.k0); t.M = mt.p_M[t.prob];
                 t.wq = (t.mat ? a.w3q : a.w1q) + (u64)mt.p_e[t.prob] * DF;
+                t.wg = (t.mat ? a.w3g : a.w1g) + (u64)mt.p_e[t.prob] * a.dfg;
                 return t;
             }
             if(list == 2){
@@ -587,6 +589,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
                 t.list = 2; t.prob = prob; t.mat = 0; t.chunk = sub / a.S2; t.sl = sub - t.chunk * a.S2;
                 t.N = a.D; t.k0 = t.sl * a.R2; t.rows = min(a.R2, a.F - t.k0); t.M = mt.p_M[prob];
                 t.wq = a.w2q + (u64)mt.p_e[prob] * DF;
+                t.wg = a.w2g + (u64)mt.p_e[prob] * a.dfg;
                 return t;
             }
             return t;
@@ -610,7 +613,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
         const int hs = cur.list == 1 ? hs1 : hs2;
         const int prob = cur.prob, chunk = cur.chunk, k0 = cur.k0, rows = cur.rows, M = cur.M;
         const int gpr = cur.N / a.group;
-        const float *srow0 = a.s + cur.wq / (u64)a.group + (size_t)k0 * gpr + (chunk * DF_CW) / a.group;
+        const float *srow0 = a.s + cur.wg + (size_t)k0 * gpr + (chunk * DF_CW) / a.group;
         u64 *dst; size_t mstride;
         if(cur.list == 1){ dst = a.part1 + ((((size_t)prob * 2 + cur.mat) * a.S1 + cur.sl) * DF_MB) * a.F; mstride = (size_t)a.F; }
         else             { dst = a.part2 + (((size_t)prob * a.S2 + cur.sl) * DF_MB) * a.D;                  mstride = (size_t)a.D; }
@@ -752,6 +755,7 @@ extern "C" int qlmx_moe_decode_forward(const float *x, const int *assign, const 
     const int npair = T * K;
     DfArgs a;
     a.x = x; a.assign = assign; a.gate = gate; a.out = out; a.d = d; a.s = s; a.w1q = w1q; a.w3q = w3q; a.w2q = w2q; a.group = group;
+    a.w1g = w1q / group; a.w3g = w3q / group; a.w2g = w2q / group; a.dfg = (u64)D * F / group;
     a.T = T; a.K = K; a.E = E; a.D = D; a.F = F;
     a.NC1 = (F + DF_CW - 1) / DF_CW; a.NC2 = (D + DF_CW - 1) / DF_CW;
     const double hits = E * (1.0 - pow(1.0 - 1.0 / E, (double)npair));

@@ -142,7 +142,8 @@ int qlmx_servo(signed char *d, signed char *r, float *s,
 
 typedef struct qlmx_gemm_prob {
     const void *A;           /* device: nn/tn [M,K]; nt [M,K] (read transposed)                  */
-    const void *B;           /* device: nt only, [M,N] activation/gradient rows; else NULL      */
+    const void *B;           /* device: nt: [M,N] activation/gradient rows; the second list of
+                              * qlmx_moe_gemm_nn_swiglu: the bf16 output; else NULL              */
     float      *C;           /* device: nn/tn [M,N]; nt [K,N]                                    */
     unsigned long long wq;   /* nn/tn: element offset of the weight matrix in the digit array    */
     unsigned long long wg;   /* nn/tn: index of the matrix's first scale group                   */

@@ -353,6 +353,20 @@ def test_mfma_more_problems_than_lanes(q, orc, mode):
     assert orc.relerr(got, want) < TOL_MFMA
 
 
+def test_paired_calls_with_more_table_entries_than_lanes(q, orc):
+    """70 experts with a second half each: 140 table entries, every other one owning no tile, looked up in
+    three passes of a wavefront."""
+    rng = np.random.default_rng(5)
+    rows = [int(r) for r in rng.integers(0, 40, 70)]
+    rows[0] = 0; rows[69] = 37
+    got, want = _pair_case(q, orc, rows, 128, 128, pkg.ACT_BF16, pkg.MATH_MFMA, 1.0, seed=15)
+    assert orc.relerr(got, want) < TOL_MFMA
+    (f, sep), want = _swiglu_case(q, orc, rows, 64, 128, pkg.ACT_BF16, pkg.MATH_MFMA, seed=16)
+    assert orc.relerr(f[0], want) < TOL_MFMA
+    for a, b in zip(f, sep):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 def test_mfma_table_ring_wraps(q, orc):
     """150 grouped launches without a synchronisation between them go more than twice round the ring of
     problem tables (and four times round the unit-table ring of the weight gradient); a launch whose

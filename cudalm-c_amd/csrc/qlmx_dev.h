@@ -42,6 +42,9 @@ __host__ __device__ __forceinline__ int qx_clamp(int v, int lo, int hi){ return 
 
 /* signed 4-bit field k (0..7) of a 32-bit word holding 8 consecutive digits (qlm.cuh:96-101) */
 __device__ __forceinline__ int qx_nib(uint32_t w, int k){ return ((int)(w << (28 - 4*k))) >> 28; }
+/* digit k of a packed word as digit / 16 in fp32 (exact): one shift and v_cvt_off_f32_i4, against two
+ * shifts and a convert for the integer route. Whoever uses it carries the factor 16 in a scale. */
+__device__ __forceinline__ float qx_nib16(uint32_t w, int k){ return __builtin_amdgcn_cvt_off_f32_i4((int)(w >> (4 * k))); }
 
 /* ---- span lookup: the owner of group gi. The table is ascending in gi0, so a binary search
  * returns what the reference's first-match linear scan returns (qlm.cuh:114-117). ---- */

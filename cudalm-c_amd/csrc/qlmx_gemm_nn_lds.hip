@@ -182,7 +182,7 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, con
     auto dequant_unit = [&](uint32_t digits, float sc, i32x4 &hi, i32x4 &lo){
         float w[8];
 #pragma unroll
-        for(int j = 0; j < 8; j++) w[j] = sc * (float)qx_nib(digits, j);
+        for(int j = 0; j < 8; j++) w[j] = (sc * 16.0f) * qx_nib16(digits, j);      /* 16 s * (digit / 16): both factors exact, the product is s * digit */
 #pragma unroll
         for(int j = 0; j < 4; j++){
             const uint32_t h = nn3_pk(w[2 * j], w[2 * j + 1]);
@@ -261,7 +261,7 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, con
         i32x4 whi[2], wlo[2];
         float wf[8][2];
         uint32_t dg[2];
-        const float sc = __int_as_float(wcur.s);
+        const float sc = __int_as_float(wcur.s) * 16.0f;     /* the digits come as digit / 16 (exact), the product is s * digit as before */
         auto item = [&](int k){
             if(k == 0)      wnext.d = nn3_gld8(pw + (size_t)tile2 * wstep);
             else if(k == 1) wnext.s = nn3_gld4(ps + (size_t)tile2 * sstep);
@@ -272,7 +272,7 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, con
                 const int q = k - 2 - NI, p = q >> 1, r = p >> 2, j = p & 3;
                 if(q == 0){ dg[0] = unit_digits(wcur, 0); dg[1] = unit_digits(wcur, 1); }
                 if((q & 1) == 0){
-                    wf[p][0] = sc * (float)qx_nib(dg[r], 2 * j); wf[p][1] = sc * (float)qx_nib(dg[r], 2 * j + 1);
+                    wf[p][0] = sc * qx_nib16(dg[r], 2 * j); wf[p][1] = sc * qx_nib16(dg[r], 2 * j + 1);
                 } else {
                     const uint32_t h = nn3_pk(wf[p][0], wf[p][1]);
                     whi[r][j] = (int)h;

@@ -124,10 +124,10 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, con
 #pragma unroll
         for(int j = 0; j < 4; j++){
             i32x4 v;
-            v[0] = (int)tn3_pk((float)qx_nib(wd[j], 0), (float)qx_nib(wd[j], 1));
-            v[1] = (int)tn3_pk((float)qx_nib(wd[j], 2), (float)qx_nib(wd[j], 3));
-            v[2] = (int)tn3_pk((float)qx_nib(wd[j], 4), (float)qx_nib(wd[j], 5));
-            v[3] = (int)tn3_pk((float)qx_nib(wd[j], 6), (float)qx_nib(wd[j], 7));
+            v[0] = (int)tn3_pk(qx_nib16(wd[j], 0), qx_nib16(wd[j], 1));
+            v[1] = (int)tn3_pk(qx_nib16(wd[j], 2), qx_nib16(wd[j], 3));
+            v[2] = (int)tn3_pk(qx_nib16(wd[j], 4), qx_nib16(wd[j], 5));
+            v[3] = (int)tn3_pk(qx_nib16(wd[j], 6), qx_nib16(wd[j], 7));
             tn3_wr(bb + wr_off[j], v);
         }
     };
@@ -214,8 +214,8 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, con
                 const int q = k - 3 - 2 * NI, j = q / 3, h = q % 3;
                 if(h < 2){
                     const uint32_t wd = (uint32_t)wcur[j];
-                    wv[j][2 * h]     = (int)tn3_pk((float)qx_nib(wd, 4 * h),     (float)qx_nib(wd, 4 * h + 1));
-                    wv[j][2 * h + 1] = (int)tn3_pk((float)qx_nib(wd, 4 * h + 2), (float)qx_nib(wd, 4 * h + 3));
+                    wv[j][2 * h]     = (int)tn3_pk(qx_nib16(wd, 4 * h),     qx_nib16(wd, 4 * h + 1));
+                    wv[j][2 * h + 1] = (int)tn3_pk(qx_nib16(wd, 4 * h + 2), qx_nib16(wd, 4 * h + 3));
                 } else tn3_wr(wbuf + wr_off[j], wv[j]);
             }
         };
@@ -250,13 +250,15 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, con
 #undef TN3_KS
         if(last){
             /* one scale group of the contraction is complete: fold it in with its fp32 scale (spreading
-             * these among the MFMAs as well costs some fifty registers, which spill) */
+             * these among the MFMAs as well costs some fifty registers, which spill). The matrix core was
+             * fed digit / 16, so the scale carries the 16: both are exact, the product is the same. */
+            const float fs16[2] = {fs_cur[0] * 16.0f, fs_cur[1] * 16.0f};
 #pragma unroll
             for(int j = 0; j < 2; j++)
 #pragma unroll
                 for(int i = 0; i < NI; i++)
 #pragma unroll
-                    for(int e = 0; e < 16; e++) acc[i][j][e] = fmaf(fs_cur[j], part[i][j][e], acc[i][j][e]);
+                    for(int e = 0; e < 16; e++) acc[i][j][e] = fmaf(fs16[j], part[i][j][e], acc[i][j][e]);
         }
         /* the digits of step st+2 and the scales of step st+1 have arrived (only the activation requests are younger) */
         asm volatile("s_waitcnt vmcnt(%3)" : "+v"(wnext), "+v"(fn[0]), "+v"(fn[1]) : "n"(2 * NI) : "memory");

@@ -39,6 +39,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train", "train5", "codec", "glue", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--step-only", action="store_true", help="train: skip the per-launch repetitions, so that a kernel trace holds nothing but steps")
     ap.add_argument("--adamw-weights", type=int, default=120 * 2 ** 20)
     ap.add_argument("--render-p", type=int, default=0, help="adamw: also write the fp32 view P (4 B/weight more)")
     return ap.parse_args()
@@ -151,7 +152,7 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
 
     tm = timed(torch, step, args.steps, args.warmup)
     per = {}
-    for name, fn, ng in calls:
+    for name, fn, ng in ([] if args.step_only else calls):
         t1 = timed(torch, fn, max(5, args.steps // 2), 2)
         per[name] = {"ms": t1["event_ms_avg"], "tflops": ng * unit / (t1["event_ms_avg"] * 1e-3) / 1e12}
     # beside the step: the forward's gate|up GEMMs with the SwiGLU in their epilogue, against the two-launch form
@@ -160,12 +161,12 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
     g_up = P([(None, act.data_ptr() + off[e] * F * 2, up.data_ptr() + off[e] * F * 4, o3 + e * D * F, (o3 + e * D * F) // group, int(cnt[e]), 0.0)
               for e in range(E)])
     extra = {}
-    for name, fn in [("fwd w1,w3 + SwiGLU, one launch", lambda: q.gemm_nn_swiglu(d, s, group, g_gate, g_up, E, D, F, ACT_BF16, MATH_MFMA, stream)),
+    for name, fn in [] if args.step_only else [("fwd w1,w3 + SwiGLU, one launch", lambda: q.gemm_nn_swiglu(d, s, group, g_gate, g_up, E, D, F, ACT_BF16, MATH_MFMA, stream)),
                      ("SwiGLU kernel alone", lambda: q.swiglu(gp, up, act, rows * F, ACT_BF16, stream))]:
         extra[name] = {"ms": timed(torch, fn, max(5, args.steps // 2), 2)["event_ms_avg"]}
     flops = 9 * unit
     tf = flops / (tm["event_ms_avg"] * 1e-3) / 1e12
-    dom = max(per, key=lambda k: per[k]["ms"])
+    dom = max(per, key=lambda k: per[k]["ms"]) if per else "not timed"
     return {
         "workload": "%s: E=%d top-%d D=%d F=%d, %d bf16 tokens -> %d expert rows, Zipf(1.1) load (max %d, min %d rows); "
                     "fwd+dgrad+wgrad = 9 grouped GEMMs in 6 launches" % (label, E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min())),

@@ -45,6 +45,16 @@ __device__ __forceinline__ int qx_nib(uint32_t w, int k){ return ((int)(w << (28
 /* digit k of a packed word as digit / 16 in fp32 (exact): one shift and v_cvt_off_f32_i4, against two
  * shifts and a convert for the integer route. Whoever uses it carries the factor 16 in a scale. */
 __device__ __forceinline__ float qx_nib16(uint32_t w, int k){ return __builtin_amdgcn_cvt_off_f32_i4((int)(w >> (4 * k))); }
+/* The same for all eight digits of a word at nine instructions: the convert takes its operand from a byte
+ * of a register (an operand modifier, no shift), so the even digits come from the bytes of w and the odd ones
+ * from the bytes of w >> 4. The empty asm keeps the shifted word a value of its own; seen through, the
+ * compiler turns "byte of w >> 4" back into a bit-field extract per digit. */
+struct QxNibs { uint32_t w, h; };
+__device__ __forceinline__ QxNibs qx_nibs(uint32_t w){ QxNibs n; n.w = w; n.h = w >> 4; asm("" : "+v"(n.h)); return n; }
+__device__ __forceinline__ float qx_nib16(const QxNibs &n, int k){
+    const uint32_t src = (k & 1) ? n.h : n.w;
+    return __builtin_amdgcn_cvt_off_f32_i4((int)((src >> (8 * (k >> 1))) & 0xFFu));
+}
 
 /* ---- span lookup: the owner of group gi. The table is ascending in gi0, so a binary search
  * returns what the reference's first-match linear scan returns (qlm.cuh:114-117). ---- */

@@ -181,8 +181,9 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, con
     };
     auto dequant_unit = [&](uint32_t digits, float sc, i32x4 &hi, i32x4 &lo){
         float w[8];
+        const QxNibs nb = qx_nibs(digits);
 #pragma unroll
-        for(int j = 0; j < 8; j++) w[j] = (sc * 16.0f) * qx_nib16(digits, j);      /* 16 s * (digit / 16): both factors exact, the product is s * digit */
+        for(int j = 0; j < 8; j++) w[j] = (sc * 16.0f) * qx_nib16(nb, j);          /* 16 s * (digit / 16): both factors exact, the product is s * digit */
 #pragma unroll
         for(int j = 0; j < 4; j++){
             const uint32_t h = nn3_pk(w[2 * j], w[2 * j + 1]);
@@ -260,7 +261,7 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, con
         WLoad wnext;
         i32x4 whi[2], wlo[2];
         float wf[8][2];
-        uint32_t dg[2];
+        QxNibs dg[2];
         const float sc = __int_as_float(wcur.s) * 16.0f;     /* the digits come as digit / 16 (exact), the product is s * digit as before */
         auto item = [&](int k){
             if(k == 0)      wnext.d = nn3_gld8(pw + (size_t)tile2 * wstep);
@@ -270,7 +271,7 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, con
                                                  (lds_void *)(lds + stage2 * NN3_A_BYTES + wave_off + (k - 2) * 4096), 16, 0, 0);
             else if(k < 2 + NI + 16){
                 const int q = k - 2 - NI, p = q >> 1, r = p >> 2, j = p & 3;
-                if(q == 0){ dg[0] = unit_digits(wcur, 0); dg[1] = unit_digits(wcur, 1); }
+                if(q == 0){ dg[0] = qx_nibs(unit_digits(wcur, 0)); dg[1] = qx_nibs(unit_digits(wcur, 1)); }
                 if((q & 1) == 0){
                     wf[p][0] = sc * qx_nib16(dg[r], 2 * j); wf[p][1] = sc * qx_nib16(dg[r], 2 * j + 1);
                 } else {

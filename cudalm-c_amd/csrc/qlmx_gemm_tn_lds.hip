@@ -124,10 +124,11 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, con
 #pragma unroll
         for(int j = 0; j < 4; j++){
             i32x4 v;
-            v[0] = (int)tn3_pk(qx_nib16(wd[j], 0), qx_nib16(wd[j], 1));
-            v[1] = (int)tn3_pk(qx_nib16(wd[j], 2), qx_nib16(wd[j], 3));
-            v[2] = (int)tn3_pk(qx_nib16(wd[j], 4), qx_nib16(wd[j], 5));
-            v[3] = (int)tn3_pk(qx_nib16(wd[j], 6), qx_nib16(wd[j], 7));
+            const QxNibs nb = qx_nibs(wd[j]);
+            v[0] = (int)tn3_pk(qx_nib16(nb, 0), qx_nib16(nb, 1));
+            v[1] = (int)tn3_pk(qx_nib16(nb, 2), qx_nib16(nb, 3));
+            v[2] = (int)tn3_pk(qx_nib16(nb, 4), qx_nib16(nb, 5));
+            v[3] = (int)tn3_pk(qx_nib16(nb, 6), qx_nib16(nb, 7));
             tn3_wr(bb + wr_off[j], v);
         }
     };
@@ -213,9 +214,9 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, con
                 /* per 16-byte unit: two conversion items, then its write */
                 const int q = k - 3 - 2 * NI, j = q / 3, h = q % 3;
                 if(h < 2){
-                    const uint32_t wd = (uint32_t)wcur[j];
-                    wv[j][2 * h]     = (int)tn3_pk(qx_nib16(wd, 4 * h),     qx_nib16(wd, 4 * h + 1));
-                    wv[j][2 * h + 1] = (int)tn3_pk(qx_nib16(wd, 4 * h + 2), qx_nib16(wd, 4 * h + 3));
+                    const QxNibs nb = qx_nibs((uint32_t)wcur[j]);
+                    wv[j][2 * h]     = (int)tn3_pk(qx_nib16(nb, 4 * h),     qx_nib16(nb, 4 * h + 1));
+                    wv[j][2 * h + 1] = (int)tn3_pk(qx_nib16(nb, 4 * h + 2), qx_nib16(nb, 4 * h + 3));
                 } else tn3_wr(wbuf + wr_off[j], wv[j]);
             }
         };

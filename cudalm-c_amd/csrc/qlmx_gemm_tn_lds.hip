@@ -147,12 +147,12 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, con
     }
 
     /* ---- fp32 scale of (this lane's output column, scale group) ---- */
-    const int ngroups = a.K >> a.gshift, spg = (1 << a.gshift) / TN3_BK;
+    const int ngroups = a.K >> a.gshift, sshift = a.gshift - 6, spg = 1 << sshift;     /* steps per scale group: a power of two */
     const float *pfold[2];
 #pragma unroll
     for(int j = 0; j < 2; j++) pfold[j] = a.s + P.wg + (size_t)(j0 + wj + j * 32 + fr) * ngroups;
     auto load_scale = [&](int step, int j) -> float {
-        int g = step / spg; g = g < ngroups * sg.nseg ? g : ngroups * sg.nseg - 1;
+        int g = step >> sshift; g = g < ngroups * sg.nseg ? g : ngroups * sg.nseg - 1;
         const long long og = g < ngroups ? (long long)g : (long long)(g - ngroups) + sg.dS;
         return tn3_gld4(pfold[j] + og);
     };
@@ -191,21 +191,27 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, con
      * A scale group's partial sums start from a zero operand instead of cleared registers. */
     constexpr int SLOTS = NI * 8, ITEMS = 3 + 2 * NI + 8 + 4;
     const f32x16 zero = (f32x16)(0.0f);
+    /* A wavefront issues one instruction every four cycles whatever its kind, so the scalar bookkeeping of a step
+     * counts like everything else: the stage numbers and the operand offsets of the tile two steps ahead are
+     * carried from step to step (a compare and an add each) instead of being derived from the step number with
+     * divisions and 64-bit multiplies. */
+    int stg = 0, stg2 = 2 % TN3_A_STAGES;
+    long long oa2 = off_a(2 < steps ? 2 : steps - 1), ow2 = off_w(2 < steps ? 2 : steps - 1);
+    const long long jump_a = sg.dA - (long long)steps1 * (TN3_BK * 2), jump_w = sg.dW - (long long)steps1 * (TN3_BK / 2);
     for(int st = 0; st < steps; st++){
         /* tile st is in, own LDS writes are done; tile st+1 may still be on its way */
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"(2 * NI) : "memory");
         __builtin_amdgcn_s_barrier();
 
-        const uint32_t sa = lds_base + (uint32_t)(st % TN3_A_STAGES) * TN3_A_BYTES;
+        const uint32_t sa = lds_base + (uint32_t)stg * TN3_A_BYTES;
         const uint32_t sbuf = lds_base + (uint32_t)(st & 1) * TN3_B_BYTES;
         const uint32_t wbuf = lds_base + (uint32_t)((st + 1) & 1) * TN3_B_BYTES;
-        const int tile2 = st + 2 < steps ? st + 2 : steps - 1, stage2 = (st + 2) % TN3_A_STAGES;   /* past the end: the last one again, never used */
-        const bool fresh = st % spg == 0, last = (st + 1) % spg == 0;
-        const long long oa2 = off_a(tile2);
+        const int stage2 = stg2;                        /* tile st+2 (past the end: the last one again, never used) goes there */
+        const bool fresh = (st & (spg - 1)) == 0, last = ((st + 1) & (spg - 1)) == 0;
         i32x4 wnext; float fn[2];
         i32x4 wv[4];
         auto item = [&](int k){
-            if(k == 0)      wnext = tn3_gld16(pw + off_w(tile2));
+            if(k == 0)      wnext = tn3_gld16(pw + ow2);
             else if(k < 3){ if(last) fn[k - 1] = load_scale(st + 1, k - 1); else fn[k - 1] = fs_cur[k - 1]; }   /* a new scale only where a group ends */
             else if(k < 3 + 2 * NI)
                 __builtin_amdgcn_global_load_lds((glb_void *)(srcA[k - 3] + oa2),
@@ -265,6 +271,12 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, con
         asm volatile("s_waitcnt vmcnt(%3)" : "+v"(wnext), "+v"(fn[0]), "+v"(fn[1]) : "n"(2 * NI) : "memory");
         wcur = wnext;
         fs_cur[0] = fn[0]; fs_cur[1] = fn[1];
+        stg = stg == TN3_A_STAGES - 1 ? 0 : stg + 1;
+        stg2 = stg2 == TN3_A_STAGES - 1 ? 0 : stg2 + 1;
+        if(st + 3 < steps){
+            oa2 += TN3_BK * 2; ow2 += TN3_BK / 2;
+            if(st + 3 == steps1){ oa2 += jump_a; ow2 += jump_w; }       /* on to the second operand pair */
+        }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);                    /* vmcnt(0), as a builtin so that the compiler knows it: no request may outlive the workgroup's LDS */
 

@@ -73,6 +73,7 @@ SIGNATURES = {
     "qlmx_moe_gemm_nn_swiglu": (c_i, [c_vp, c_vp, c_i, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_nt": (c_i, [c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_decode_forward": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_moe_decode_forward_noalloc": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_step_touched": (c_i, [c_vp] * 10 + [c_i, c_i, c_i, c_f, c_f, c_f, c_f, c_f, c_f, c_f, c_u64, c_u64, c_vp, c_i, c_vp]),
     "qlmx_sqsum": (c_i, [c_vp, c_u64, c_vp, c_vp]),
     "qlmx_gnorm": (c_i, [c_vp, c_i, c_i, c_vp, c_vp]),
@@ -163,6 +164,9 @@ class Qlmx:
 
     def decode_forward(self, x, assign, gate, out, d, s, group, w1q, w3q, w2q, T, K, E, D, F, stream=None):
         self.call("qlmx_moe_decode_forward", x, assign, gate, out, d, s, group, w1q, w3q, w2q, T, K, E, D, F, stream)
+
+    def decode_forward_noalloc(self, x, assign, gate, out, d, s, group, w1q, w3q, w2q, T, K, E, D, F, stream=None):
+        self.call("qlmx_moe_decode_forward_noalloc", x, assign, gate, out, d, s, group, w1q, w3q, w2q, T, K, E, D, F, stream)
 
     def step_touched(self, P, Gc, d, r, s, m8, m8s, v8, v8s, touched, ntouched, group, dmax, lr, b1, b2, wd, sref,
                      inv_bc1, inv_sqrt_bc2, t, nt, gs=None, v4=0, stream=None):

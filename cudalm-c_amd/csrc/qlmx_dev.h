@@ -11,6 +11,7 @@
 void qlmx_set_error(const char *fmt, ...);
 int qlmx_cu_count(void);
 int  qlmx_check_ready(void);
+int  qlmx_decode_setup(int device);   /* per-device state of the decode entry points; qlmx_init calls it */
 #define QLMX_HIP(call, what)                                                                  \
     do { hipError_t e_ = (call);                                                              \
          if(e_ != hipSuccess){ qlmx_set_error("%s: %s", what, hipGetErrorString(e_));         \

@@ -281,8 +281,9 @@ int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const
  *   2. down tasks     (problem, 256-column chunk of D, K slice of F)                -> part2
  *      input rows h = silu(g) * u come from part1
  *   3. combine tasks  (token, 256-column chunk of D): out += gate * y from part2, passes in order.
- * Hand-over between lists: every partial sum is stored as one 8-byte word {value, epoch of this
- * call}; a consumer re-reads a word until it carries the current epoch. There are no flags to set,
+ * Hand-over between lists: every partial sum is stored as one 8-byte word {value, tag of this
+ * call}; a consumer re-reads a word until it carries the current tag (`epoch` below; the kernel
+ * derives it from a device word, see its first lines). There are no flags to set,
  * clear or fence, and a consumer pays one memory round trip when its producer is already done.
  * Every workgroup finishes all of its tasks of one list before it starts the next, tasks of list 1
  * never wait, and the grid is sized to be co-resident, so the waits cannot deadlock; they are also
@@ -321,6 +322,7 @@ struct DfArgs {
     int T, K, E, D, F;
     int R1, S1, NC1, R2, S2, NC2;
     u64 *part1, *part2; unsigned epoch; unsigned *status;
+    unsigned *ctl;            /* device words: [0] tag of the last finished call, [1] workgroups of this call that are done */
 };
 
 struct DfMeta {
@@ -506,8 +508,17 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
     __shared__ __align__(16) float xs[DF_NG][DF_RMAX][DF_MB];   /* x[m][r] * scale(r, g), the four m side by side */
     __shared__ float red[4 * DF_MB * DF_CW];
     __shared__ int giveup;
+    __shared__ unsigned tag;
     const int tid = threadIdx.x;
-    if(tid == 0) giveup = 0;
+    /* The tag of this call's partial sums is one more than the last finished call's, which lives in
+     * device memory: the host passes no counter, so a launch recorded in a graph tags every replay
+     * afresh. Every workgroup reads the word here; the last workgroup to finish moves it on (end of
+     * the kernel), which cannot happen before all of them have read it. 0 is the cleared state. */
+    if(tid == 0){
+        giveup = 0;
+        const unsigned last = __hip_atomic_load(a.ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        tag = last == 0xFFFFFFFFu ? 1u : last + 1u;
+    }
     const int npair = a.T * a.K;
     const int ng = a.group >= DF_CW ? 1 : DF_CW / a.group;
 
@@ -518,6 +529,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
         mt.ein[tid] = e;
     }
     __syncthreads();
+    a.epoch = __builtin_amdgcn_readfirstlane(tag);
     {
         const int j = tid & 63, part = tid >> 6, e = mt.ein[j];
         int rank = 0;
@@ -693,21 +705,77 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
             }
         }
     }
+    /* the last workgroup to get here closes the call: clears the count and publishes the tag */
+    if(tid == 0){
+        const unsigned done = __hip_atomic_fetch_add(a.ctl + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if(done == gridDim.x - 1){
+            __hip_atomic_store(a.ctl + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(a.ctl, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
 }
 #undef DF_LOAD
 
-struct DfWorkspace { u64 *part[2] = {nullptr, nullptr}; size_t words[2] = {0, 0}; unsigned *status = nullptr; unsigned epoch = 0; int grid = 0; };
-static DfWorkspace g_df;
+/* ------------------------------------------------------------------------------------------
+ * Host side. Per device: the launch shape, a status word in pinned host memory, a grow-only
+ * workspace for qlmx_moe_decode_forward, and the address of the fixed device array that
+ * qlmx_moe_decode_forward_noalloc uses instead. All of it is set up by qlmx_init (nothing is
+ * allocated by the entry points afterwards, except when the grow-only workspace has to grow).
+ * ---------------------------------------------------------------------------------------- */
+#define DF_CTL_BYTES 256
+/* Scratch of the allocation-free entry point: control words, then both lists of tagged partial sums.
+ * Every call on a device shares this one array; it is never cleared (words carry the tag of the call
+ * that wrote them, and static device memory starts as zeros = "never written"). */
+static __device__ __align__(256) unsigned char scratch[DF_CTL_BYTES + QLMX_DECODE_SCRATCH_BYTES];
 
-/* tagged partial sums: grow-only, cleared when (re)allocated so that no word carries a live epoch */
-static int df_reserve(int which, size_t words, hipStream_t st){
-    if(words <= g_df.words[which]) return QLMX_OK;
+struct DfSpace { u64 *part[2] = {nullptr, nullptr}; size_t words[2] = {0, 0}; unsigned *ctl = nullptr; };
+struct DfDevice {
+    bool ready = false;
+    unsigned *status = nullptr;            /* pinned host word a kernel sets when a bounded wait ran out */
+    int grid = 0;                          /* co-resident workgroups */
+    unsigned char *fixed = nullptr;        /* device address of `scratch` on this device */
+    DfSpace grown;                         /* qlmx_moe_decode_forward's workspace */
+};
+#define DF_MAX_DEVICES 16
+static DfDevice g_dfdev[DF_MAX_DEVICES];
+
+/* called by qlmx_init with `device` current */
+int qlmx_decode_setup(int device){
+    QLMX_REQUIRE(device >= 0 && device < DF_MAX_DEVICES, "decode setup: device %d is beyond the %d this library keeps state for", device, DF_MAX_DEVICES);
+    DfDevice &dv = g_dfdev[device];
+    if(dv.ready) return QLMX_OK;
+    QLMX_HIP(hipHostMalloc((void **)&dv.status, 64, hipHostMallocDefault), "decode status word");
+    *dv.status = 0;
+    int nb = 0; hipDeviceProp_t pr;
+    QLMX_HIP(hipGetDeviceProperties(&pr, device), "decode device properties");
+    QLMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, k_decode_fused, DF_THREADS, 0), "decode occupancy");
+    if(nb > 3) nb = 3;
+    dv.grid = (nb * pr.multiProcessorCount) & ~7;
+    QLMX_REQUIRE(dv.grid >= 8, "decode setup: device too small (%d resident workgroups)", dv.grid);
+    /* `scratch` names the array in host code; its memory on this device is wherever the loader put it */
+    void *sym = nullptr;
+    QLMX_HIP(hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)), "decode scratch address");
+    dv.fixed = (unsigned char *)sym;
+    QLMX_HIP(hipMalloc((void **)&dv.grown.ctl, DF_CTL_BYTES), "decode control words");
+    QLMX_HIP(hipMemset(dv.grown.ctl, 0, DF_CTL_BYTES), "decode control words clear");
+    dv.ready = true;
+    return QLMX_OK;
+}
+
+/* tagged partial sums: grow-only, cleared when (re)allocated so that no word carries a live tag */
+static int df_reserve(DfSpace &ws, int which, size_t words, hipStream_t st){
+    if(words <= ws.words[which]) return QLMX_OK;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    QLMX_HIP(hipStreamIsCapturing(st, &cap), "decode capture query");
+    QLMX_REQUIRE(cap == hipStreamCaptureStatusNone,
+                 "qlmx_moe_decode_forward: the workspace would have to grow while the stream is being captured; run the largest "
+                 "shape once outside the capture first, or use qlmx_moe_decode_forward_noalloc");
     QLMX_HIP(hipStreamSynchronize(st), "decode workspace sync");
-    if(g_df.part[which]) QLMX_HIP(hipFree(g_df.part[which]), "decode workspace free");
-    g_df.part[which] = nullptr; g_df.words[which] = 0;
-    QLMX_HIP(hipMalloc((void **)&g_df.part[which], words * sizeof(u64)), "decode partial sums");
-    QLMX_HIP(hipMemset(g_df.part[which], 0, words * sizeof(u64)), "decode partial sums clear");
-    g_df.words[which] = words;
+    if(ws.part[which]) QLMX_HIP(hipFree(ws.part[which]), "decode workspace free");
+    ws.part[which] = nullptr; ws.words[which] = 0;
+    QLMX_HIP(hipMalloc((void **)&ws.part[which], words * sizeof(u64)), "decode partial sums");
+    QLMX_HIP(hipMemset(ws.part[which], 0, words * sizeof(u64)), "decode partial sums clear");
+    ws.words[which] = words;
     return QLMX_OK;
 }
 
@@ -722,34 +790,26 @@ static int df_rows(int Kdim, double tasks_per_slice, int grid){
     return R;
 }
 
-extern "C" int qlmx_moe_decode_forward(const float *x, const int *assign, const float *gate, float *out,
-                                       const signed char *d, const float *s, int group,
-                                       unsigned long long w1q, unsigned long long w3q, unsigned long long w2q,
-                                       int T, int K, int E, int D, int F, void *stream){
+/* Both entry points: checks, launch shape, workspace (`fixed`: the static array, else the grow-only one), launch. */
+static int df_forward(bool fixed, const char *who, const float *x, const int *assign, const float *gate, float *out,
+                      const signed char *d, const float *s, int group, u64 w1q, u64 w3q, u64 w2q,
+                      int T, int K, int E, int D, int F, hipStream_t st){
     int rc = qlmx_check_ready(); if(rc) return rc;
-    hipStream_t st = (hipStream_t)stream;
-    QLMX_REQUIRE(x && assign && gate && out && d && s, "qlmx_moe_decode_forward: NULL buffer");
-    QLMX_REQUIRE(T > 0 && K > 0 && E > 0, "qlmx_moe_decode_forward: T=%d K=%d E=%d", T, K, E);
-    if(T * K > DEC_MAXPAIR){ qlmx_set_error("qlmx_moe_decode_forward: %d (pass, token) pairs exceed the limit of %d", T * K, DEC_MAXPAIR); return QLMX_E_LIMIT; }
-    QLMX_REQUIRE(D % 32 == 0 && F % 32 == 0 && D <= 8192 && F <= 8192, "qlmx_moe_decode_forward: D=%d F=%d must be multiples of 32, at most 8192", D, F);
-    QLMX_REQUIRE(group == 128 || (group > 0 && group % DF_CW == 0), "qlmx_moe_decode_forward: group %d is not supported (128 or a multiple of 256)", group);
-    QLMX_REQUIRE(F % group == 0 && D % group == 0, "qlmx_moe_decode_forward: group %d must divide D and F", group);
+    QLMX_REQUIRE(x && assign && gate && out && d && s, "%s: NULL buffer", who);
+    QLMX_REQUIRE(T > 0 && K > 0 && E > 0, "%s: T=%d K=%d E=%d", who, T, K, E);
+    if(T * K > DEC_MAXPAIR){ qlmx_set_error("%s: %d (pass, token) pairs exceed the limit of %d", who, T * K, DEC_MAXPAIR); return QLMX_E_LIMIT; }
+    QLMX_REQUIRE(D % 32 == 0 && F % 32 == 0 && D <= 8192 && F <= 8192, "%s: D=%d F=%d must be multiples of 32, at most 8192", who, D, F);
+    QLMX_REQUIRE(group == 128 || (group > 0 && group % DF_CW == 0), "%s: group %d is not supported (128 or a multiple of 256)", who, group);
+    QLMX_REQUIRE(F % group == 0 && D % group == 0, "%s: group %d must divide D and F", who, group);
     QLMX_REQUIRE(w1q % group == 0 && w3q % group == 0 && w2q % group == 0 && ((uintptr_t)d & 15) == 0,
-                 "qlmx_moe_decode_forward: weight offsets must be multiples of the group and the digit array 16-byte aligned");
-    if(!g_df.status){
-        QLMX_HIP(hipHostMalloc((void **)&g_df.status, 64, hipHostMallocDefault), "decode status word");
-        *g_df.status = 0;
-        int nb = 0, dev = 0; hipDeviceProp_t pr;
-        QLMX_HIP(hipGetDevice(&dev), "decode device");
-        QLMX_HIP(hipGetDeviceProperties(&pr, dev), "decode device properties");
-        QLMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, k_decode_fused, DF_THREADS, 0), "decode occupancy");
-        if(nb > 3) nb = 3;
-        g_df.grid = (nb * pr.multiProcessorCount) & ~7;
-        QLMX_REQUIRE(g_df.grid >= 8, "qlmx_moe_decode_forward: device too small (%d resident workgroups)", g_df.grid);
-    }
-    if(*(volatile unsigned *)g_df.status){
-        *g_df.status = 0;
-        qlmx_set_error("qlmx_moe_decode_forward: an earlier call gave up waiting for a task of its own grid; its output is invalid");
+                 "%s: weight offsets must be multiples of the group and the digit array 16-byte aligned", who);
+    int device = -1;
+    QLMX_HIP(hipGetDevice(&device), "decode device");
+    QLMX_REQUIRE(device >= 0 && device < DF_MAX_DEVICES && g_dfdev[device].ready, "%s: qlmx_init has not run for device %d", who, device);
+    DfDevice &dv = g_dfdev[device];
+    if(*(volatile unsigned *)dv.status){
+        *dv.status = 0;
+        qlmx_set_error("%s: an earlier decode call gave up waiting for a task of its own grid; its output is invalid", who);
         return QLMX_E_HIP;
     }
     const int npair = T * K;
@@ -759,16 +819,41 @@ extern "C" int qlmx_moe_decode_forward(const float *x, const int *assign, const 
     a.T = T; a.K = K; a.E = E; a.D = D; a.F = F;
     a.NC1 = (F + DF_CW - 1) / DF_CW; a.NC2 = (D + DF_CW - 1) / DF_CW;
     const double hits = E * (1.0 - pow(1.0 - 1.0 / E, (double)npair));
-    a.R1 = df_rows(D, 2.0 * hits * a.NC1, g_df.grid); a.S1 = (D + a.R1 - 1) / a.R1;
-    a.R2 = DF_RMAX;                                     a.S2 = (F + a.R2 - 1) / a.R2;
-    rc = df_reserve(0, (size_t)npair * 2 * a.S1 * DF_MB * F, st); if(rc) return rc;
-    rc = df_reserve(1, (size_t)npair * a.S2 * DF_MB * D, st); if(rc) return rc;
-    a.part1 = g_df.part[0]; a.part2 = g_df.part[1]; a.status = g_df.status;
-    a.epoch = ++g_df.epoch;
-    if(a.epoch == 0) a.epoch = ++g_df.epoch;          /* 0 is the cleared state */
+    a.R1 = df_rows(D, 2.0 * hits * a.NC1, dv.grid); a.S1 = (D + a.R1 - 1) / a.R1;
+    a.R2 = DF_RMAX;                                  a.S2 = (F + a.R2 - 1) / a.R2;
+    const size_t words1 = (size_t)npair * 2 * a.S1 * DF_MB * F, words2 = (size_t)npair * a.S2 * DF_MB * D;
+    if(fixed){
+        if((words1 + words2) * sizeof(u64) > (size_t)QLMX_DECODE_SCRATCH_BYTES){
+            qlmx_set_error("%s: T=%d K=%d D=%d F=%d needs %zu bytes of partial sums, the fixed scratch holds %zu",
+                           who, T, K, D, F, (words1 + words2) * sizeof(u64), (size_t)QLMX_DECODE_SCRATCH_BYTES);
+            return QLMX_E_LIMIT;
+        }
+        a.ctl = (unsigned *)dv.fixed;
+        a.part1 = (u64 *)(dv.fixed + DF_CTL_BYTES); a.part2 = a.part1 + words1;
+    } else {
+        rc = df_reserve(dv.grown, 0, words1, st); if(rc) return rc;
+        rc = df_reserve(dv.grown, 1, words2, st); if(rc) return rc;
+        a.ctl = dv.grown.ctl; a.part1 = dv.grown.part[0]; a.part2 = dv.grown.part[1];
+    }
+    a.status = dv.status; a.epoch = 0;
     const long long most = (long long)2 * npair * a.NC1 * a.S1;
-    const int grid = (int)std::min<long long>(g_df.grid, (most + 7) & ~7LL);
+    const int grid = (int)std::min<long long>(dv.grid, (most + 7) & ~7LL);
     hipLaunchKernelGGL(k_decode_fused, dim3(grid), dim3(DF_THREADS), 0, st, a);
     QLMX_LAUNCH_CHECK("decode launch");
     return QLMX_OK;
+}
+
+extern "C" int qlmx_moe_decode_forward(const float *x, const int *assign, const float *gate, float *out,
+                                       const signed char *d, const float *s, int group,
+                                       unsigned long long w1q, unsigned long long w3q, unsigned long long w2q,
+                                       int T, int K, int E, int D, int F, void *stream){
+    return df_forward(false, "qlmx_moe_decode_forward", x, assign, gate, out, d, s, group, w1q, w3q, w2q, T, K, E, D, F, (hipStream_t)stream);
+}
+
+/* The same layer over the fixed device array: no hipMalloc, hipFree or other allocating call on any path. */
+extern "C" int qlmx_moe_decode_forward_noalloc(const float *x, const int *assign, const float *gate, float *out,
+                                               const signed char *d, const float *s, int group,
+                                               unsigned long long w1q, unsigned long long w3q, unsigned long long w2q,
+                                               int T, int K, int E, int D, int F, void *stream){
+    return df_forward(true, "qlmx_moe_decode_forward_noalloc", x, assign, gate, out, d, s, group, w1q, w3q, w2q, T, K, E, D, F, (hipStream_t)stream);
 }

@@ -46,6 +46,7 @@ extern "C" int qlmx_init(int device){
         qlmx_set_error("qlmx_init: device is %s; this library carries gfx950 code only", pr.gcnArchName);
         return QLMX_E_NODEV;
     }
+    int rc = qlmx_decode_setup(device); if(rc) return rc;
     g_ready = 1;
     return QLMX_OK;
 }

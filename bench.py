@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=30)
-    ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train", "train5", "codec", "glue", "copy"])
+    ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train", "train5", "c5", "codec", "glue", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--step-only", action="store_true", help="train: skip the per-launch repetitions, so that a kernel trace holds nothing but steps")
     ap.add_argument("--adamw-weights", type=int, default=120 * 2 ** 20)
@@ -175,6 +175,129 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": None, "kernel": "k_gemm_nn_lds, k_gemm_tn_lds, k_gemm_nt_lds (all 6 launches; slowest: %s)" % dom,
                      "note": "algorithmic flops only; the forward issues two MFMAs per product (bf16 hi+lo weight split)"},
+    }
+
+
+# --------------------------------------------------------------------------------------------- c5
+def bench_c5(torch, q, args, L=8, E=64, D=2048, F=1408, tokens=32768, topk=4):
+    """Config 5 whole: 8 layers x (E=64, top-4, D=2048, F=1408), 131072 expert rows per layer with Zipf(1.1) loads
+    (a different draw per layer): every layer's 9 expert GEMMs in the order of moe_forward / moe_backward
+    (cudalm.cu:4211-4225, 4333-4366) over that layer's own 553.6 M packed weights, the weight gradients written
+    into one fp32 G of 4.43 G elements; then one Integer AdamW step (cudalm.cu:6082-6103) over all 4.43 G weights.
+    A step of this workload is heavy (about 0.1 s), so it is timed over max(3, K // 10) steps after max(1, W // 10)
+    warm-up steps; both figures are in the result."""
+    import numpy as np
+    from cudalm_c_amd.binding import ACT_BF16, MATH_MFMA, SPAN_DTYPE
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev); g.manual_seed(0)
+    group = 128
+    EDF = E * D * F
+    nlayer = 3 * EDF
+    nq = L * nlayer
+    ng = nq // group
+    rows = tokens * topk
+    steps, warmup = max(3, args.steps // 10), max(1, args.warmup // 10)
+
+    def chunks(n, fn, dtype):
+        out = torch.empty(n, dtype=dtype, device=dev)
+        for i in range(0, n, 1 << 30):
+            m = min(1 << 30, n - i)
+            out[i:i + m] = fn(m)
+        return out
+
+    def packed(m):
+        b = torch.randint(0, 256, (m,), dtype=torch.int16, device=dev, generator=g).to(torch.uint8)
+        lo = b & 15; hi = b >> 4
+        lo = torch.where(lo == 8, torch.zeros_like(lo), lo); hi = torch.where(hi == 8, torch.zeros_like(hi), hi)
+        return (lo | (hi << 4)).view(torch.int8)
+
+    d = chunks(nq // 2, packed, torch.int8)
+    s = (0.02 * 3 / 7) * (0.5 + torch.rand(ng, device=dev, generator=g))
+    G = torch.zeros(nq, device=dev)
+
+    def bf16(n):
+        return torch.randn(n, device=dev, generator=g).to(torch.bfloat16)
+
+    Xp, ap, dyp, dgp, dup = bf16(rows * D), bf16(rows * F), bf16(rows * D), bf16(rows * F), bf16(rows * F)
+    gp = torch.empty(rows * F, device=dev); up = torch.empty(rows * F, device=dev); yp = torch.empty(rows * D, device=dev)
+    dap = torch.empty(rows * F, device=dev); dXp = torch.empty(rows * D, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    P = q.problems
+    calls = []
+    loads = []
+    for l in range(L):
+        cnt = zipf_counts(E, tokens, topk, seed=100 + l)
+        loads.append((int(cnt.max()), int(cnt.min())))
+        off = np.concatenate([[0], np.cumsum(cnt)]).astype(int)
+        o1, o3, o2 = l * nlayer, l * nlayer + EDF, l * nlayer + 2 * EDF
+
+        def items(A, a_w, B, b_w, Cm, c_w, wbase, per_expert_c=False, beta=0.0):
+            return [(A.data_ptr() + int(off[e]) * a_w * 2, (B.data_ptr() + int(off[e]) * b_w * 2) if B is not None else None,
+                     (Cm.data_ptr() + (wbase + e * D * F) * 4) if per_expert_c else (Cm.data_ptr() + int(off[e]) * c_w * 4),
+                     wbase + e * D * F, (wbase + e * D * F) // group, int(cnt[e]), beta) for e in range(E)]
+
+        p_w13 = P(items(Xp, D, None, 0, gp, F, o1) + items(Xp, D, None, 0, up, F, o3))
+        p_w2 = P(items(ap, F, None, 0, yp, D, o2))
+        p_g2 = P(items(ap, F, dyp, D, G, 0, o2, True))
+        p_d2 = P(items(dyp, D, None, 0, dap, F, o2))
+        p_g13 = P(items(Xp, D, dgp, F, G, 0, o1, True) + items(Xp, D, dup, F, G, 0, o3, True))
+        p_d1 = P(items(dgp, F, None, 0, dXp, D, o1)); p_d3 = P(items(dup, F, None, 0, dXp, D, o3, beta=1.0))
+        calls += [
+            (lambda p=p_w13: q.gemm_nn(d, s, group, p, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream)),
+            (lambda p=p_w2: q.gemm_nn(d, s, group, p, E, F, D, ACT_BF16, MATH_MFMA, stream)),
+            (lambda p=p_g2: q.gemm_nt(p, E, F, D, ACT_BF16, MATH_MFMA, stream)),
+            (lambda p=p_d2: q.gemm_tn(d, s, group, p, E, D, F, ACT_BF16, MATH_MFMA, stream)),
+            (lambda p=p_g13: q.gemm_nt(p, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream)),
+            (lambda p=p_d1, pp=p_d3: q.gemm_tn_pair(d, s, group, p, pp, E, F, D, ACT_BF16, MATH_MFMA, stream)),
+        ]
+
+    def gemms():
+        for fn in calls:
+            fn()
+
+    tg = timed(torch, gemms, steps, warmup)
+    flops = L * 9 * 2.0 * rows * D * F
+    tf = flops / (tg["event_ms_avg"] * 1e-3) / 1e12
+    del Xp, ap, dyp, dgp, dup, gp, up, yp, dap, dXp
+
+    # ---- the optimizer step over every weight of the stack ----
+    def ri(lo, hi, dtype):
+        return lambda m: torch.randint(lo, hi, (m,), dtype=torch.int16, device=dev, generator=g).to(dtype)
+    r = chunks(nq, ri(-64, 65, torch.int8), torch.int8)
+    m8 = chunks(nq, ri(-127, 128, torch.int8), torch.int8)
+    v8 = chunks(nq, ri(0, 256, torch.uint8), torch.uint8)
+    m8s = (3e-3 / 127) * (0.5 + torch.rand(ng, device=dev, generator=g))
+    v8s = (3e-3 / 255) * (0.5 + torch.rand(ng, device=dev, generator=g))
+    tab = np.zeros(3 * L, dtype=SPAN_DTYPE)
+    smean = float(s.mean())
+    for i in range(3 * L):
+        tab[i] = (i * EDF, i * EDF, i * EDF, EDF, i * (EDF // group), EDF // group, smean, 0)
+    sp = torch.from_numpy(tab.view(np.uint8)).to(dev)
+    gscale = 1e-3 / max(float(G[:1 << 24].std()), 1e-20)      # the weight gradients just computed, brought to the ~1e-3 scale the config names
+    state = {"t": 0}
+    b1, b2 = 0.9, 0.95
+
+    def step():
+        state["t"] += 1
+        t = state["t"]
+        q.step(None, G, d, r, s, m8, m8s, v8, v8s, sp, 3 * L, group, 7, 3e-4, b1, b2, 0.1, gscale, None,
+               1.0 / (1.0 - b1 ** t), 1.0 / (1.0 - b2 ** t) ** 0.5, 0, t, 1, None, 1, 0, ng, 0, stream)
+
+    ta = timed(torch, step, steps, warmup)
+    bytes_per_w = 11.0 + 20.0 / 128
+    gbs = nq * bytes_per_w / (ta["event_ms_avg"] * 1e-3) / 1e9
+    return {
+        "workload": "C5 whole stack: %d layers x (E=%d top-%d D=%d F=%d), %d bf16 tokens -> %d expert rows per layer, Zipf(1.1) load per layer "
+                    "(max/min rows %s); fwd+dgrad+wgrad = %d grouped GEMMs in %d launches, then one Integer AdamW step over %d weights"
+                    % (L, E, topk, D, F, tokens, rows, "/".join("%d:%d" % x for x in loads[:2]) + "...", 9 * L, 6 * L, nq),
+        "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tg["wall_ms"] + ta["wall_ms"], "dtype": "bf16",
+        "steps": steps, "warmup": warmup,
+        "gemm": {"ms": tg["event_ms_avg"], "tflops": tf, "tflop_per_step": flops / 1e12},
+        "adamw": {"ms": ta["event_ms_avg"], "gbs": gbs, "weights": nq, "weights_per_s": nq / (ta["event_ms_avg"] * 1e-3), "bytes_per_weight": bytes_per_w},
+        "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": None, "kernel": "k_gemm_nn_lds, k_gemm_tn_lds, k_gemm_nt_lds (all %d launches)" % (6 * L)},
+        "roofline_adamw": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                           "kernel": "k_qlmx_step<adam>, one launch over all %d weights" % nq},
     }
 
 
@@ -472,14 +595,14 @@ def main():
     pkg = load_package()
     q = pkg.load()           # raises if libqlmx.so is missing or no gfx950 device
     torch.cuda.set_device(0)
-    want = ["train", "decode", "adamw"] if args.workload == "all" else [args.workload]
-    runners = {"adamw": bench_adamw, "train": bench_train, "decode": bench_decode, "copy": bench_copy, "codec": bench_codec, "glue": bench_glue,
+    want = ["train", "decode", "adamw", "c5"] if args.workload == "all" else [args.workload]
+    runners = {"adamw": bench_adamw, "train": bench_train, "decode": bench_decode, "copy": bench_copy, "codec": bench_codec, "glue": bench_glue, "c5": bench_c5,
                "train5": lambda t, qq, a: bench_train(t, qq, a, E=64, D=2048, F=1408, tokens=32768, topk=4, label="C5 train layer (one of 8)")}
     results = {}
     for w in want:
         if w in runners:
             results[w] = runners[w](torch, q, args)
-    first = next(results[w] for w in ["train", "train5", "decode", "adamw", "codec", "glue", "copy"] if w in results)
+    first = next(results[w] for w in ["train", "train5", "c5", "decode", "adamw", "codec", "glue", "copy"] if w in results)
     line = {
         "metric": "QLM expert dequant-GEMM TFLOP/s & GB/s (% roofline); int-AdamW GB/s",
         "value": first["value"], "unit": first["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -113,6 +113,7 @@ class Oracle(_Lib):
         self._q4n_d = s("orc_q4n_dequantize", c_i, [c_vp, c_sz, c_vp, c_sz, c_i])
         self._ws_new = s("orc_moe_ws_new", c_vp, [c_i, c_i, c_i, c_i, c_i])
         self._ws_free = s("orc_moe_ws_free", None, [c_vp])
+        self._ws_bf16 = s("orc_moe_ws_bf16", None, [c_vp, c_i])
         self._moe_fwd = s("orc_moe_forward", c_i, [c_vp] * 8)
         self._moe_bwd = s("orc_moe_backward", None, [c_vp] * 12)
         self._fill_normal = s("orc_fill_normal", None, [c_vp, c_sz, c_u64, c_u64, c_f])
@@ -161,6 +162,26 @@ class Oracle(_Lib):
 
     def servo(self, d, r, s, tab, group, dmax, f_hi, f_lo, packed, ngrp):
         self._servo(_p(d), _p(r), _p(s), _p(tab), len(tab), group, dmax, f_hi, f_lo, packed, ngrp)
+
+    def step_slice(self, G, d, r, s, m8, m8s, v8, v8s, qi0, gi0, sref, group, dmax, lr, b1, b2, wd, gscale,
+                   inv_bc1, inv_sqrt_bc2, lrmode, t, adam, v4=0):
+        """The step over a cut-out piece of a much larger packed state: the arrays hold only elements
+        qi0 .. qi0+r.size (groups gi0 ..) of the whole, and the arithmetic (hash keys are functions of the
+        global element index) is that of the whole sweep. Groups are independent, so this equals the same
+        groups of a step over everything. The pointers handed to the C function are moved back by the
+        piece's offset; only the piece is ever touched."""
+        n = r.size
+        assert n % group == 0 and qi0 % 2 == 0 and d.size * 2 == n and G.size == n and s.size * group == n
+        tab = np.zeros(1, dtype=SPAN_DTYPE)
+        tab[0] = (0, 0, qi0, n, gi0, n // group, sref, 0)
+        for a in (G, d, r, s, m8, m8s, v8, v8s):
+            assert a.flags["C_CONTIGUOUS"]
+
+        def back(a, off_bytes):
+            return c_vp(a.ctypes.data - off_bytes)
+        self._step(None, _p(G), back(d, qi0 // 2), back(r, qi0), back(s, 4 * gi0), back(m8, qi0), back(m8s, 4 * gi0),
+                   back(v8, qi0), back(v8s, 4 * gi0), _p(tab), 1, group, dmax, lr, b1, b2, wd, gscale, None,
+                   inv_bc1, inv_sqrt_bc2, lrmode, t, adam, None, 1, gi0, n // group, v4)
 
     def gemm_nn(self, A, B, Cm, M, K, N):
         self._gemm_nn(_p(A), _p(B), _p(Cm), M, K, N)
@@ -242,9 +263,11 @@ class Oracle(_Lib):
         ok = self._q4n_d(_p(buf), buf.size, _p(P), n, group)
         return ok, P
 
-    def moe_forward(self, x, w1, w3, w2, assign, gate, out, N, D, F, E, K):
-        """returns (rc, ws) -- keep ws for moe_backward, free with moe_ws_free"""
+    def moe_forward(self, x, w1, w3, w2, assign, gate, out, N, D, F, E, K, bf16_inter=False):
+        """returns (rc, ws) -- keep ws for moe_backward, free with moe_ws_free. bf16_inter: the GEMM inputs
+        (Xp, ap, dyp, dgp, dup) are stored rounded to bf16 in both directions, as the reference's GPU path does."""
         ws = self._ws_new(N, D, F, E, K)
+        self._ws_bf16(ws, 1 if bf16_inter else 0)
         rc = self._moe_fwd(ws, _p(x), _p(w1), _p(w3), _p(w2), _p(assign), _p(gate), _p(out))
         return rc, ws
 

@@ -589,6 +589,9 @@ orc_moe_ws *orc_moe_ws_new(int N, int D, int F, int E, int K){
     w->dap = (float *)malloc(4*nf); w->dgp = (float *)malloc(4*nf); w->dup = (float *)malloc(4*nf);
     return w;
 }
+void orc_moe_ws_bf16(orc_moe_ws *w, int on){ w->bf16_inter = on; }
+void orc_bf16_round_n(float *x, size_t n);
+static void inter(const orc_moe_ws *w, float *x, size_t n){ if(w->bf16_inter) orc_bf16_round_n(x, n); }
 void orc_moe_ws_free(orc_moe_ws *w){
     if(!w) return;
     free(w->perm); free(w->off); free(w->Xp); free(w->yp); free(w->gp); free(w->up); free(w->ap);
@@ -603,6 +606,7 @@ static void experts_fwd(orc_moe_ws *w, const int *off, const float *w1, const fl
         orc_gemm_nn(w->Xp + (size_t)off[e]*D, w3 + e*DF, w->up + (size_t)off[e]*F, ne, D, F);
     }
     orc_swiglu(w->gp, w->up, w->ap, (size_t)w->N*F);
+    inter(w, w->ap, (size_t)w->N*F);
     for(int e = 0; e < w->E; e++){
         int ne = off[e+1] - off[e]; if(!ne) continue;
         orc_gemm_nn(w->ap + (size_t)off[e]*F, w2 + e*DF, w->yp + (size_t)off[e]*D, ne, F, D);
@@ -622,6 +626,7 @@ int orc_moe_forward(orc_moe_ws *w, const float *x, const float *w1, const float 
     for(int k = 0; k < w->K; k++){
         int *prm = w->perm + (size_t)k*N, *off = w->off + (size_t)k*(E+1);
         orc_gather(x, prm, w->Xp, N, D);
+        inter(w, w->Xp, (size_t)N*D);
         experts_fwd(w, off, w1, w3, w2);
         orc_scatter_gate(w->yp, prm, gate + (size_t)k*N, out, N, D);
     }
@@ -638,14 +643,17 @@ void orc_moe_backward(orc_moe_ws *w, const float *x, const float *w1, const floa
     for(int k = 0; k < w->K; k++){
         int *prm = w->perm + (size_t)k*N, *off = w->off + (size_t)k*(E+1);
         orc_gather(x, prm, w->Xp, N, D);
+        inter(w, w->Xp, (size_t)N*D);
         experts_fwd(w, off, w1, w3, w2);
         orc_moe_dgate(dout, w->yp, prm, gate + (size_t)k*N, dgate + (size_t)k*N, w->dyp, N, D);
+        inter(w, w->dyp, (size_t)N*D);
         for(int e = 0; e < E; e++){
             int ne = off[e+1] - off[e]; if(!ne) continue;
             orc_gemm_nt(w->ap + (size_t)off[e]*F, w->dyp + (size_t)off[e]*D, Gw2 + e*DF, ne, F, D);
             orc_gemm_tn(w->dyp + (size_t)off[e]*D, w2 + e*DF, w->dap + (size_t)off[e]*F, ne, D, F, 0.0f);
         }
         orc_swiglu_bwd(w->gp, w->up, w->dap, w->dgp, w->dup, (size_t)N*F);
+        inter(w, w->dgp, (size_t)N*F); inter(w, w->dup, (size_t)N*F);
         for(int e = 0; e < E; e++){
             int ne = off[e+1] - off[e]; if(!ne) continue;
             orc_gemm_nt(w->Xp + (size_t)off[e]*D, w->dgp + (size_t)off[e]*F, Gw1 + e*DF, ne, D, F);

@@ -102,7 +102,11 @@ typedef struct {
     int *off;       /* [K][E+1]    */
     float *Xp, *gp, *up, *ap, *yp;           /* per-pass scratch, N rows      */
     float *dyp, *dap, *dgp, *dup, *dXp;      /* backward scratch              */
+    int bf16_inter;  /* 1: the GEMM inputs Xp, ap, dyp, dgp, dup are stored rounded to bf16, as the reference's
+                      * GPU path stores them (hbf buffers of bfm_ffn / bfm_bwd, cudalm.cu:4001-4008, 4061-4087);
+                      * everything else stays fp32. 0 (default): the CPU build's all-fp32 layer. */
 } orc_moe_ws;
+void orc_moe_ws_bf16(orc_moe_ws *w, int on);
 orc_moe_ws *orc_moe_ws_new(int N, int D, int F, int E, int K);
 void orc_moe_ws_free(orc_moe_ws *w);
 int  orc_moe_forward(orc_moe_ws *w, const float *x, const float *w1, const float *w3, const float *w2,

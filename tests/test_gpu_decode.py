@@ -79,7 +79,7 @@ def test_gemv_small_rows_vs_oracle(q, orc, K, N):
         assert orc.relerr(o.cpu().numpy(), want) < 1e-5
 
 
-@pytest.mark.parametrize("T,E,D,F,K", [(1, 32, 768, 2048, 2), (4, 8, 768, 2048, 2), (16, 8, 768, 2048, 2),
+@pytest.mark.parametrize("T,E,D,F,K", [(1, 32, 768, 2048, 2), (4, 32, 768, 2048, 2), (16, 32, 768, 2048, 2), (4, 8, 768, 2048, 2), (16, 8, 768, 2048, 2),
                                        (16, 4, 256, 384, 4), (5, 3, 128, 256, 1), (7, 6, 1024, 640, 3), (3, 4, 2048, 256, 2)])
 def test_decode_forward_vs_oracle_layer(q, orc, T, E, D, F, K):
     import torch

@@ -158,3 +158,12 @@ def test_train_size_mfma_vs_fp32_kernels_and_properties(q, orc, E, D, F, rows):
         orc.gemm_tn(B, P, want, m, F, D, 0.0)
         got = dX1[int(off[e]) * D:(int(off[e]) + m) * D].cpu().numpy()
         assert orc.relerr(got, want) < 1e-3
+    # weight gradients of the most loaded expert (its contraction is the one the launch cuts into slices) and
+    # of the least loaded one, over all of their rows, against the oracle
+    for e in (int(np.argmax(cnt)), int(np.argmin(np.where(cnt > 0, cnt, 1 << 30)))):
+        m = int(cnt[e])
+        A = X[int(off[e]) * D:(int(off[e]) + m) * D].float().cpu().numpy()
+        B = dY[int(off[e]) * F:(int(off[e]) + m) * F].float().cpu().numpy()
+        want = np.zeros(D * F, f32)
+        orc.gemm_nt(A, B, want, m, D, F)
+        assert orc.relerr(G1[e * D * F:(e + 1) * D * F].cpu().numpy(), want) < 1e-3, (e, m)

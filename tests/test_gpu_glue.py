@@ -6,7 +6,8 @@ points, against the CPU oracle (orc_moe_forward / orc_moe_backward follow cudalm
 Bars: indices (assign, perm, off), gate probabilities and every pure data move are bit-exact; SwiGLU
 and the dot product of the gate gradient follow the oracle to 1e-6 relative L2; layer outputs to 1e-5
 with the fp32 GEMMs. With the bf16 MFMA GEMMs each GEMM meets 1e-3 on equal inputs (tested with the
-GEMMs); the whole layer, whose intermediates are then stored as bf16, is held to 4e-3 here."""
+GEMMs); the whole layer, whose GEMM inputs are then stored as bf16, meets 1e-3 against the oracle's layer
+with the same five buffers rounded to bf16, and 4e-3 against the all-fp32 layer."""
 import numpy as np
 import pytest
 
@@ -290,9 +291,11 @@ class GpuLayer:
 def test_layer_forward_backward_vs_oracle(q, orc, math, N, E, D, F, K):
     import torch
     mth = pkg.MATH_MFMA if math == "mfma" else pkg.MATH_F32
-    # bf16 storage of the intermediates (ap, dyp, dgp, dup) alone is worth 2^-9/sqrt(3) = 1.1e-3 of relative
-    # error per element; the reference holds its own bf16 path to 3e-2 (cudalm.cu:10430)
-    tol = 4e-3 if math == "mfma" else 1e-5
+    # MFMA layer: the GEMM inputs ap, dyp, dgp, dup are stored as bf16 (as the reference's GPU path stores them,
+    # cudalm.cu:4001-4008, 4061-4087). The oracle rounds the same five buffers, so what is compared is the GEMMs'
+    # own error: 1e-3 as for every matmul output. Against the all-fp32 layer the storage rounding alone is worth
+    # 2^-9/sqrt(3) = 1.1e-3 per rounded operand; that end-to-end distance is checked second, at 4e-3.
+    tol = 1e-3 if math == "mfma" else 1e-5
     d, s, P, n = encode_layer(orc, 40 + N, E, D, F)
     x = orc.normal(N * D, 41, 1)
     dout = orc.normal(N * D, 41, 2)
@@ -303,12 +306,16 @@ def test_layer_forward_backward_vs_oracle(q, orc, math, N, E, D, F, K):
     orc.router_topk(rt, pr, asn, gate, N, E, K)
     # oracle
     w_out = np.zeros(N * D, f32)
-    rc, ws = orc.moe_forward(x, P[:n], P[n:2 * n], P[2 * n:], asn, gate, w_out, N, D, F, E, K)
-    assert rc == 0
-    w_dx = np.zeros(N * D, f32); w_dgate = np.zeros(K * N, f32)
-    w_G = [np.zeros(n, f32) for _ in range(3)]
-    orc.moe_backward(ws, x, P[:n], P[n:2 * n], P[2 * n:], gate, dout, w_dx, w_dgate, w_G[0], w_G[1], w_G[2])
-    orc.moe_ws_free(ws)
+    def oracle_layer(bf16_inter):
+        o = np.zeros(N * D, f32)
+        rc, ws = orc.moe_forward(x, P[:n], P[n:2 * n], P[2 * n:], asn, gate, o, N, D, F, E, K, bf16_inter=bf16_inter)
+        assert rc == 0
+        dx_, dg_ = np.zeros(N * D, f32), np.zeros(K * N, f32)
+        Gs = [np.zeros(n, f32) for _ in range(3)]
+        orc.moe_backward(ws, x, P[:n], P[n:2 * n], P[2 * n:], gate, dout, dx_, dg_, Gs[0], Gs[1], Gs[2])
+        orc.moe_ws_free(ws)
+        return o, dx_, dg_, Gs
+    w_out, w_dx, w_dgate, w_G = oracle_layer(math == "mfma")
     # library: router and grouping on the device too
     dpr, dasn, dgt = zeros(N * E), zeros(K * N, torch.int32), zeros(K * N)
     q.router_topk(dev(rt), dpr, dasn, dgt, N, E, K)
@@ -321,8 +328,14 @@ def test_layer_forward_backward_vs_oracle(q, orc, math, N, E, D, F, K):
     L.backward(dx_, dgt, ddout, dx, dgate, G[0], G[1], G[2])
     torch.cuda.synchronize()
     assert np.array_equal(dasn.cpu().numpy(), asn)
-    assert orc.relerr(out.cpu().numpy(), w_out) < tol
-    assert orc.relerr(dx.cpu().numpy(), w_dx) < tol
-    assert orc.relerr(dgate.cpu().numpy(), w_dgate) < tol
-    for got, want in zip(G, w_G):
-        assert orc.relerr(got.cpu().numpy(), want) < tol
+    got = {"out": out, "dx": dx, "dgate": dgate, "G_w1": G[0], "G_w3": G[1], "G_w2": G[2]}
+    want = {"out": w_out, "dx": w_dx, "dgate": w_dgate, "G_w1": w_G[0], "G_w3": w_G[1], "G_w2": w_G[2]}
+    errs = {k: orc.relerr(got[k].cpu().numpy(), want[k]) for k in got}
+    print("layer %s N=%d E=%d D=%d F=%d relative L2 per output:" % (math, N, E, D, F), {k: "%.2e" % v for k, v in errs.items()})
+    assert max(errs.values()) < tol, errs
+    if math == "mfma":
+        f_out, f_dx, f_dgate, f_G = oracle_layer(False)             # the CPU build's all-fp32 layer, end to end
+        want = {"out": f_out, "dx": f_dx, "dgate": f_dgate, "G_w1": f_G[0], "G_w3": f_G[1], "G_w2": f_G[2]}
+        e2e = {k: orc.relerr(got[k].cpu().numpy(), want[k]) for k in got}
+        print("    against the all-fp32 layer:", {k: "%.2e" % v for k, v in e2e.items()})
+        assert max(e2e.values()) < 4e-3, e2e

@@ -448,7 +448,7 @@ def cpu_adamw(args):
         t_used += time.perf_counter() - t0
         reps += 1
     gbs = nq * 15.16 * reps / t_used / 1e9
-    return {"value": gbs, "unit": "GB/s", "cores": threads, "kind": kind,
+    return {"value": gbs, "unit": "GB/s", "cores": threads, "cpu": cpu_model(), "kind": kind,
             "sample": "Integer AdamW (P rendered, 15.16 B/weight) over %d weights x %d steps, %s" % (nq, reps, "cpu_kern.h cpu_qlm_step" if kind == "reference" else "oracle/qlm_oracle.c"),
             "weights_per_s": nq * reps / t_used}
 
@@ -572,9 +572,90 @@ def cpu_gemm(args):
         t_used += time.perf_counter() - t0
         reps += 1
     tf = 3 * 2.0 * M * D * F * reps / t_used / 1e12
-    return {"value": tf, "unit": "TFLOP/s", "cores": threads, "kind": kind,
+    return {"value": tf, "unit": "TFLOP/s", "cores": threads, "cpu": cpu_model(), "kind": kind,
             "sample": "one expert, %d rows, D=%d F=%d: fwd + dgrad + wgrad fp32 SGEMM on the rendered view, %d repetitions (%s)"
                       % (M, D, F, reps, "cpu_rt.h sg_core via g_ab/g_abt_b/g_atb" if kind == "reference" else "oracle/qlm_oracle.c")}
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_decode(args, E=32, D=768, F=2048, topk=2, T=16, layers=2):
+    """Reference CPU path of the decode shape on a bounded sample: the expert part of moe_forward for T=16 tokens top-2
+    (cudalm.cu:4193-4228: per expert hit mg_ab on w1 and w3, flush, SwiGLU, mg_ab on w2, flush; with <= 4 rows per
+    expert the reference SGEMM takes its small-R path, cpu_rt.h:233-258) over `layers` distinct layers of rendered
+    fp32 weights, cycled for about 10 s. The rate is quoted in the GPU leg's unit -- bytes of PACKED digits and scales
+    of the distinct experts hit per second -- although the CPU path reads the 8x larger fp32 view."""
+    import numpy as np
+    from oracle.binding import Oracle, Ref, have_ref
+    orc = Oracle()
+    threads = min(16, os.cpu_count() or 1)
+    kind = "reference" if have_ref() else "port"
+    lib = Ref(threads=threads) if kind == "reference" else orc
+    orc.set_threads(threads)
+    per_expert = 3 * D * F // 2 + 3 * D * F // 128 * 4
+    rng = np.random.default_rng(0)
+    W = [[orc.normal(E * D * F, 0, 40 + 3 * l + j, 0.02) for j in range(3)] for l in range(layers)]
+    x = orc.normal(T * D, 0, 50)
+    plans, hits = [], 0
+    for l in range(layers):
+        logits = rng.standard_normal((T, E))
+        top = np.argsort(-logits, axis=1)[:, :topk]
+        plan = []
+        for e in np.unique(top):
+            toks = np.concatenate([np.nonzero(top[:, k] == e)[0] for k in range(topk)])
+            plan.append((int(e), np.ascontiguousarray(x.reshape(T, D)[toks].reshape(-1)), len(toks)))
+        hits += len(plan)
+        plans.append(plan)
+    grouped = kind == "reference"
+
+    def layer(l):
+        bufs = []
+        for e, xe, m in plans[l]:
+            gp = np.zeros(m * F, np.float32); up = np.zeros(m * F, np.float32)
+            w1 = W[l][0][e * D * F:(e + 1) * D * F]; w3 = W[l][1][e * D * F:(e + 1) * D * F]
+            if grouped:
+                lib.gemm_nn(xe, w1, gp, m, D, F, grouped=True); lib.gemm_nn(xe, w3, up, m, D, F, grouped=True)
+            else:
+                lib.gemm_nn(xe, w1, gp, m, D, F); lib.gemm_nn(xe, w3, up, m, D, F)
+            bufs.append((e, m, gp, up))
+        if grouped:
+            lib.mg_flush()
+        outs = []
+        for e, m, gp, up in bufs:
+            ap = np.zeros(m * F, np.float32); yp = np.zeros(m * D, np.float32)
+            lib.swiglu(gp, up, ap)
+            w2 = W[l][2][e * D * F:(e + 1) * D * F]
+            if grouped:
+                lib.gemm_nn(ap, w2, yp, m, F, D, grouped=True)
+            else:
+                lib.gemm_nn(ap, w2, yp, m, F, D)
+            outs.append(yp)
+        if grouped:
+            lib.mg_flush()
+        return outs
+
+    layer(0)
+    reps, t_used = 0, 0.0
+    while t_used < 10.0 and reps < 100000:
+        t0 = time.perf_counter()
+        for l in range(layers):
+            layer(l)
+        t_used += time.perf_counter() - t0
+        reps += 1
+    gbs = hits * per_expert * reps / t_used / 1e9
+    return {"value": gbs, "unit": "GB/s", "cores": threads, "cpu": cpu_model(), "kind": kind,
+            "sample": "expert part of moe_forward, T=%d top-%d over %d layers (E=%d D=%d F=%d, %d expert hits), %d repetitions; bytes counted as "
+                      "packed digits + scales of the experts hit (the GPU leg's unit; the CPU path reads the fp32 view, 8x that); %s"
+                      % (T, topk, layers, E, D, F, hits, reps, "cudalm.cu mg_ab + mg_flush -> cpu_rt.h small-R SGEMM, cpu_kern.h swiglu" if grouped else "oracle/qlm_oracle.c"),
+            "ms_per_layer": t_used / reps / layers * 1e3}
 
 
 # HBM bytes from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the 1 GiB copy calibration); the runs,
@@ -619,10 +700,14 @@ def main():
     if not args.no_cpu:
         if "adamw" in results:
             results["adamw"]["cpu_baseline"] = cpu_adamw(args)
+        if "decode" in results:
+            results["decode"]["cpu_baseline"] = cpu_decode(args)
         if "train" in results:
             line["cpu_baseline"] = cpu_gemm(args)
         elif "adamw" in results:
             line["cpu_baseline"] = results["adamw"]["cpu_baseline"]
+        elif "decode" in results:
+            line["cpu_baseline"] = results["decode"]["cpu_baseline"]
     print(json.dumps(line))
 
 

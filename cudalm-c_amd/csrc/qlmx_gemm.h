@@ -196,14 +196,18 @@ struct UnitUpload { DevProb *hprob; DevUnit *hunit; const DevProb *dprob; const 
 int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot);                         /* tables to fill (pinned, read by the kernel); waits for the slot's last user */
 int qlmx_unit_done(int slot, hipStream_t stream);                                  /* after the kernel launch */
 int qlmx_chain_reserve(int nflags, int *first, unsigned *epoch);                   /* flags for one launch */
+/* one-shot switches of the time-out tests (qlmx_test_force_wait_timeout): true once after being armed */
+bool qlmx_test_take_forced_timeout(int which);
 
 /* chain hand-over; every thread of the workgroup calls both */
-__device__ __forceinline__ void qx_chain_wait(int *flags, int flag, unsigned epoch, int seq, unsigned *status){
+/* `limit` polls at most (QX_CHAIN_SPINS in production; the time-out test passes 1 together with an epoch
+ * nobody publishes, so that every wait gives up at once and the kernel still runs to its end) */
+__device__ __forceinline__ void qx_chain_wait(int *flags, int flag, unsigned epoch, int seq, unsigned *status, int limit){
     if(threadIdx.x == 0){
         const int want = (int)((epoch << 4) | (unsigned)seq);
         int spins = 0;
-        while(__hip_atomic_load(flags + flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want && ++spins < QX_CHAIN_SPINS) __builtin_amdgcn_s_sleep(16);
-        if(spins >= QX_CHAIN_SPINS) __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        while(__hip_atomic_load(flags + flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want && ++spins < limit) __builtin_amdgcn_s_sleep(16);
+        if(spins >= limit) __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     __syncthreads();
 }

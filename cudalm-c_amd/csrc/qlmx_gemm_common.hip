@@ -154,7 +154,11 @@ int qlmx_upload_done(int slot, hipStream_t stream){ return guard_launched(g_ring
  * problem table and a unit table; chain flags handed out round the ring of a fixed array
  * (a launch's flags carry its epoch, so nothing is ever cleared). ---- */
 #define UNIT_SLOTS 32
-#define CHAIN_FLAGS (1 << 18)
+/* A launch takes at most CHAIN_MAX_PER_LAUNCH flags from a cursor that wraps; a unit-ring slot is only handed out
+ * again after its launch has finished, so at most UNIT_SLOTS launches are in flight and the array holds all of
+ * their flags plus the stretch a wrap may skip: flags of two live launches never overlap. */
+#define CHAIN_MAX_PER_LAUNCH (1 << 16)
+#define CHAIN_FLAGS ((UNIT_SLOTS + 1) * CHAIN_MAX_PER_LAUNCH)
 static char      *g_unit_h = nullptr;
 static RingGuard  g_unit_guard = {UNIT_SLOTS, 8, 0, {}};
 static int       *g_chain_flags = nullptr;
@@ -179,6 +183,7 @@ static int unit_init(void){
 int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot_out){
     int rc = unit_init(); if(rc) return rc;
     if(*(volatile unsigned *)g_chain_status){
+        *g_chain_status = 0;                      /* reported once, by this call */
         qlmx_set_error("grouped gemm: an earlier launch gave up waiting for a partial sum of a split contraction; its output is incomplete");
         return QLMX_E_HIP;
     }
@@ -195,10 +200,25 @@ int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot_out){
 int qlmx_unit_done(int slot, hipStream_t stream){ return guard_launched(g_unit_guard, slot, stream); }
 
 int qlmx_chain_reserve(int nflags, int *first, unsigned *epoch){
-    QLMX_REQUIRE(nflags <= CHAIN_FLAGS / 4, "grouped gemm: %d chained tiles in one launch", nflags);
+    QLMX_REQUIRE(nflags <= CHAIN_MAX_PER_LAUNCH, "grouped gemm: %d chained tiles in one launch", nflags);
     if(g_chain_cursor + nflags > CHAIN_FLAGS) g_chain_cursor = 0;
     *first = g_chain_cursor; g_chain_cursor += nflags;
     g_chain_epoch = (g_chain_epoch + 1) & 0x0FFFFFFFu;
     *epoch = g_chain_epoch;
+    return QLMX_OK;
+}
+
+/* ---- time-out tests: the host arms a one-shot switch; the next launch of that kind then waits, for a single
+ * poll, for a hand-over tag that nobody publishes, so every one of its waits gives up, every workgroup still runs to
+ * its end, the output is wrong and the status word is set -- exactly what a real time-out leaves behind. ---- */
+static bool g_forced[3] = {false, false, false};
+bool qlmx_test_take_forced_timeout(int which){
+    if(which < 1 || which > 2 || !g_forced[which]) return false;
+    g_forced[which] = false;
+    return true;
+}
+extern "C" int qlmx_test_force_wait_timeout(int which){
+    QLMX_REQUIRE(which == 1 || which == 2, "qlmx_test_force_wait_timeout: 1 = decode layer, 2 = split weight-gradient contraction");
+    g_forced[which] = true;
     return QLMX_OK;
 }

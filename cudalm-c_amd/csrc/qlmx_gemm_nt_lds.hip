@@ -36,6 +36,7 @@ typedef float  f32x16 __attribute__((ext_vector_type(16)));
 #define NT3_STAGE_BYTES (NT3_A_BYTES + NT3_B_BYTES)
 
 struct Nt3Args { const DevProb *pr; const DevUnit *units; int *flags; unsigned *status; unsigned epoch;
+                 unsigned wait_epoch; int wait_limit;      /* what a slice waits for (= epoch) and for how many polls */
                  int nprob, ntiles, tiles_n, rows_p; int K, N; const void *zeros; };
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -219,7 +220,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
         return;
     }
     /* one slice of a split contraction: add to what the slices before have left, past the caches */
-    if(seq > 0) qx_chain_wait(a.flags, flag, a.epoch, seq, a.status);
+    if(seq > 0) qx_chain_wait(a.flags, flag, a.wait_epoch, seq, a.status, a.wait_limit);
     qx_store_tiles<4, 2, true>(acc, c, row, i0 + wi, a.K, (size_t)a.N, seq > 0 || P.beta != 0.0f);
     if(seq + 1 < nseq) qx_chain_publish(a.flags, flag, a.epoch, seq);
 }
@@ -315,6 +316,8 @@ int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N
                 a.nprob = n; a.ntiles = grid; a.tiles_n = N / NT3_BN; a.rows_p = 1; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
                 int first = 0; a.epoch = 0;
                 if(nflags){ rc = qlmx_chain_reserve(nflags, &first, &a.epoch); if(rc) return rc; }
+                a.wait_epoch = a.epoch; a.wait_limit = QX_CHAIN_SPINS;
+                if(nflags && qlmx_test_take_forced_timeout(2)){ a.wait_epoch = a.epoch ^ 0x00A5A5A5u; a.wait_limit = 1; }
                 for(int p = 0; p < n; p++) uu.hprob[p].flag0 += first;
                 hipLaunchKernelGGL(k_gemm_nt_lds, dim3(grid), dim3(256), 0, st, a);
                 QLMX_LAUNCH_CHECK("grouped gemm nt (scheduled) launch");
@@ -325,7 +328,7 @@ int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N
     ProbUpload up; int slot;
     int rc = qlmx_upload_problems(probs, nprob, GEMM_NT, K, N, NT3_BM, NT3_BN, st, &up, &slot); if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;
-    Nt3Args a; a.units = nullptr; a.flags = nullptr; a.status = nullptr; a.epoch = 0; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.tiles_n = N / NT3_BN; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
+    Nt3Args a; a.units = nullptr; a.flags = nullptr; a.status = nullptr; a.epoch = 0; a.wait_epoch = 0; a.wait_limit = 0; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.tiles_n = N / NT3_BN; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
     a.rows_p = up.ntiles / (a.tiles_n * up.nprob);
     int grid;
     if(a.rows_p & 7) grid = 8 * a.tiles_n * a.rows_p * ((up.nprob + 7) / 8);

@@ -322,6 +322,7 @@ struct DfArgs {
     int T, K, E, D, F;
     int R1, S1, NC1, R2, S2, NC2;
     u64 *part1, *part2; unsigned epoch; unsigned *status;
+    unsigned wait_xor; int spin_limit;   /* waits look for epoch ^ wait_xor (0) for at most spin_limit polls; the time-out test changes both */
     unsigned *ctl;            /* device words: [0] tag of the last finished call, [1] workgroups of this call that are done */
 };
 
@@ -341,7 +342,7 @@ __device__ __forceinline__ void df_st(u64 *p, float v, unsigned epoch){
  * looked at. */
 #define DF_SLICE_STEP 4
 template<int NSRC>
-__device__ __forceinline__ void df_sum_wait(const u64 *const (&src)[NSRC], size_t stride, int S, unsigned epoch,
+__device__ __forceinline__ void df_sum_wait(const u64 *const (&src)[NSRC], size_t stride, int S, unsigned epoch, int limit,
                                             volatile int *giveup, unsigned *status, float (&v)[NSRC]){
     int spins = 0;
     for(;;){
@@ -364,7 +365,7 @@ __device__ __forceinline__ void df_sum_wait(const u64 *const (&src)[NSRC], size_
                 }
         }
         if(ok) break;
-        if(++spins > DF_SPIN_LIMIT || *giveup){ *(volatile unsigned *)status = 1u; *giveup = 1; break; }
+        if(++spins > limit || *giveup){ *(volatile unsigned *)status = 1u; *giveup = 1; break; }
         __builtin_amdgcn_s_sleep(2);
     }
 }
@@ -374,13 +375,13 @@ __device__ __forceinline__ void df_sum_wait(const u64 *const (&src)[NSRC], size_
  * other, so the full read that follows rarely has to repeat, and while a producer is still busy only
  * n threads per workgroup poll instead of all of them. */
 template<class ADDR>
-__device__ __forceinline__ void df_wait_first(int n, unsigned epoch, volatile int *giveup, unsigned *status, ADDR addr){
+__device__ __forceinline__ void df_wait_first(int n, unsigned epoch, int limit, volatile int *giveup, unsigned *status, ADDR addr){
     for(int i = threadIdx.x; i < n; i += DF_THREADS){
         const u64 *p = addr(i);
         if(!p) continue;
         int spins = 0;
         while((unsigned)(__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) != epoch){
-            if(++spins > DF_SPIN_LIMIT || *giveup){ *(volatile unsigned *)status = 1u; *giveup = 1; break; }
+            if(++spins > limit || *giveup){ *(volatile unsigned *)status = 1u; *giveup = 1; break; }
             __builtin_amdgcn_s_sleep(4);
         }
     }
@@ -647,7 +648,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
             } else {
                 const u64 *p1 = a.part1 + (((size_t)prob * 2) * a.S1 * DF_MB) * a.F + k0;
                 const size_t sstride = (size_t)DF_MB * a.F;
-                df_wait_first(2 * a.S1, a.epoch, &giveup, a.status, [=](int i){ return p1 + (size_t)i * sstride; });
+                df_wait_first(2 * a.S1, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, [=](int i){ return p1 + (size_t)i * sstride; });
                 if(tid < rows){
                     float sc[DF_NG];
 #pragma unroll
@@ -660,7 +661,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
                             /* h = silu(gate) * up (k_swiglu, cudalm.cu:2430-2432), both summed over the K slices in order */
                             const u64 *const src[2] = { p1 + (size_t)m * a.F + tid, p1 + (size_t)a.S1 * sstride + (size_t)m * a.F + tid };
                             float gu[2];
-                            df_sum_wait<2>(src, sstride, a.S1, a.epoch, &giveup, a.status, gu);
+                            df_sum_wait<2>(src, sstride, a.S1, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, gu);
                             hv[m] = (gu[0] / (1.0f + expf(-gu[0]))) * gu[1];
                         }
                     }
@@ -686,7 +687,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
             const int col = chunk * DF_CW + tid;
             {
                 const int S2 = a.S2, T = a.T, Dd = a.D; const int *pp = mt.pair_prob, *pm = mt.pair_m; const u64 *p2 = a.part2;
-                df_wait_first(a.K * S2, a.epoch, &giveup, a.status, [=](int i) -> const u64 * {
+                df_wait_first(a.K * S2, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, [=](int i) -> const u64 * {
                     const int j = (i / S2) * T + n, prob = pp[j];
                     if(prob < 0) return nullptr;
                     return p2 + (((size_t)prob * S2 + i % S2) * DF_MB + pm[j]) * Dd + chunk * DF_CW; });
@@ -698,7 +699,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
                     if(prob < 0) continue;
                     const u64 *const src[1] = { a.part2 + (((size_t)prob * a.S2) * DF_MB + mt.pair_m[j]) * a.D + col };
                     float y[1];
-                    df_sum_wait<1>(src, (size_t)DF_MB * a.D, a.S2, a.epoch, &giveup, a.status, y);
+                    df_sum_wait<1>(src, (size_t)DF_MB * a.D, a.S2, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, y);
                     o = o + a.gate[j] * y[0];
                 }
                 a.out[(size_t)n * a.D + col] = o;
@@ -836,6 +837,8 @@ static int df_forward(bool fixed, const char *who, const float *x, const int *as
         a.ctl = dv.grown.ctl; a.part1 = dv.grown.part[0]; a.part2 = dv.grown.part[1];
     }
     a.status = dv.status; a.epoch = 0;
+    a.wait_xor = 0; a.spin_limit = DF_SPIN_LIMIT;
+    if(qlmx_test_take_forced_timeout(1)){ a.wait_xor = 0x40000000u; a.spin_limit = 0; }
     const long long most = (long long)2 * npair * a.NC1 * a.S1;
     const int grid = (int)std::min<long long>(dv.grid, (most + 7) & ~7LL);
     hipLaunchKernelGGL(k_decode_fused, dim3(grid), dim3(DF_THREADS), 0, st, a);

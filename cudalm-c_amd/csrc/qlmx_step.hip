@@ -343,23 +343,53 @@ extern "C" int qlmx_step_touched(float *P, const float *Gc, signed char *d, sign
 /* ---- gradient-norm clipping around the step (cudalm.cu:2794-2820, CPU twins cpu_kern.h:533-546) ----
  * k_sqsum: 64 partial sums of squares; partial c covers G[n*c/64 .. n*(c+1)/64), is accumulated in
  * double and rounded to float once (the CPU path's definition; the reference's GPU kernel sums
- * strided in fp32 and differs from its own CPU kernel in the last bits). Here a workgroup sums its
- * chunk in double, lanes strided, then a fixed tree: the order of the double additions is not the
- * CPU's, which can move the double sum by a few units in its last place -- far below half a float
- * ulp except on an exact tie. */
+ * strided in fp32 and differs from its own CPU kernel in the last bits). The 64 partials are the
+ * contract, 64 workgroups are not: each chunk is cut into SQ_W pieces, one workgroup each (1024
+ * workgroups for the 256 CUs), which sum in double -- lanes strided, then a fixed tree -- and leave
+ * their sum in a device array; the workgroup that arrives last at a chunk (a counter) adds the SQ_W
+ * sums in piece order, so the result does not depend on arrival order. The order of the double
+ * additions is not the CPU's, which can move the double sum by a few units in its last place -- far
+ * below half a float ulp except on an exact tie. The array and the counters are static device
+ * memory (the last workgroup resets its counter): calls that overlap on different streams would
+ * mix their pieces and are not supported. */
+#define SQ_W 16
+static __device__ double   g_sq_piece[64 * SQ_W];
+static __device__ unsigned g_sq_count[64];
 __global__ void __launch_bounds__(256) k_qlmx_sqsum(const float *G, unsigned long long n, float *part){
     __shared__ double red[256];
-    const unsigned long long c = blockIdx.x, nb = gridDim.x;
-    const unsigned long long i0 = n * c / nb, i1 = n * (c + 1) / nb;
+    const unsigned c = blockIdx.x / SQ_W, w = blockIdx.x % SQ_W;
+    const unsigned long long c0 = n * c / 64, c1 = n * (c + 1) / 64, len = c1 - c0;
+    const unsigned long long i0 = c0 + len * w / SQ_W, i1 = c0 + len * (w + 1) / SQ_W;
     double s = 0.0;
-    for(unsigned long long i = i0 + threadIdx.x; i < i1; i += 256){ const double g = (double)G[i]; s += g * g; }
+    /* 16-byte loads over the aligned middle, single elements at both ends */
+    unsigned long long a0 = (i0 + 3) & ~3ULL; if(a0 > i1) a0 = i1;
+    const unsigned long long a1 = a0 + ((i1 - a0) & ~3ULL);
+    for(unsigned long long i = i0 + threadIdx.x; i < a0; i += 256){ const double g = (double)G[i]; s += g * g; }
+    if((((uintptr_t)G) & 15) == 0){
+        for(unsigned long long i = a0 + 4ULL * threadIdx.x; i < a1; i += 1024){
+            const float4 v = *(const float4 *)(G + i);
+            s += (double)v.x * (double)v.x; s += (double)v.y * (double)v.y; s += (double)v.z * (double)v.z; s += (double)v.w * (double)v.w;
+        }
+    } else {
+        for(unsigned long long i = a0 + threadIdx.x; i < a1; i += 256){ const double g = (double)G[i]; s += g * g; }
+    }
+    for(unsigned long long i = a1 + threadIdx.x; i < i1; i += 256){ const double g = (double)G[i]; s += g * g; }
     red[threadIdx.x] = s;
     __syncthreads();
     for(int o = 128; o > 0; o >>= 1){
         if((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
         __syncthreads();
     }
-    if(threadIdx.x == 0) part[c] = (float)red[0];
+    if(threadIdx.x == 0){
+        __hip_atomic_store(&g_sq_piece[c * SQ_W + w], red[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned before = __hip_atomic_fetch_add(&g_sq_count[c], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if(before == SQ_W - 1){
+            double t = 0.0;
+            for(int k = 0; k < SQ_W; k++) t += __hip_atomic_load(&g_sq_piece[c * SQ_W + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            part[c] = (float)t;
+            __hip_atomic_store(&g_sq_count[c], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
 }
 
 /* k_gnorm (cudalm.cu:2811-2816 = cpu_kern.h:541-546): part = G's 64 partials followed by nside more
@@ -378,7 +408,7 @@ __global__ void k_qlmx_gnorm(const float *part, int nside, int clip_side, float 
 extern "C" int qlmx_sqsum(const float *G, unsigned long long n, float *part64, void *stream){
     int rc = qlmx_check_ready(); if(rc) return rc;
     QLMX_REQUIRE(G && part64, "qlmx_sqsum: NULL buffer");
-    hipLaunchKernelGGL(k_qlmx_sqsum, dim3(64), dim3(256), 0, (hipStream_t)stream, G, n, part64);
+    hipLaunchKernelGGL(k_qlmx_sqsum, dim3(64 * SQ_W), dim3(256), 0, (hipStream_t)stream, G, n, part64);
     QLMX_LAUNCH_CHECK("qlmx_sqsum launch");
     return QLMX_OK;
 }

@@ -1,89 +1,147 @@
 /* qlm_host.cpp -- see qlm_host.h. Host logic only; every device operation goes through libqlmx. */
 #include "qlm_host.h"
+#include <fcntl.h>
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <sys/stat.h>
+#include <unistd.h>
+#include <algorithm>
+#include <functional>
+#include <numeric>
+#include <string>
 #include <vector>
+
+typedef unsigned long long u64;
 
 static void ck(int rc, const char *what){
     if(rc != QLMX_OK){ fprintf(stderr, "HIP error: %s at %s\n", qlmx_last_error(), what); exit(1); }
 }
 void *dmalloc(size_t bytes){ void *p = NULL; ck(qlmx_malloc(&p, bytes), "hipMalloc"); return p; }
 
-/* qlm.cuh:448-455 */
-void qlm_add_span(Qlm *q, unsigned long long pof, unsigned long long n){
-    if(q->nspan >= QLM_MAXSPAN) return;
-    QSpanD *sp = &q->spanH[q->nspan];
-    sp->pof = pof; sp->gof = pof; sp->qi0 = q->nq; sp->n = n;
-    sp->gi0 = (int)q->ngrp; sp->ngrp = (int)((n + q->group - 1) / q->group);
-    sp->sref = 1.0f;
-    q->nq += n; q->ngrp += sp->ngrp; q->nspan++;
+/* ---------------------------------------------------------------------------------------------
+ * Configuration. The reference reads its switches from the environment inside qlm_gpu_init
+ * (qlm.cuh:459-474); here they are parsed once into a value that init applies. The rules are the
+ * reference's: bits -> largest digit {<=2: 1, 3: 3, 4: 7, else 127}; group clamped to [32, 256];
+ * "abs" selects the absolute LR mode; "qlion" the sign optimizer; the rail-fraction target defaults
+ * to 0.60 for ternary digits and 1.5 elements per group otherwise, with a +-50 % dead band.
+ * ------------------------------------------------------------------------------------------- */
+namespace {
+struct QlmKnobs { int dmax, group, lrmode, servo_every, adam, v4; float fstar; };
+
+const char *env_or(const char *name, const char *fallback){ const char *v = getenv(name); return v ? v : fallback; }
+
+QlmKnobs knobs_from_env(){
+    QlmKnobs k;
+    const int bits = atoi(env_or("QLM_BITS", "4"));
+    k.dmax = bits <= 2 ? 1 : bits == 3 ? 3 : bits == 4 ? 7 : 127;
+    k.group = std::min(256, std::max(32, atoi(env_or("QLM_GROUP", "128"))));
+    k.lrmode = strcmp(env_or("QLM_LRMODE", "rel"), "abs") == 0;
+    k.servo_every = atoi(env_or("QLM_SERVO", "100"));
+    k.adam = strcmp(env_or("QLM_OPT", ""), "qlion") != 0;
+    k.v4 = atoi(env_or("QLM_V4", "0")) != 0;
+    const char *fs = getenv("QLM_FSTAR");
+    k.fstar = fs ? (float)atof(fs) : (k.dmax == 1 ? 0.60f : 1.5f / (float)k.group);
+    return k;
 }
 
-/* qlm.cuh:458-541: environment, span table, float gaps, allocation, encode, frozen reference scales,
- * first render. */
-void qlm_gpu_init(Qlm *q, const QlmSpanDesc *spans, int nspan, float *P, size_t np){
-    memset(q, 0, sizeof(*q));
-    const char *e;
-    int bits = (e = getenv("QLM_BITS")) ? atoi(e) : 4;
-    q->dmax  = bits <= 2 ? 1 : bits == 3 ? 3 : bits == 4 ? 7 : 127;
-    q->group = (e = getenv("QLM_GROUP")) ? atoi(e) : 128;
-    if(q->group < 32) q->group = 32;
-    if(q->group > 256) q->group = 256;
-    q->lrmode = (e = getenv("QLM_LRMODE")) ? (!strcmp(e, "abs") ? 1 : 0) : 0;
-    q->servo_every = (e = getenv("QLM_SERVO")) ? atoi(e) : 100;
-    q->adam = 1;
-    q->v4 = (e = getenv("QLM_V4")) ? (atoi(e) != 0) : 0;
-    if((e = getenv("QLM_OPT")) && !strcmp(e, "qlion")) q->adam = 0;
-    q->fstar = (e = getenv("QLM_FSTAR")) ? (float)atof(e) : (q->dmax == 1 ? 0.60f : 1.5f / (float)q->group);
-    q->f_hi = q->fstar * 1.5f; q->f_lo = q->fstar * 0.5f;
-    q->np = np;
-    q->render_p = P != NULL;
+/* Every device array a Qlm owns, with its size: one table drives allocation, clearing and release. */
+struct OwnedArray { void **slot; size_t bytes; bool cleared; };
+std::vector<OwnedArray> owned_arrays(Qlm *q){
+    const size_t nq = q->nq, ng4 = (size_t)q->ngrp * 4;
+    std::vector<OwnedArray> t = {
+        {(void **)&q->d,  (size_t)qlmx_qd_bytes(q->nq, q->packed), false},
+        {(void **)&q->r,  nq, false},
+        {(void **)&q->m8, nq, true},
+        {(void **)&q->s,  ng4, false},
+        {(void **)&q->m8s, ng4, true},
+        {(void **)&q->statD, 4 * sizeof(long long), true},
+        {(void **)&q->spanD, (size_t)q->nspan * sizeof(QSpanD), false},
+    };
+    if(q->adam){ t.push_back({(void **)&q->v8, nq, true}); t.push_back({(void **)&q->v8s, ng4, true}); }
+    return t;
+}
 
+void upload_spans(Qlm *q, const char *what){
+    ck(qlmx_memcpy_h2d(q->spanD, q->spanH, (size_t)q->nspan * sizeof(QSpanD)), what);
+}
+
+/* The parameters between and around the quantized spans stay in floating point; the reference keeps
+ * their optimizer moments compact, so each gap gets its offset in P, its length and its offset in the
+ * compact arrays (qlm.cuh:492-501). Spans are in ascending order of pof. */
+void index_float_gaps(Qlm *q){
+    q->nfs = 0; q->nfloat = 0;
+    auto add = [&](u64 from, u64 to){
+        if(to <= from) return;
+        q->fs_off[q->nfs] = from; q->fs_n[q->nfs] = to - from; q->fs_cs[q->nfs] = q->nfloat;
+        q->nfloat += to - from; q->nfs++;
+    };
+    u64 edge = 0;
+    for(int i = 0; i < q->nspan; i++){ add(edge, q->spanH[i].pof); edge = q->spanH[i].pof + q->spanH[i].n; }
+    add(edge, q->np);
+}
+
+/* sref of every span = mean of its group scales, summed in double in group order (qlm.cuh:527-536;
+ * the order is part of the contract: the relative-LR step divides by this float) */
+void freeze_reference_scales(Qlm *q){
+    std::vector<float> scales(q->ngrp);
+    ck(qlmx_memcpy_d2h(scales.data(), q->s, (size_t)q->ngrp * 4), "qlm s d2h");
+    for(int i = 0; i < q->nspan; i++){
+        QSpanD &sp = q->spanH[i];
+        const float *first = scales.data() + sp.gi0;
+        sp.sref = (float)(std::accumulate(first, first + sp.ngrp, 0.0) / (double)sp.ngrp);
+    }
+    upload_spans(q, "qlm span h2d (sref)");
+}
+}  // namespace
+
+/* qlm.cuh:448-455: a span is appended behind everything registered so far */
+void qlm_add_span(Qlm *q, unsigned long long pof, unsigned long long n){
+    if(q->nspan >= QLM_MAXSPAN) return;
+    QSpanD sp;
+    sp.pof = sp.gof = pof; sp.n = n; sp.qi0 = q->nq;
+    sp.gi0 = (int)q->ngrp; sp.ngrp = (int)((n + (u64)q->group - 1) / (u64)q->group);
+    sp.sref = 1.0f;
+    q->spanH[q->nspan++] = sp;
+    q->nq += n; q->ngrp += (u64)sp.ngrp;
+}
+
+/* qlm.cuh:458-541: switches, span table, float gaps, device state, and -- when the caller still holds an
+ * fp32 view P -- encode, frozen reference scales and the first render. */
+void qlm_gpu_init(Qlm *q, const QlmSpanDesc *spans, int nspan, float *P, size_t np){
+    *q = Qlm();
+    const QlmKnobs k = knobs_from_env();
+    q->dmax = k.dmax; q->group = k.group; q->lrmode = k.lrmode; q->servo_every = k.servo_every;
+    q->adam = k.adam; q->v4 = k.v4; q->packed = k.dmax <= 7;
+    q->fstar = k.fstar; q->f_hi = 1.5f * k.fstar; q->f_lo = 0.5f * k.fstar;
+    q->np = np; q->render_p = P != NULL;
     q->spanH = (QSpanD *)calloc(QLM_MAXSPAN, sizeof(QSpanD));
     for(int i = 0; i < nspan; i++) qlm_add_span(q, spans[i].pof, spans[i].n);
-    {   /* float spans = the gaps between quantized spans */
-        unsigned long long cur = 0;
-        for(int i = 0; i < q->nspan; i++){
-            if(q->spanH[i].pof > cur){ q->fs_off[q->nfs] = cur; q->fs_n[q->nfs] = q->spanH[i].pof - cur; q->nfs++; }
-            cur = q->spanH[i].pof + q->spanH[i].n;
-        }
-        if(cur < np){ q->fs_off[q->nfs] = cur; q->fs_n[q->nfs] = np - cur; q->nfs++; }
-        unsigned long long acc = 0;
-        for(int i = 0; i < q->nfs; i++){ q->fs_cs[i] = acc; acc += q->fs_n[i]; }
-        q->nfloat = acc;
+    index_float_gaps(q);
+    for(const OwnedArray &a : owned_arrays(q)){
+        *a.slot = dmalloc(a.bytes);
+        if(a.cleared) ck(qlmx_memset(*a.slot, 0, a.bytes, NULL), "qlm state clear");
     }
-    q->packed = (q->dmax <= 7);
-    q->d  = (signed char *)dmalloc((size_t)qlmx_qd_bytes(q->nq, q->packed));
-    q->r  = (signed char *)dmalloc(q->nq);
-    q->m8 = (signed char *)dmalloc(q->nq);
-    q->v8 = q->adam ? (unsigned char *)dmalloc(q->nq) : NULL;
-    ck(qlmx_memset(q->m8, 0, q->nq, NULL), "qlm m8 zero");
-    if(q->adam) ck(qlmx_memset(q->v8, 0, q->nq, NULL), "qlm v8 zero");
-    q->s   = (float *)dmalloc(q->ngrp * 4);
-    q->m8s = (float *)dmalloc(q->ngrp * 4);
-    q->v8s = q->adam ? (float *)dmalloc(q->ngrp * 4) : NULL;
-    ck(qlmx_memset(q->m8s, 0, q->ngrp * 4, NULL), "qlm m8s zero");
-    if(q->adam) ck(qlmx_memset(q->v8s, 0, q->ngrp * 4, NULL), "qlm v8s zero");
-    q->statD = (long long *)dmalloc(4 * 8);
-    ck(qlmx_memset(q->statD, 0, 32, NULL), "qlm stat zero");
-    q->spanD = (QSpanD *)dmalloc((size_t)q->nspan * sizeof(QSpanD));
-    ck(qlmx_memcpy_h2d(q->spanD, q->spanH, (size_t)q->nspan * sizeof(QSpanD)), "qlm span h2d");
+    upload_spans(q, "qlm span h2d");
     if(P){
         ck(qlmx_encode(P, q->d, q->r, q->s, q->spanD, q->nspan, q->group, q->dmax, q->packed, (int)q->ngrp, NULL), "qlm encode");
-        /* freeze each span's reference scale: mean of its group scales, in double (qlm.cuh:527-536) */
-        std::vector<float> sh(q->ngrp);
-        ck(qlmx_memcpy_d2h(sh.data(), q->s, q->ngrp * 4), "qlm s d2h");
-        for(int i = 0; i < q->nspan; i++){
-            double acc = 0;
-            for(int g = 0; g < q->spanH[i].ngrp; g++) acc += sh[q->spanH[i].gi0 + g];
-            q->spanH[i].sref = (float)(acc / (double)q->spanH[i].ngrp);
-        }
-        ck(qlmx_memcpy_h2d(q->spanD, q->spanH, (size_t)q->nspan * sizeof(QSpanD)), "qlm span h2d 2");
-        ck(qlmx_render(P, q->d, q->s, q->spanD, q->nspan, q->group, q->packed, 0, (int)q->ngrp, NULL), "qlm render");
+        freeze_reference_scales(q);
+        qlm_gpu_render(q, P);
     }
     q->on = 1;
+}
+
+void qlm_free(Qlm *q){
+    for(const OwnedArray &a : owned_arrays(q)) if(*a.slot) qlmx_free(*a.slot);
+    free(q->spanH);
+    *q = Qlm();
+}
+
+/* first group and number of groups of spans [span0, span0 + nspans) */
+static void group_range(const Qlm *q, int span0, int nspans, int *gi0, int *ng){
+    *gi0 = q->spanH[span0].gi0; *ng = 0;
+    for(int i = span0; i < span0 + nspans; i++) *ng += q->spanH[i].ngrp;
 }
 
 void qlm_gpu_render(Qlm *q, float *P){
@@ -91,8 +149,7 @@ void qlm_gpu_render(Qlm *q, float *P){
 }
 /* qlm.cuh:586-591 generalised: render the groups of spans [span0, span0+nspans) */
 void qlm_render_spans(Qlm *q, float *P, int span0, int nspans){
-    int gi0 = q->spanH[span0].gi0, ng = 0;
-    for(int i = span0; i < span0 + nspans; i++) ng += q->spanH[i].ngrp;
+    int gi0, ng; group_range(q, span0, nspans, &gi0, &ng);
     ck(qlmx_render(P, q->d, q->s, q->spanD, q->nspan, q->group, q->packed, gi0, ng, NULL), "qlm render layer");
 }
 
@@ -104,20 +161,25 @@ void qlm_step_launch(float *P, const float *G, signed char *d, signed char *r, f
                      float lr, float b1, float b2, float wd, float gscale, const float *gsp,
                      float inv_bc1, float inv_sqrt_bc2, int lrmode,
                      unsigned long long t, int adam, long long *stat, int packed, int gi_base, int ng){
-    static int v4 = -1;
-    if(v4 < 0){ const char *e = getenv("QLM_V4"); v4 = e && atoi(e); }
+    static const int v4 = knobs_from_env().v4;
     ck(qlmx_step(P, G, d, r, s, m8, m8s, v8, v8s, sp, nspan, group, dmax, lr, b1, b2, wd, gscale, gsp,
                  inv_bc1, inv_sqrt_bc2, lrmode, t, adam, stat, packed, gi_base, ng, v4, NULL), "qlm step");
 }
 
-/* cudalm.cu:6082-6103 without the float spans' AdamW */
+/* One step over groups [gi0, gi0 + ng) of q with the bias corrections already inverted */
+static void step_groups(Qlm *q, float *P, const float *G, int gi0, int ng, float lr, float b1, float b2, float wd,
+                        float gscale, const float *gsp, float bc1, float bc2, int t, long long *stat){
+    qlm_step_launch(q->render_p ? P : NULL, G, q->d, q->r, q->s, q->m8, q->m8s, q->v8, q->v8s, q->spanD, q->nspan,
+                    q->group, q->dmax, lr, b1, b2, wd, gscale, gsp, 1.0f / bc1, 1.0f / sqrtf(bc2), q->lrmode,
+                    (unsigned long long)t, q->adam, stat, q->packed, gi0, ng);
+}
+
+/* cudalm.cu:6082-6103 without the float spans' AdamW: the whole-model step, then the scale servo on its period */
 void qlm_gpu_update(Qlm *q, float *P, float *G, float lr, float b1, float b2, float wd,
                     float bc1, float bc2, int t, const float *gs){
-    float inv_bc1 = 1.0f / bc1, inv_sqrt_bc2 = 1.0f / sqrtf(bc2);
-    qlm_step_launch(q->render_p ? P : NULL, G, q->d, q->r, q->s, q->m8, q->m8s, q->v8, q->v8s, q->spanD, q->nspan,
-                    q->group, q->dmax, lr, b1, b2, wd, 1.0f, gs, inv_bc1, inv_sqrt_bc2, q->lrmode,
-                    (unsigned long long)t, q->adam, getenv("CUDALM_QLM_DIAG") ? q->statD : NULL, q->packed, 0, (int)q->ngrp);
-    if(q->servo_every > 0 && (t % q->servo_every) == 0)
+    step_groups(q, P, G, 0, (int)q->ngrp, lr, b1, b2, wd, 1.0f, gs, bc1, bc2, t, getenv("CUDALM_QLM_DIAG") ? q->statD : NULL);
+    const bool servo_due = q->servo_every > 0 && t % q->servo_every == 0;
+    if(servo_due)
         ck(qlmx_servo(q->d, q->r, q->s, q->spanD, q->nspan, q->group, q->dmax, q->f_hi, q->f_lo, q->packed, (int)q->ngrp, NULL), "qlm servo");
 }
 
@@ -125,15 +187,10 @@ void qlm_gpu_update(Qlm *q, float *P, float *G, float lr, float b1, float b2, fl
 void qlm_fused_spans(Qlm *q, float *P, float *G, int span0, int nspans, size_t g0, size_t gn, float *part64,
                      float lr, float wd, int t, float prev_gn){
     const float b1 = 0.9f, b2 = 0.95f;
-    const float bc1 = 1.0f - powf(b1, (float)t), bc2 = 1.0f - powf(b2, (float)t);
-    const float inv_bc1 = 1.0f / bc1, inv_sqrt_bc2 = 1.0f / sqrtf(bc2);
-    const float gscale = prev_gn > 1.0f ? 1.0f / prev_gn : 1.0f;
     ck(qlmx_sqsum(G + g0, (unsigned long long)gn, part64, NULL), "fused sqsum");
-    int gi0 = q->spanH[span0].gi0, ng = 0;
-    for(int i = span0; i < span0 + nspans; i++) ng += q->spanH[i].ngrp;
-    qlm_step_launch(q->render_p ? P : NULL, G, q->d, q->r, q->s, q->m8, q->m8s, q->v8, q->v8s, q->spanD, q->nspan,
-                    q->group, q->dmax, lr, b1, b2, wd, gscale, NULL, inv_bc1, inv_sqrt_bc2, q->lrmode,
-                    (unsigned long long)t, q->adam, NULL, q->packed, gi0, ng);
+    int gi0, ng; group_range(q, span0, nspans, &gi0, &ng);
+    step_groups(q, P, G, gi0, ng, lr, b1, b2, wd, prev_gn > 1.0f ? 1.0f / prev_gn : 1.0f, NULL,
+                1.0f - powf(b1, (float)t), 1.0f - powf(b2, (float)t), t, NULL);
 }
 void qlm_fused_layer(Qlm *q, float *P, float *G, size_t layer_g0, size_t layer_gn, float *gnpart, int l,
                      float lr, float wd, int t, float prev_gn){
@@ -145,9 +202,7 @@ float qlm_fused_tail(const float *gnpart, int L, const float *extra, int nextra)
     std::vector<float> ph(nsl + nex);
     if(nsl) ck(qlmx_memcpy_d2h(ph.data(), gnpart, nsl * 4), "fused sqsum d2h");
     if(nex) ck(qlmx_memcpy_d2h(ph.data() + nsl, extra, nex * 4), "fused tail sqsum d2h");
-    double ss = 0;
-    for(size_t i = 0; i < nsl + nex; i++) ss += ph[i];
-    return (float)sqrt(ss);
+    return (float)sqrt(std::accumulate(ph.begin(), ph.end(), 0.0));
 }
 
 /* qlm.cuh:678-683 */
@@ -156,96 +211,169 @@ double qlm_persist_bytes(const Qlm *q){
          + (double)q->ngrp * 4.0 * (q->adam ? 3.0 : 2.0);
 }
 
-/* ---- .opt.q checkpoint: magic QLMH, int hdr[6] = {dmax, group, adam, nspan, packed, iter},
- * u64 nq, ngrp, nfloat, bf16 Mc, Vc (float spans), packed d, r, m8, [v8], fp32 s, m8s, [v8s],
- * trailer "SREF" + nspan + per-span sref, trailer "PGN1" + previous grad norm (qlm.cuh:702-738).
- * Written to <path>.tmp and renamed, as the reference does. ---- */
-int qlm_save(const Qlm *q, const char *path, int iter, float prev_gn){
-    char tmp[1300]; snprintf(tmp, sizeof tmp, "%s.tmp", path);
-    FILE *f = fopen(tmp, "wb"); if(!f) return 0;
-    int hdr[6] = {q->dmax, q->group, q->adam, q->nspan, q->packed, iter};
-    unsigned long long nq = q->nq, ng = q->ngrp, nf = q->nfloat, nd = qlmx_qd_bytes(nq, q->packed);
-    std::vector<signed char> hd(nd), hr(nq), hm(nq);
-    std::vector<unsigned char> hv(q->adam ? nq : 0);
-    std::vector<float> hs(ng), hms(ng), hvs(q->adam ? ng : 0);
-    std::vector<bf16> hM(nf, 0), hV(nf, 0);
-    if(q->Mc && nf) ck(qlmx_memcpy_d2h(hM.data(), q->Mc, nf * 2), "qlm save Mc");
-    if(q->Vc && nf) ck(qlmx_memcpy_d2h(hV.data(), q->Vc, nf * 2), "qlm save Vc");
-    ck(qlmx_memcpy_d2h(hd.data(), q->d, nd), "qlm save d");
-    ck(qlmx_memcpy_d2h(hr.data(), q->r, nq), "qlm save r");
-    ck(qlmx_memcpy_d2h(hm.data(), q->m8, nq), "qlm save m8");
-    if(q->adam) ck(qlmx_memcpy_d2h(hv.data(), q->v8, nq), "qlm save v8");
-    ck(qlmx_memcpy_d2h(hs.data(), q->s, ng * 4), "qlm save s");
-    ck(qlmx_memcpy_d2h(hms.data(), q->m8s, ng * 4), "qlm save m8s");
-    if(q->adam) ck(qlmx_memcpy_d2h(hvs.data(), q->v8s, ng * 4), "qlm save v8s");
-    int ok = fwrite("QLMH", 1, 4, f) == 4 && fwrite(hdr, 4, 6, f) == 6
-          && fwrite(&nq, 8, 1, f) == 1 && fwrite(&ng, 8, 1, f) == 1 && fwrite(&nf, 8, 1, f) == 1
-          && fwrite(hM.data(), 2, nf, f) == nf && fwrite(hV.data(), 2, nf, f) == nf
-          && fwrite(hd.data(), 1, nd, f) == nd && fwrite(hr.data(), 1, nq, f) == nq
-          && fwrite(hm.data(), 1, nq, f) == nq && (q->adam ? fwrite(hv.data(), 1, nq, f) == nq : 1)
-          && fwrite(hs.data(), 4, ng, f) == ng && fwrite(hms.data(), 4, ng, f) == ng
-          && (q->adam ? fwrite(hvs.data(), 4, ng, f) == ng : 1);
-    if(ok){ int ns = q->nspan; ok = fwrite("SREF", 1, 4, f) == 4 && fwrite(&ns, 4, 1, f) == 1;
-            for(int i = 0; ok && i < ns; i++) ok = fwrite(&q->spanH[i].sref, 4, 1, f) == 1; }
-    if(ok) ok = fwrite("PGN1", 1, 4, f) == 4 && fwrite(&prev_gn, 4, 1, f) == 1;
-    if(fflush(f) != 0) ok = 0;
-    if(fclose(f) != 0) ok = 0;
-    if(!ok){ remove(tmp); return 0; }
-    return rename(tmp, path) == 0;
+/* ---------------------------------------------------------------------------------------------
+ * .opt.q checkpoint (qlm.cuh:702-788). Bytes, in order:
+ *   "QLMH", int32 x6 {dmax, group, adam, nspan, packed, iter}, u64 x3 {nq, ngrp, nfloat},
+ *   bf16 Mc[nfloat], bf16 Vc[nfloat], d, r, m8, [v8 when adam], fp32 s, m8s, [v8s when adam],
+ *   "SREF", int32 nspan, fp32 sref[nspan], "PGN1", fp32 previous gradient norm.
+ * The body is a list of sections; the writer and the reader walk the same list, and each section moves
+ * through one bounce buffer piece by piece (the state of a large model does not fit the host twice).
+ * A section lives in device memory (the Qlm's arrays) or in host memory (the *_host entry points that
+ * tools and CPU tests use); `absent` sections are written as zeros and skipped when read.
+ * ------------------------------------------------------------------------------------------- */
+namespace {
+struct Section { void *ptr; size_t bytes; bool absent; };
+struct OptqBody {
+    int hdr[6]; u64 nq, ngrp, nfloat;
+    std::vector<Section> sections;
+    float *sref; int nspan;
+    bool device;                   /* where the sections' memory is */
+};
+
+OptqBody describe(int dmax, int group, int adam, int nspan, int packed, u64 nq, u64 ngrp, u64 nfloat,
+                  void *Mc, void *Vc, void *d, void *r, void *m8, void *v8, void *s, void *m8s, void *v8s, bool device){
+    OptqBody b;
+    const int hdr[6] = {dmax, group, adam, nspan, packed, 0};
+    memcpy(b.hdr, hdr, sizeof hdr);
+    b.nq = nq; b.ngrp = ngrp; b.nfloat = nfloat; b.nspan = nspan; b.sref = NULL; b.device = device;
+    const size_t nd = (size_t)qlmx_qd_bytes(nq, packed);
+    b.sections = {{Mc, (size_t)nfloat * 2, Mc == NULL}, {Vc, (size_t)nfloat * 2, Vc == NULL},
+                  {d, nd, false}, {r, (size_t)nq, false}, {m8, (size_t)nq, false}};
+    if(adam) b.sections.push_back({v8, (size_t)nq, false});
+    b.sections.push_back({s, (size_t)ngrp * 4, false});
+    b.sections.push_back({m8s, (size_t)ngrp * 4, false});
+    if(adam) b.sections.push_back({v8s, (size_t)ngrp * 4, false});
+    return b;
 }
 
-/* qlm.cuh:740-788: a file of another shape is ignored with a warning and 0 is returned */
-int qlm_load(Qlm *q, const char *path, int *iter, float *prev_gn){
-    FILE *f = fopen(path, "rb"); if(!f) return 0;
-    char mg[4]; int hdr[6]; unsigned long long nq, ng, nf;
-    if(fread(mg, 1, 4, f) != 4 || memcmp(mg, "QLMH", 4)){ fclose(f); return 0; }
-    if(fread(hdr, 4, 6, f) != 6 || fread(&nq, 8, 1, f) != 1 || fread(&ng, 8, 1, f) != 1 || fread(&nf, 8, 1, f) != 1){ fclose(f); return 0; }
-    if(hdr[0] != q->dmax || hdr[1] != q->group || hdr[2] != q->adam || hdr[4] != q->packed
-       || nq != q->nq || ng != q->ngrp || nf > q->nfloat){
-        fprintf(stderr, "[qlm] %s has a different shape (bits/group/opt) -- ignoring\n", path);
-        fclose(f); return 0;
+const size_t BOUNCE = (size_t)8 << 20;
+
+bool put(FILE *f, const void *p, size_t n){ return fwrite(p, 1, n, f) == n; }
+bool get(FILE *f, void *p, size_t n){ return fread(p, 1, n, f) == n; }
+
+bool write_section(FILE *f, const Section &sec, bool device, std::vector<unsigned char> &bounce){
+    for(size_t at = 0; at < sec.bytes; at += BOUNCE){
+        const size_t n = std::min(BOUNCE, sec.bytes - at);
+        const void *src = (const unsigned char *)sec.ptr + at;
+        if(sec.absent){ memset(bounce.data(), 0, n); src = bounce.data(); }
+        else if(device){ ck(qlmx_memcpy_d2h(bounce.data(), src, n), "qlm save d2h"); src = bounce.data(); }
+        if(!put(f, src, n)) return false;
     }
+    return true;
+}
+bool read_section(FILE *f, const Section &sec, bool device, std::vector<unsigned char> &bounce){
+    for(size_t at = 0; at < sec.bytes; at += BOUNCE){
+        const size_t n = std::min(BOUNCE, sec.bytes - at);
+        void *dst = (unsigned char *)sec.ptr + at;
+        if(sec.absent || device){
+            if(!get(f, bounce.data(), n)) return false;
+            if(!sec.absent) ck(qlmx_memcpy_h2d(dst, bounce.data(), n), "qlm load h2d");
+        } else if(!get(f, dst, n)) return false;
+    }
+    return true;
+}
+
+/* fflush + fsync + close, rename over the target, fsync of the directory: after an unclean shutdown the
+ * name refers either to the old complete file or to the new complete one (the reference's save_commit,
+ * cudalm.cu:509-519, gives the reason: a checkpoint of full length whose tail was zeros). */
+bool commit_file(FILE *f, bool ok, const std::string &tmp, const std::string &path){
+    ok = ok && !ferror(f) && fflush(f) == 0 && !ferror(f) && fsync(fileno(f)) == 0;
+    if(fclose(f) != 0) ok = false;
+    if(!ok || rename(tmp.c_str(), path.c_str()) != 0){ remove(tmp.c_str()); return false; }
+    const size_t slash = path.find_last_of('/');
+    const std::string dir = slash == std::string::npos ? "." : (slash == 0 ? "/" : path.substr(0, slash));
+    const int dfd = open(dir.c_str(), O_RDONLY);
+    if(dfd >= 0){ fsync(dfd); close(dfd); }
+    return true;
+}
+
+bool write_optq(const char *path, OptqBody &b, int iter, float prev_gn){
+    const std::string tmp = std::string(path) + ".tmp";
+    FILE *f = fopen(tmp.c_str(), "wb");
+    if(!f) return false;
+    std::vector<unsigned char> bounce(BOUNCE);
+    b.hdr[5] = iter;
+    bool ok = put(f, "QLMH", 4) && put(f, b.hdr, sizeof b.hdr) && put(f, &b.nq, 8) && put(f, &b.ngrp, 8) && put(f, &b.nfloat, 8);
+    for(size_t i = 0; ok && i < b.sections.size(); i++) ok = write_section(f, b.sections[i], b.device, bounce);
+    ok = ok && put(f, "SREF", 4) && put(f, &b.nspan, 4) && put(f, b.sref, (size_t)b.nspan * 4);
+    ok = ok && put(f, "PGN1", 4) && put(f, &prev_gn, 4);
+    return commit_file(f, ok, tmp, path);
+}
+
+/* 0: unreadable, of another shape, or shorter than its header promises (nothing of `b` is touched);
+ * 1: loaded. *have_sref says whether the reference-scale trailer was there. */
+int read_optq(const char *path, OptqBody &b, int *iter, float *prev_gn, bool *have_sref){
+    FILE *f = fopen(path, "rb");
+    if(!f) return 0;
+    struct Closer { FILE *f; ~Closer(){ fclose(f); } } closer{f};
+    char magic[4]; int hdr[6]; u64 nq, ngrp, nfloat;
+    if(!get(f, magic, 4) || memcmp(magic, "QLMH", 4) != 0) return 0;
+    if(!get(f, hdr, sizeof hdr) || !get(f, &nq, 8) || !get(f, &ngrp, 8) || !get(f, &nfloat, 8)) return 0;
+    const bool same_shape = hdr[0] == b.hdr[0] && hdr[1] == b.hdr[1] && hdr[2] == b.hdr[2] && hdr[4] == b.hdr[4]
+                         && nq == b.nq && ngrp == b.ngrp && nfloat <= b.nfloat;
+    if(!same_shape){ fprintf(stderr, "[qlm] %s was written for another shape (digits, group or optimizer differ): ignored\n", path); return 0; }
+    if(nfloat < b.nfloat)       /* float parameters appended since the file was written keep their zero moments */
+        fprintf(stderr, "[qlm] %s: %llu float parameters are newer than the file and start from zero moments\n", path, b.nfloat - nfloat);
+    b.sections[0].bytes = b.sections[1].bytes = (size_t)nfloat * 2;
+    size_t body = 0;
+    for(const Section &s : b.sections) body += s.bytes;
+    struct stat st;
+    if(fstat(fileno(f), &st) != 0 || (u64)st.st_size < 4 + sizeof hdr + 24 + body) return 0;     /* truncated: leave the state alone */
+    std::vector<unsigned char> bounce(BOUNCE);
+    for(const Section &s : b.sections) if(!read_section(f, s, b.device, bounce)) return 0;
     if(iter) *iter = hdr[5];
-    unsigned long long nd = qlmx_qd_bytes(nq, q->packed);
-    std::vector<signed char> hd(nd), hr(nq), hm(nq);
-    std::vector<unsigned char> hv(q->adam ? nq : 0);
-    std::vector<float> hs(ng), hms(ng), hvs(q->adam ? ng : 0);
-    std::vector<bf16> hM(nf), hV(nf);
-    int ok = fread(hM.data(), 2, nf, f) == nf && fread(hV.data(), 2, nf, f) == nf
-          && fread(hd.data(), 1, nd, f) == nd && fread(hr.data(), 1, nq, f) == nq
-          && fread(hm.data(), 1, nq, f) == nq && (q->adam ? fread(hv.data(), 1, nq, f) == nq : 1)
-          && fread(hs.data(), 4, ng, f) == ng && fread(hms.data(), 4, ng, f) == ng
-          && (q->adam ? fread(hvs.data(), 4, ng, f) == ng : 1);
-    std::vector<float> sr; int have_sref = 0;
-    if(ok){ char tm[4]; int ns = 0;
-        if(fread(tm, 1, 4, f) == 4 && !memcmp(tm, "SREF", 4) && fread(&ns, 4, 1, f) == 1 && ns == q->nspan){
-            sr.resize(ns); have_sref = fread(sr.data(), 4, (size_t)ns, f) == (size_t)ns; }
-        float pg;
-        if(have_sref && fread(tm, 1, 4, f) == 4 && !memcmp(tm, "PGN1", 4) && fread(&pg, 4, 1, f) == 1 && pg > 0.0f && isfinite(pg) && prev_gn) *prev_gn = pg; }
-    fclose(f);
-    if(!ok) return 0;
+    char tag[4]; int ns = 0; float pg = 0.0f;
+    std::vector<float> sr;
+    *have_sref = get(f, tag, 4) && memcmp(tag, "SREF", 4) == 0 && get(f, &ns, 4) && ns == b.nspan
+              && (sr.resize((size_t)ns), get(f, sr.data(), (size_t)ns * 4));
+    if(*have_sref){
+        std::copy(sr.begin(), sr.end(), b.sref);
+        if(get(f, tag, 4) && memcmp(tag, "PGN1", 4) == 0 && get(f, &pg, 4) && pg > 0.0f && isfinite(pg) && prev_gn) *prev_gn = pg;
+    }
+    return 1;
+}
+}  // namespace
+
+int qlm_save(const Qlm *q, const char *path, int iter, float prev_gn){
+    OptqBody b = describe(q->dmax, q->group, q->adam, q->nspan, q->packed, q->nq, q->ngrp, q->nfloat,
+                          q->Mc, q->Vc, q->d, q->r, q->m8, q->v8, q->s, q->m8s, q->v8s, true);
+    std::vector<float> sref(q->nspan);
+    for(int i = 0; i < q->nspan; i++) sref[i] = q->spanH[i].sref;
+    b.sref = sref.data();
+    return write_optq(path, b, iter, prev_gn) ? 1 : 0;
+}
+
+int qlm_load(Qlm *q, const char *path, int *iter, float *prev_gn){
+    OptqBody b = describe(q->dmax, q->group, q->adam, q->nspan, q->packed, q->nq, q->ngrp, q->nfloat,
+                          q->Mc, q->Vc, q->d, q->r, q->m8, q->v8, q->s, q->m8s, q->v8s, true);
+    std::vector<float> sref(q->nspan);
+    b.sref = sref.data();
+    bool have_sref = false;
+    if(!read_optq(path, b, iter, prev_gn, &have_sref)) return 0;
     if(have_sref){
-        for(int i = 0; i < q->nspan; i++) q->spanH[i].sref = sr[i];
-        ck(qlmx_memcpy_h2d(q->spanD, q->spanH, (size_t)q->nspan * sizeof(QSpanD)), "qlm load span");
+        for(int i = 0; i < q->nspan; i++) q->spanH[i].sref = sref[i];
+        upload_spans(q, "qlm load span");
     } else
-        fprintf(stderr, "[qlm] %s has no reference-scale record: sref is re-derived from the current weights\n", path);
-    if(q->Mc && nf) ck(qlmx_memcpy_h2d(q->Mc, hM.data(), nf * 2), "qlm load Mc");
-    if(q->Vc && nf) ck(qlmx_memcpy_h2d(q->Vc, hV.data(), nf * 2), "qlm load Vc");
-    ck(qlmx_memcpy_h2d(q->d, hd.data(), nd), "qlm load d");
-    ck(qlmx_memcpy_h2d(q->r, hr.data(), nq), "qlm load r");
-    ck(qlmx_memcpy_h2d(q->m8, hm.data(), nq), "qlm load m8");
-    if(q->adam) ck(qlmx_memcpy_h2d(q->v8, hv.data(), nq), "qlm load v8");
-    ck(qlmx_memcpy_h2d(q->s, hs.data(), ng * 4), "qlm load s");
-    ck(qlmx_memcpy_h2d(q->m8s, hms.data(), ng * 4), "qlm load m8s");
-    if(q->adam) ck(qlmx_memcpy_h2d(q->v8s, hvs.data(), ng * 4), "qlm load v8s");
+        fprintf(stderr, "[qlm] %s carries no reference scales: the spans keep the ones derived at init, so the relative step size may change here\n", path);
     return 1;
 }
 
-void qlm_free(Qlm *q){
-    void *p[] = {q->d, q->r, q->m8, q->v8, q->s, q->m8s, q->v8s, q->statD, q->spanD};
-    for(void *x : p) if(x) qlmx_free(x);
-    free(q->spanH);
-    memset(q, 0, sizeof(*q));
+/* The same file format over host memory (no device needed): for tools and for the byte-level tests
+ * against files the reference wrote. */
+extern "C" int qlm_optq_write_host(const char *path, const QlmOptqHost *v){
+    OptqBody b = describe(v->dmax, v->group, v->adam, v->nspan, v->packed, v->nq, v->ngrp, v->nfloat,
+                          v->Mc, v->Vc, v->d, v->r, v->m8, v->v8, v->s, v->m8s, v->v8s, false);
+    b.sref = v->sref;
+    return write_optq(path, b, v->iter, v->prev_gn) ? 1 : 0;
+}
+extern "C" int qlm_optq_read_host(const char *path, QlmOptqHost *v){
+    OptqBody b = describe(v->dmax, v->group, v->adam, v->nspan, v->packed, v->nq, v->ngrp, v->nfloat,
+                          v->Mc, v->Vc, v->d, v->r, v->m8, v->v8, v->s, v->m8s, v->v8s, false);
+    b.sref = v->sref;
+    bool have_sref = false;
+    const int ok = read_optq(path, b, &v->iter, &v->prev_gn, &have_sref);
+    v->have_sref = have_sref;
+    return ok;
 }
 
 /* ---------------------------------------------------------------------------------------------

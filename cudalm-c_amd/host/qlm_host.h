@@ -77,6 +77,31 @@ int   qlm_save(const Qlm *q, const char *path, int iter, float prev_gn); /* qlm.
 int   qlm_load(Qlm *q, const char *path, int *iter, float *prev_gn);    /* qlm.cuh:740 */
 void  qlm_free(Qlm *q);
 
+/* The .opt.q file format over HOST memory (plain C, no device needed): what qlm_save / qlm_load write and
+ * read, for tools and for byte-level checks against files written by the reference. All pointers are host
+ * arrays of the sizes the header fields imply (Mc, Vc: nfloat bf16, may be NULL = zeros / skipped;
+ * v8, v8s only when adam; sref: nspan floats). read fills the arrays, iter, prev_gn (left alone when the
+ * file has no valid one) and have_sref; both return 1 on success, 0 otherwise. */
+typedef struct {
+    int dmax, group, adam, nspan, packed, iter;
+    unsigned long long nq, ngrp, nfloat;
+    bf16 *Mc, *Vc;
+    signed char *d, *r, *m8;
+    unsigned char *v8;
+    float *s, *m8s, *v8s;
+    float *sref;
+    float prev_gn;
+    int have_sref;
+} QlmOptqHost;
+#ifdef __cplusplus
+extern "C" {
+#endif
+int qlm_optq_write_host(const char *path, const QlmOptqHost *v);
+int qlm_optq_read_host(const char *path, QlmOptqHost *v);
+#ifdef __cplusplus
+}
+#endif
+
 /* grouped expert GEMMs: row-major, B points into the (possibly virtual) fp32 view P */
 void mg_bind(const Qlm *q, const float *Pbase, int act_dtype, int math);
 void mg_ab(const void *A, const float *B, float *C, int M, int K, int N);                /* cudalm.cu:3247 */

@@ -17,8 +17,62 @@ static float nrand(){ float u1 = urand(); if(u1 < 1e-9f) u1 = 1e-9f; float u2 = 
 static int ok_all = 1;
 static void check(const char *name, double v, double tol){ printf("  %-34s %.3e  %s\n", name, v, v <= tol ? "OK" : "FAIL"); if(!(v <= tol)) ok_all = 0; }
 
-int main(){
+/* Spans of the given sizes laid out behind `prefix` float parameters with `gap` more between them. */
+static std::vector<QlmSpanDesc> layout(int prefix, int gap, int nsizes, char **sizes, size_t *np){
+    std::vector<QlmSpanDesc> sp; size_t at = (size_t)prefix;
+    for(int i = 0; i < nsizes; i++){ const size_t n = strtoull(sizes[i], NULL, 10); sp.push_back({at, n}); at += n + (size_t)gap; }
+    *np = at - (size_t)gap + 2;
+    return sp;
+}
+static std::vector<unsigned char> slurp(const char *path){
+    std::vector<unsigned char> b; FILE *f = fopen(path, "rb"); if(!f) return b;
+    fseek(f, 0, SEEK_END); b.resize((size_t)ftell(f)); fseek(f, 0, SEEK_SET);
+    if(fread(b.data(), 1, b.size(), f) != b.size()) b.clear();
+    fclose(f); return b;
+}
+
+/* qlm_selftest optq IN OUT PREFIX GAP N0 [N1 ...]: a Qlm of that layout without weights, qlm_load(IN) into its
+ * device state, qlm_save(OUT) from it. The caller compares the two files.
+ * qlm_selftest sref PFILE OUT PREFIX GAP N0 [N1 ...]: qlm_gpu_init from the fp32 parameters in PFILE; OUT gets
+ * the frozen reference scale of every span followed by all group scales (raw fp32). */
+static int tool(int argc, char **argv){
+    if(argc < 7){ fprintf(stderr, "usage: %s optq|sref IN OUT PREFIX GAP N0 [N1 ...]\n", argv[0]); return 2; }
+    size_t np = 0;
+    std::vector<QlmSpanDesc> sp = layout(atoi(argv[4]), atoi(argv[5]), argc - 6, argv + 6, &np);
+    Qlm q;
+    if(!strcmp(argv[1], "optq")){
+        qlm_gpu_init(&q, sp.data(), (int)sp.size(), NULL, np);
+        if(q.nfloat){
+            q.Mc = (bf16 *)dmalloc(q.nfloat * 2); q.Vc = (bf16 *)dmalloc(q.nfloat * 2);
+            qlmx_memset(q.Mc, 0, q.nfloat * 2, NULL); qlmx_memset(q.Vc, 0, q.nfloat * 2, NULL);
+        }
+        int iter = -1; float pg = 1.0f;
+        if(!qlm_load(&q, argv[2], &iter, &pg)){ fprintf(stderr, "qlm_load failed\n"); return 1; }
+        if(!qlm_save(&q, argv[3], iter, pg)){ fprintf(stderr, "qlm_save failed\n"); return 1; }
+        printf("optq: iter %d prev_gn %g nq %llu ngrp %llu nfloat %llu\n", iter, pg, q.nq, q.ngrp, q.nfloat);
+        return 0;
+    }
+    if(!strcmp(argv[1], "sref")){
+        std::vector<unsigned char> raw = slurp(argv[2]);
+        if(raw.size() != np * 4){ fprintf(stderr, "sref: %s holds %zu bytes, the layout needs %zu\n", argv[2], raw.size(), np * 4); return 1; }
+        float *Pd = (float *)dmalloc(np * 4);
+        qlmx_memcpy_h2d(Pd, raw.data(), np * 4);
+        qlm_gpu_init(&q, sp.data(), (int)sp.size(), Pd, np);
+        std::vector<float> out(q.nspan + q.ngrp);
+        for(int i = 0; i < q.nspan; i++) out[i] = q.spanH[i].sref;
+        qlmx_memcpy_d2h(out.data() + q.nspan, q.s, q.ngrp * 4);
+        FILE *f = fopen(argv[3], "wb");
+        if(!f || fwrite(out.data(), 4, out.size(), f) != out.size()){ fprintf(stderr, "sref: cannot write %s\n", argv[3]); return 1; }
+        fclose(f);
+        printf("sref: %d spans %llu groups, %d float gaps holding %llu parameters\n", q.nspan, q.ngrp, q.nfs, q.nfloat);
+        return 0;
+    }
+    fprintf(stderr, "unknown mode %s\n", argv[1]); return 2;
+}
+
+int main(int argc, char **argv){
     if(qlmx_init(0) != QLMX_OK){ fprintf(stderr, "%s\n", qlmx_last_error()); return 2; }
+    if(argc > 1) return tool(argc, argv);
     printf("[selftest] %s\n", qlmx_device_name());
     /* a toy layer: 16 floats of "norm", then w1, w3 [D,F] x E and w2 [F,D] x E */
     const int E = 3, D = 128, F = 256, N = 40;

@@ -268,6 +268,13 @@ int qlmx_moe_dgate(const float *dout, const float *yp, const int *perm, const fl
 int qlmx_swiglu(const float *G, const float *U, void *O, size_t n, int out_dtype, void *stream);
 int qlmx_swiglu_bwd(const float *Gg, const float *U, const float *dact, void *dg, void *du, size_t n, int out_dtype, void *stream);
 
+/* Test hook (no counterpart in the reference). The decode layer (which = 1) and the split contractions of
+ * qlmx_moe_gemm_nt (which = 2) hand partial results from workgroup to workgroup through bounded waits. Arming the
+ * hook makes the NEXT launch of that kind wait -- for one poll -- for a tag nobody publishes: every wait gives up
+ * at once, every workgroup still runs to its end, the launch's output is invalid, and the following call of that
+ * entry point returns QLMX_E_HIP once, exactly as after a real time-out. One-shot; the call after that is normal. */
+int qlmx_test_force_wait_timeout(int which);
+
 /* =====================================================================================
  * q4n wire format (host only, no device needed): quantize_params / dequantize_params with qtype 3
  * (cudalm.cu:638-656 and 688-696). Per group: fp32 scale + packed nibbles, or a NaN scale followed by

@@ -349,6 +349,9 @@ class Ref(_Lib):
         self._swiglu = s("ref_swiglu", None, [c_vp, c_vp, c_vp, c_sz])
         self._swiglu_bwd = s("ref_swiglu_bwd", None, [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz])
         self._q4n_q = s("ref_q4n_quantize", c_sz, [c_vp, c_sz, c_i, c_vp, c_sz])
+        optq = [c_i, c_i, c_i, c_i, c_vp, c_i, c_u64] + [c_vp] * 9
+        self._qlm_save = s("ref_qlm_save", c_i, [C.c_char_p, c_i, c_f] + optq)
+        self._qlm_load = s("ref_qlm_load", c_i, [C.c_char_p, c_vp, c_vp] + optq)
         self._ng_step = s("ref_ng_q4_step", None, [c_vp] * 10 + [c_i, c_i, c_i, c_f, c_f, c_f, c_f, c_f, c_f, c_f,
                                                                  C.c_uint64, C.c_uint64, c_vp])
         self._q4n_d = s("ref_q4n_dequantize", c_i, [c_vp, c_sz, c_vp, c_sz, c_i])
@@ -416,6 +419,20 @@ class Ref(_Lib):
         self._swiglu_bwd(_p(Gg), _p(U), _p(dact), _p(dg), _p(du), Gg.size)
 
 
+def _ref_qlm_save(self, path, iter_, prev_gn, dmax, group, adam, packed, tab, nfloat, Mc, Vc, d, r, m8, v8, s, m8s, v8s):
+    """the reference's qlm_save (qlm.cuh:702-738) over host arrays; returns its status"""
+    return self._qlm_save(path.encode(), iter_, prev_gn, dmax, group, adam, packed, _p(tab), len(tab), nfloat,
+                          _p(Mc), _p(Vc), _p(d), _p(r), _p(m8), _p(v8), _p(s), _p(m8s), _p(v8s))
+
+
+def _ref_qlm_load(self, path, dmax, group, adam, packed, tab, nfloat, Mc, Vc, d, r, m8, v8, s, m8s, v8s, prev_gn=1.0):
+    """the reference's qlm_load (qlm.cuh:740-788) into host arrays; returns (status, iter, prev_gn); tab's sref is updated"""
+    it = C.c_int(-1); pg = C.c_float(prev_gn)
+    ok = self._qlm_load(path.encode(), C.addressof(it), C.addressof(pg), dmax, group, adam, packed, _p(tab), len(tab), nfloat,
+                        _p(Mc), _p(Vc), _p(d), _p(r), _p(m8), _p(v8), _p(s), _p(m8s), _p(v8s))
+    return ok, it.value, pg.value
+
+
 def _ref_q4n_quantize(self, P, group):
     cap = 4 * P.size + 4 * ((P.size + group - 1) // group) + 16
     out = np.zeros(cap, np.uint8)
@@ -448,6 +465,8 @@ def _ref_gnorm(self, part, nside, clip_side):
     return gs
 
 
+Ref.qlm_save = _ref_qlm_save
+Ref.qlm_load = _ref_qlm_load
 Ref.sqsum = _ref_sqsum
 Ref.gnorm = _ref_gnorm
 Ref.step_touched = _ref_step_touched

@@ -121,4 +121,36 @@ int ref_q4n_dequantize(const unsigned char*buf,size_t len,float*P,size_t n,int g
     Rd r; r.p=buf; r.end=buf+len; return dequantize_params(&r,P,n,3,group);
 }
 
+/* ---- qlm.cuh:702-788: the .opt.q checkpoint, written and read by the reference's own functions over a Qlm
+ * put together from host arrays (under CUDALM_CPU device memory is host memory). `spans` is the span table
+ * (qi0/gi0/ngrp/sref as the caller filled them); prev_gn goes through the global the reference uses. ---- */
+static void ref_qlm_view(Qlm*q,int dmax,int group,int adam,int packed,QSpanD*spans,int nspan,
+                         unsigned long long nfloat,bf16*Mc,bf16*Vc,signed char*d,signed char*r,signed char*m8,
+                         unsigned char*v8,float*s,float*m8s,float*v8s){
+    memset(q,0,sizeof *q);
+    q->on=1; q->dmax=dmax; q->group=group; q->adam=adam; q->packed=packed; q->nspan=nspan;
+    q->spanH=spans; q->spanD=(QSpanD*)malloc((size_t)nspan*sizeof(QSpanD));
+    for(int i=0;i<nspan;i++){ q->nq+=spans[i].n; q->ngrp+=(unsigned long long)spans[i].ngrp; }
+    q->nfloat=nfloat; q->Mc=Mc; q->Vc=Vc; q->d=d; q->r=r; q->m8=m8; q->v8=v8; q->s=s; q->m8s=m8s; q->v8s=v8s;
+}
+int ref_qlm_save(const char*path,int iter,float prev_gn,int dmax,int group,int adam,int packed,QSpanD*spans,int nspan,
+                 unsigned long long nfloat,unsigned short*Mc,unsigned short*Vc,signed char*d,signed char*r,signed char*m8,
+                 unsigned char*v8,float*s,float*m8s,float*v8s){
+    Qlm*q=(Qlm*)malloc(sizeof(Qlm));
+    ref_qlm_view(q,dmax,group,adam,packed,spans,nspan,nfloat,(bf16*)Mc,(bf16*)Vc,d,r,m8,v8,s,m8s,v8s);
+    g_prev_gn=prev_gn;
+    int ok=qlm_save(q,path,iter);
+    free(q->spanD); free(q); return ok;
+}
+int ref_qlm_load(const char*path,int*iter,float*prev_gn,int dmax,int group,int adam,int packed,QSpanD*spans,int nspan,
+                 unsigned long long nfloat,unsigned short*Mc,unsigned short*Vc,signed char*d,signed char*r,signed char*m8,
+                 unsigned char*v8,float*s,float*m8s,float*v8s){
+    Qlm*q=(Qlm*)malloc(sizeof(Qlm));
+    ref_qlm_view(q,dmax,group,adam,packed,spans,nspan,nfloat,(bf16*)Mc,(bf16*)Vc,d,r,m8,v8,s,m8s,v8s);
+    g_prev_gn=*prev_gn;
+    int ok=qlm_load(q,path,iter);
+    *prev_gn=g_prev_gn;
+    free(q->spanD); free(q); return ok;
+}
+
 } /* extern "C" */

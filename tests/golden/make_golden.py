@@ -296,7 +296,37 @@ def golden_q4n():
     save("q4n", dims=np.array([n, group]), P=P, buf=buf, back=back, buf64=buf64)
 
 
+def golden_optq():
+    """.opt.q checkpoints written by the reference's qlm_save (qlm.cuh:702-738): Integer AdamW state and
+    integer Lion state (no v8 / v8s sections), two spans around float parameters (compact bf16 moments),
+    with the SREF and PGN1 trailers. The fixture holds every input array and the file's bytes."""
+    import tempfile
+    group = 128
+    for tag, adam in (("adam", 1), ("lion", 0)):
+        sizes = [128 * 3, 128 * 2]
+        tab, nq, ng = make_spans(sizes, group, pofs=[7, 7 + sizes[0] + 4])
+        nfloat = 7 + 4 + 2
+        seed = 950 + adam
+        d = gen.digits(nq, seed, 1); r = gen.int8(nq, seed, 2, -64, 64); m8 = gen.int8(nq, seed, 3, -127, 127)
+        v8 = gen.u8(nq, seed, 4, 0, 255)
+        s = gen.uniform(ng, seed, 5, 0.5, 1.5) * f32(0.02 * 3 / 7)
+        m8s = gen.uniform(ng, seed, 6, 0.5, 1.5) * f32(3e-3 / 127)
+        v8s = gen.uniform(ng, seed, 7, 0.5, 1.5) * f32(3e-3 / 255)
+        Mc = (gen.normal(nfloat, seed, 8).view(np.uint32) >> 16).astype(np.uint16)
+        Vc = (gen.uniform(nfloat, seed, 9).view(np.uint32) >> 16).astype(np.uint16)
+        tab["sref"] = [f32(0.0123), f32(0.0077)]
+        with tempfile.TemporaryDirectory() as td:
+            path = os.path.join(td, "ck.opt.q")
+            ok = ref.qlm_save(path, 4321, 2.5, 7, group, adam, 1, tab, nfloat, Mc, Vc, d, r, m8, v8 if adam else None,
+                              s, m8s, v8s if adam else None)
+            assert ok == 1
+            data = np.fromfile(path, dtype=np.uint8)
+        save("optq_" + tag, dims=np.array([7, group, adam, 1, 4321, nfloat]), prev_gn=np.array([2.5], f32), tab=tab.view(np.uint8),
+             Mc=Mc, Vc=Vc, d=d, r=r, m8=m8, v8=v8, s=s, m8s=m8s, v8s=v8s, optq=data)
+
+
 if __name__ == "__main__":
+    golden_optq()
     golden_gnorm()
     golden_q4n()
     golden_step_touched()

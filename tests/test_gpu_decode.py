@@ -195,6 +195,34 @@ def test_decode_repeated_calls_alternating_shapes(q, orc):
         assert orc.relerr(out.cpu().numpy(), want) < 2e-5
 
 
+def test_decode_wait_timeout_is_reported_once(q, orc):
+    """The waits between the three task lists are bounded. Forced from the host (qlmx_test_force_wait_timeout: for
+    one launch every wait looks, for one poll, for a tag nobody writes) all of them give up, the kernel still ends
+    normally, the NEXT call returns QLMX_E_HIP once, and the call after that is correct again."""
+    import torch
+    T, E, D, F, K = 8, 8, 256, 512, 2
+    d, s, P, n = encode_layer(orc, 51, E, D, F)
+    x = orc.normal(T * D, 51, 2)
+    rt = orc.normal(T * E, 51, 3)
+    pr = np.zeros(T * E, f32); asn = np.zeros(K * T, np.int32); gate = np.zeros(K * T, f32)
+    orc.router_topk(rt, pr, asn, gate, T, E, K)
+    want = np.zeros(T * D, f32)
+    rc, ws = orc.moe_forward(x, P[:n], P[n:2 * n], P[2 * n:], asn, gate, want, T, D, F, E, K)
+    orc.moe_ws_free(ws)
+    args = (dev(x), dev(asn), dev(gate))
+    dd, ds = dev(d), dev(s)
+    out = torch.zeros(T * D, device="cuda")
+    q.call("qlmx_test_force_wait_timeout", 1)
+    q.decode_forward(*args, out, dd, ds, 128, 0, n, 2 * n, T, K, E, D, F)      # gives up everywhere, ends normally
+    torch.cuda.synchronize()
+    with pytest.raises(pkg.QlmxError, match="gave up waiting"):
+        q.decode_forward(*args, out, dd, ds, 128, 0, n, 2 * n, T, K, E, D, F)
+    out.zero_()
+    q.decode_forward(*args, out, dd, ds, 128, 0, n, 2 * n, T, K, E, D, F)
+    torch.cuda.synchronize()
+    assert orc.relerr(out.cpu().numpy(), want) < 2e-5
+
+
 def test_decode_limits(q):
     import torch
     z = torch.zeros(65536, device="cuda")

@@ -40,6 +40,46 @@ def test_host_mirror_selftest_binary():
     assert p.returncode == 0 and "ALL PASS" in p.stdout, p.stdout
 
 
+@pytest.mark.parametrize("tag", ["adam", "lion"])
+def test_host_mirror_loads_and_rewrites_a_reference_checkpoint(golden, tmp_path, tag):
+    """qlm_load of a .opt.q file written by the reference's qlm_save (fixture) into device state, then qlm_save
+    from that state: the two files are byte-identical (layout of the fixture: 7 float parameters, span of 384,
+    4 floats, span of 256, 2 floats)."""
+    g = golden("optq_" + tag)
+    src, dst = str(tmp_path / "ref.opt.q"), str(tmp_path / "mine.opt.q")
+    g["optq"].tofile(src)
+    env = dict(os.environ)
+    if tag == "lion":
+        env["QLM_OPT"] = "qlion"
+    p = subprocess.run([os.path.join(PKG_DIR, "qlm_selftest"), "optq", src, dst, "7", "4", "384", "256"], env=env,
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert p.returncode == 0, p.stdout
+    assert "iter 4321 prev_gn 2.5" in p.stdout and "nfloat 13" in p.stdout, p.stdout
+    assert np.array_equal(np.fromfile(dst, dtype=np.uint8), g["optq"])
+
+
+def test_host_mirror_init_reference_scales_equal_the_oracle(orc, tmp_path):
+    """qlm_gpu_init (qlm.cuh:458-541) on the device against the oracle: group scales bit for bit and every
+    span's frozen reference scale (mean of its scales, double sum in group order) bit for bit."""
+    sizes = [128 * 300, 128 * 77 + 40, 128 * 1000]
+    prefix, gap = 16, 8
+    tab, nq, ng = make_spans(sizes, 128, pofs=[prefix, prefix + sizes[0] + gap, prefix + sizes[0] + sizes[1] + 2 * gap])
+    np_ = prefix + sum(sizes) + 2 * gap + 2
+    P = orc.normal(np_, 77, 1, 0.02)
+    src, dst = str(tmp_path / "P.f32"), str(tmp_path / "sref.f32")
+    P.tofile(src)
+    p = subprocess.run([os.path.join(PKG_DIR, "qlm_selftest"), "sref", src, dst, str(prefix), str(gap)] + [str(n) for n in sizes],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert p.returncode == 0, p.stdout
+    assert "4 float gaps holding %d parameters" % (prefix + 2 * gap + 2) in p.stdout, p.stdout
+    got = np.fromfile(dst, dtype=f32)
+    d = np.zeros((nq + 1) // 2 + 64, np.int8); r = np.zeros(nq, np.int8); s = np.zeros(ng, f32)
+    orc.encode(P, d, r, s, tab, 128, 7, 1, ng)
+    orc.span_sref(tab, s)
+    assert np.array_equal(got[3:].view(np.uint32), s.view(np.uint32))
+    assert np.array_equal(got[:3].view(np.uint32), tab["sref"].astype(f32).view(np.uint32))
+
+
 def test_c4_full_adamw_sweep_bit_exact(q, orc):
     """Config 4: 120*2^20 weights, seeded random integer state, grads ~N(0,1e-3), lr 3e-4,
     betas (0.9, 0.95), wd 0.1, t=1: d, r, m8, v8, m8s, v8s byte-identical to the CPU oracle."""

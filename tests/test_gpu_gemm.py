@@ -331,6 +331,20 @@ def test_mfma_nt_split_contraction(q, orc, beta):
     assert orc.relerr(got3, want3) < TOL_MFMA
 
 
+def test_mfma_nt_split_contraction_timeout_is_reported_once(q, orc):
+    """A slice's wait for its predecessor is bounded. Forced from the host (qlmx_test_force_wait_timeout: the next
+    launch waits for one poll for a tag nobody publishes) every wait gives up, every workgroup still finishes, and
+    the NEXT nt call reports QLMX_E_HIP -- once; the call after it is a normal, correct launch."""
+    import torch
+    q.call("qlmx_test_force_wait_timeout", 2)
+    run_case(q, orc, "nt", 4, [1700, 40, 0, 333], 256, 256, pkg.ACT_BF16, pkg.MATH_MFMA, seed=16)     # completes; output not checked
+    torch.cuda.synchronize()
+    with pytest.raises(pkg.QlmxError, match="gave up waiting"):
+        run_case(q, orc, "nt", 4, [1700, 40, 0, 333], 256, 256, pkg.ACT_BF16, pkg.MATH_MFMA, seed=16)
+    got, want = run_case(q, orc, "nt", 4, [1700, 40, 0, 333], 256, 256, pkg.ACT_BF16, pkg.MATH_MFMA, seed=16)
+    assert orc.relerr(got, want) < TOL_MFMA
+
+
 @pytest.mark.parametrize("mode", ["nn", "tn"])
 def test_mfma_last_tile_heights(q, orc, mode):
     """The last row tile of a problem runs at the smallest height (in steps of 64 rows) that holds it:

@@ -28,7 +28,8 @@ MATH_F32, MATH_MFMA = 0, 1
 
 
 def lib_path():
-    return os.path.join(HERE, "libqlmx.so")
+    """QLMX_LIB names another build of the library (comparing two builds in one harness)"""
+    return os.environ.get("QLMX_LIB") or os.path.join(HERE, "libqlmx.so")
 
 
 def _ptr(x):
@@ -75,6 +76,7 @@ SIGNATURES = {
     "qlmx_moe_decode_forward": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_decode_forward_noalloc": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_test_force_wait_timeout": (c_i, [c_i]),
+    "qlmx_test_sqrt_form": (c_i, [C.c_uint, c_u64, c_vp, c_vp]),
     "qlmx_step_touched": (c_i, [c_vp] * 10 + [c_i, c_i, c_i, c_f, c_f, c_f, c_f, c_f, c_f, c_f, c_u64, c_u64, c_vp, c_i, c_vp]),
     "qlmx_sqsum": (c_i, [c_vp, c_u64, c_vp, c_vp]),
     "qlmx_gnorm": (c_i, [c_vp, c_i, c_i, c_vp, c_vp]),

@@ -57,6 +57,28 @@ __device__ __forceinline__ float qx_gdiv(float a, const GroupDiv &d){
     return a / d.b;
 }
 
+/* Correctly rounded square root for a whole row of values at a lower price. sqrtf() as the compiler expands it
+ * is v_sqrt_f32 (good to one unit in the last place) followed by a test of both neighbours through exact
+ * residuals, wrapped in a rescaling for subnormal inputs and a pass-through for 0 and infinity: 17 instructions.
+ * For x >= 2^-96 the wrapping does nothing, and what is left -- the same instruction, the same two tests, hence the
+ * same bits -- takes 9. The caller uses this form only when every lane's values are above the bound (a wavefront-
+ * uniform choice) and sqrtf() otherwise; infinity passes through both. */
+__device__ __forceinline__ float qx_sqrt_above_2m96(float x){
+    const float s = __builtin_amdgcn_sqrtf(x);
+    const float dn = __uint_as_float(__float_as_uint(s) - 1u), up = __uint_as_float(__float_as_uint(s) + 1u);
+    const float rdn = __builtin_fmaf(-dn, s, x), rup = __builtin_fmaf(-up, s, x);
+    float r = rdn <= 0.0f ? dn : s;
+    r = rup > 0.0f ? up : r;
+    return r;
+}
+__device__ __forceinline__ int qx_med3i(int v, int lo, int hi){            /* clamp in one instruction; lo <= hi */
+    int r; asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi)); return r;
+}
+/* the carry of a residual that left [-64, 64] (qlm.cuh:232-236: rr > 64 ? ((rr-65)>>7)+1 : rr < -64 ? -(((-rr-65)>>7)+1) : 0)
+ * without branches: for rr >= 0 that is (rr + 63) >> 7, for rr < 0 it is floor((rr + 64) / 128), i.e. the same
+ * shift of rr + 63 + 1. Checked against the branching form over all of [-40000, 40000] on the host. */
+__host__ __device__ __forceinline__ int qx_carry(int rr){ return (rr + 63 - (rr >> 31)) >> 7; }
+
 /* New first moment, new (stored form of the) second moment and the clamped Adam ratio u of one
  * element: qlm.cuh:209-229. */
 template<bool ADAM>
@@ -98,7 +120,9 @@ __device__ __forceinline__ ElemRes step_elem(const GroupCtx &c, float graw, int 
     return o;
 }
 
-template<bool ADAM>
+/* STAT: the four counters are kept; HASP: the fp32 view is written. Both are fixed per launch, so they are
+ * template parameters and the usual launch (neither) carries no trace of them. */
+template<bool ADAM, bool STAT, bool HASP>
 __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
     const int lane16 = threadIdx.x & 15;
     const int team = (int)((blockIdx.x * (unsigned)blockDim.x + threadIdx.x) >> 4);
@@ -128,7 +152,7 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
     const uint64_t ktv = kt + 0xBEEFULL * QLMX_KT;
 
     unsigned long long st_carry = 0, st_rail = 0, st_zero = 0, st_idl = 0;
-    const bool want_stat = a.stat != nullptr;
+    const bool want_stat = STAT;
 
     const bool fast = a.vec_ok && a.group == 128 && a.packed && n == 128 && ((pof | qi0 | gof) & 7ULL) == 0;
     if(fast){
@@ -142,58 +166,114 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
         uint2 vw = make_uint2(0u, 0u);
         if(ADAM) vw = *(const uint2 *)(a.v8 + q);
         const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
-        float mn[8], rv[8], pv[8];
+        float mn[8], rv[8], uu[8];
+        /* ---- moments (qlm.cuh:209-229); the square roots of a lane's eight values are taken together ---- */
+        if(ADAM){
+            float vv[8], vmin = 1.0f;
+#pragma unroll
+            for(int k = 0; k < 8; k++){
+                const uint32_t mword = k < 4 ? mw.x : mw.y, vword = k < 4 ? vw.x : vw.y;
+                const int sh = 8 * (k & 3);
+                const float gr = gv[k] * c.gs;
+                const float mv = (float)(int)(signed char)(mword >> sh) * c.ms_old;
+                float sv = (float)((vword >> sh) & 0xFFu) * c.vs_old; if(c.v4) sv = sv * sv;
+                mn[k] = c.b1 * mv + c.omb1 * gr;
+                vv[k] = c.b2 * (sv * sv) + c.omb2 * gr * gr;
+                vmin = fminf(vmin, vv[k]);
+            }
+            /* NaN compares false and takes the general form with the rest of its wavefront */
+            if(__builtin_amdgcn_ballot_w64(!(vmin >= 0x1p-96f)) == 0){
+#pragma unroll
+                for(int k = 0; k < 8; k++) rv[k] = qx_sqrt_above_2m96(vv[k]);
+            } else {
+#pragma unroll
+                for(int k = 0; k < 8; k++) rv[k] = sqrtf(vv[k]);
+            }
+#pragma unroll
+            for(int k = 0; k < 8; k++){
+                const float u = (mn[k] * c.inv_bc1) / (rv[k] * c.inv_sqrt_bc2 + c.veps);
+                uu[k] = fmaxf(-8.0f, fminf(8.0f, u));
+                if(c.v4) rv[k] = sqrtf(rv[k]);
+            }
+        } else {
+#pragma unroll
+            for(int k = 0; k < 8; k++){
+                const uint32_t mword = k < 4 ? mw.x : mw.y;
+                float r0;
+                elem_moments<false>(c, gv[k], (int)(signed char)(mword >> (8 * (k & 3))), 0, mn[k], r0, uu[k]);
+                rv[k] = r0;
+            }
+        }
+        /* ---- digits and residuals (qlm.cuh:230-242). Every new byte or nibble enters its word from the top
+         * (one funnel shift each), so after all eight the first element sits lowest. ---- */
+        float pv[8];
         uint32_t dnew = 0, rn0 = 0, rn1 = 0;
         float am = 0.0f, vm = 0.0f;
         uint64_t key = q * QLMX_KI;
 #pragma unroll
         for(int k = 0; k < 8; k++){
-            const uint32_t rword = k < 4 ? rw.x : rw.y, mword = k < 4 ? mw.x : mw.y, vword = k < 4 ? vw.x : vw.y;
-            const int sh = 8 * (k & 3);
-            const int rold = (int)(signed char)(rword >> sh);
-            const int m8v  = (int)(signed char)(mword >> sh);
-            const int v8v  = (int)((vword >> sh) & 0xFFu);
-            const int dd   = qx_nib(dw, k);
-            ElemRes o = step_elem<ADAM>(c, gv[k], m8v, v8v, dd, rold, key + kt);
-            mn[k] = o.mn; rv[k] = o.rv;
-            pv[k] = c.sg * (float)o.dd;
-            dnew |= ((uint32_t)o.dd & 15u) << (4 * k);
-            if(k < 4) rn0 |= ((uint32_t)o.rr & 0xFFu) << sh; else rn1 |= ((uint32_t)o.rr & 0xFFu) << sh;
-            am = fmaxf(am, fabsf(o.mn)); vm = fmaxf(vm, o.rv);
-            if(want_stat){
-                unsigned ai = (unsigned)(o.idl < 0 ? -o.idl : o.idl);
+            const uint32_t rword = k < 4 ? rw.x : rw.y;
+            const int rold = (int)(signed char)(rword >> (8 * (k & 3)));
+            const int dd = qx_nib(dw, k);
+            const int idl = qx_sround(-(c.L * uu[k] + c.dec * (float)dd), key + kt);
+            const int rr0 = rold + idl;
+            const int cy = qx_carry(rr0);
+            const int rr = rr0 - cy * 128;
+            const int dn = qx_med3i(dd + cy, -c.dmax, c.dmax);
+            if(HASP) pv[k] = c.sg * (float)dn;
+            dnew = __builtin_amdgcn_alignbit((uint32_t)dn, dnew, 4);
+            if(k < 4) rn0 = __builtin_amdgcn_alignbit((uint32_t)rr, rn0, 8); else rn1 = __builtin_amdgcn_alignbit((uint32_t)rr, rn1, 8);
+            am = fmaxf(am, fabsf(mn[k])); vm = fmaxf(vm, rv[k]);
+            if(STAT){
+                unsigned ai = (unsigned)(idl < 0 ? -idl : idl);
                 st_idl = st_idl > ai ? st_idl : ai;
-                st_carry += (unsigned)(o.carry < 0 ? -o.carry : o.carry);
-                st_rail += (o.dd == c.dmax) | (o.dd == -c.dmax);
-                st_zero += (o.dd == 0);
+                st_carry += (unsigned)(cy < 0 ? -cy : cy);
+                st_rail += (dn == c.dmax) | (dn == -c.dmax);
+                st_zero += (dn == 0);
             }
             key += QLMX_KI;
         }
         *(uint32_t *)(a.d + (q >> 1)) = dnew;
         *(uint2 *)(a.r + q) = make_uint2(rn0, rn1);
-        if(a.P){
+        if(HASP){
             /* the rendered view is not read again by this launch: written past the caches */
             typedef float f4 __attribute__((ext_vector_type(4)));
             f4 p0 = {pv[0], pv[1], pv[2], pv[3]}, p1 = {pv[4], pv[5], pv[6], pv[7]};
             __builtin_nontemporal_store(p0, (f4 *)(a.P + pof + e0));
             __builtin_nontemporal_store(p1, (f4 *)(a.P + pof + e0 + 4));
         }
+        /* ---- fresh scales and the re-quantised moments (qlm.cuh:244-278) ---- */
         am = qx_row16_max(am); vm = qx_row16_max(vm);
         const float ms = am > 0.0f ? am / 127.0f : 1e-12f;
         const float vs = vm > 0.0f ? vm / 255.0f : 1e-12f;
         const GroupDiv dms = qx_mkdiv(ms), dvs = qx_mkdiv(vs);
         if(lane16 == 0){ a.m8s[gi] = ms; if(ADAM) a.v8s[gi] = vs; }
+        /* one choice for the wavefront: the reciprocal form when all four groups allow it (the usual case) */
+        const bool recip = __builtin_amdgcn_ballot_w64(!(dms.fast && (!ADAM || dvs.fast))) == 0;
         uint32_t mo0 = 0, mo1 = 0, vo0 = 0, vo1 = 0;
         key = q * QLMX_KI;
 #pragma unroll
         for(int k = 0; k < 8; k++){
-            const int sh = 8 * (k & 3);
-            int mq = qx_clamp(qx_sround(qx_gdiv(mn[k], dms), key + ktm), -127, 127);
-            if(k < 4) mo0 |= ((uint32_t)mq & 0xFFu) << sh; else mo1 |= ((uint32_t)mq & 0xFFu) << sh;
+            float qm, qv = 0.0f;
+            if(recip){
+                const float t = mn[k] * dms.y; qm = fmaf(fmaf(-t, dms.b, mn[k]), dms.y, t);
+                if(ADAM){ const float w = rv[k] * dvs.y; qv = fmaf(fmaf(-w, dvs.b, rv[k]), dvs.y, w); }
+            } else {
+                qm = mn[k] / ms;
+                if(ADAM) qv = rv[k] / vs;
+            }
+            const int mq = qx_med3i(qx_sround(qm, key + ktm), -127, 127);
+            if(k < 4) mo0 = __builtin_amdgcn_alignbit((uint32_t)mq, mo0, 8); else mo1 = __builtin_amdgcn_alignbit((uint32_t)mq, mo1, 8);
             if(ADAM){
-                int vq = qx_clamp(qx_sround(qx_gdiv(rv[k], dvs), key + ktv), 0, 255);
-                if(vq == 0 && rv[k] > 0.0f) vq = 1;
-                if(k < 4) vo0 |= (uint32_t)vq << sh; else vo1 |= (uint32_t)vq << sh;
+                /* floor + stochastic increment stay in floating point (whole numbers, exact); the conversion that
+                 * packs the byte saturates to [0, 255], which is the clamp of qlm.cuh:274; a positive moment
+                 * never rounds to the code 0 (qlm.cuh:275) */
+                const float fl = floorf(qv);
+                const uint32_t h = qx_hash(key + ktv);
+                const float ur = (float)(h >> 8) * (1.0f / 16777216.0f);
+                float vq = fl + (ur < (qv - fl) ? 1.0f : 0.0f);
+                vq = fmaxf(vq, rv[k] > 0.0f ? 1.0f : 0.0f);
+                if(k < 4) vo0 = __builtin_amdgcn_cvt_pk_u8_f32(vq, k & 3, vo0); else vo1 = __builtin_amdgcn_cvt_pk_u8_f32(vq, k & 3, vo1);
             }
             key += QLMX_KI;
         }
@@ -273,6 +353,17 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
     }
 }
 
+template<bool ADAM> static void step_launch_opt(const StepParams &a, unsigned blocks, hipStream_t st){
+    const bool stat = a.stat != nullptr, hasp = a.P != nullptr;
+    if(stat && hasp)  hipLaunchKernelGGL((k_qlmx_step<ADAM, true, true>),   dim3(blocks), dim3(256), 0, st, a);
+    else if(stat)     hipLaunchKernelGGL((k_qlmx_step<ADAM, true, false>),  dim3(blocks), dim3(256), 0, st, a);
+    else if(hasp)     hipLaunchKernelGGL((k_qlmx_step<ADAM, false, true>),  dim3(blocks), dim3(256), 0, st, a);
+    else              hipLaunchKernelGGL((k_qlmx_step<ADAM, false, false>), dim3(blocks), dim3(256), 0, st, a);
+}
+static void step_launch(const StepParams &a, bool adam, unsigned blocks, hipStream_t st){
+    if(adam) step_launch_opt<true>(a, blocks, st); else step_launch_opt<false>(a, blocks, st);
+}
+
 /* qlm_step_launch (qlm.cuh:377-397) */
 extern "C" int qlmx_step(float *P, const float *G, signed char *d, signed char *r, const float *s,
               signed char *m8, float *m8s, unsigned char *v8, float *v8s,
@@ -300,8 +391,7 @@ extern "C" int qlmx_step(float *P, const float *G, signed char *d, signed char *
                && ((uintptr_t)d & 3) == 0;
     const unsigned blocks = (unsigned)((ng + 15) / 16);
     hipStream_t st = (hipStream_t)stream;
-    if(adam) hipLaunchKernelGGL(k_qlmx_step<true>,  dim3(blocks), dim3(256), 0, st, a);
-    else     hipLaunchKernelGGL(k_qlmx_step<false>, dim3(blocks), dim3(256), 0, st, a);
+    step_launch(a, adam != 0, blocks, st);
     QLMX_LAUNCH_CHECK("qlmx_step launch");
     return QLMX_OK;
 }
@@ -335,7 +425,7 @@ extern "C" int qlmx_step_touched(float *P, const float *Gc, signed char *d, sign
     a.one.pof = 0; a.one.gof = 0; a.one.qi0 = 0; a.one.n = nt; a.one.gi0 = 0;
     a.one.ngrp = (int)((nt + (unsigned long long)group - 1) / (unsigned long long)group); a.one.sref = sref;
     const unsigned blocks = (unsigned)((ntouched + 15) / 16);
-    hipLaunchKernelGGL(k_qlmx_step<true>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+    step_launch(a, true, blocks, (hipStream_t)stream);
     QLMX_LAUNCH_CHECK("qlmx_step_touched launch");
     return QLMX_OK;
 }
@@ -418,5 +508,25 @@ extern "C" int qlmx_gnorm(const float *part, int nside, int clip_side, float *gs
     QLMX_REQUIRE(part && gs && nside >= 0, "qlmx_gnorm: bad arguments");
     hipLaunchKernelGGL(k_qlmx_gnorm, dim3(1), dim3(1), 0, (hipStream_t)stream, part, nside, clip_side, gs);
     QLMX_LAUNCH_CHECK("qlmx_gnorm launch");
+    return QLMX_OK;
+}
+
+/* ---- test hook: the short square-root form against sqrtf() over a range of bit patterns ---- */
+__global__ void __launch_bounds__(256) k_qlmx_test_sqrt(unsigned first, unsigned long long count, unsigned long long *mismatches){
+    unsigned long long bad = 0;
+    for(unsigned long long i = (unsigned long long)blockIdx.x * 256 + threadIdx.x; i < count; i += (unsigned long long)gridDim.x * 256){
+        const float x = __uint_as_float(first + (unsigned)i);
+        const float a = qx_sqrt_above_2m96(x), b = sqrtf(x);
+        bad += __float_as_uint(a) != __float_as_uint(b);
+    }
+    if(bad) atomicAdd(mismatches, bad);
+}
+extern "C" int qlmx_test_sqrt_form(unsigned first_bits, unsigned long long count, unsigned long long *mismatches_dev, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(mismatches_dev, "qlmx_test_sqrt_form: NULL counter");
+    QLMX_REQUIRE(first_bits >= 0x0F800000u && (unsigned long long)first_bits + count <= 0x7F800001ULL,
+                 "qlmx_test_sqrt_form: the range must lie inside [2^-96, +infinity]");
+    hipLaunchKernelGGL(k_qlmx_test_sqrt, dim3(4096), dim3(256), 0, (hipStream_t)stream, first_bits, count, mismatches_dev);
+    QLMX_LAUNCH_CHECK("sqrt test launch");
     return QLMX_OK;
 }

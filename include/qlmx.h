@@ -274,6 +274,11 @@ int qlmx_swiglu_bwd(const float *Gg, const float *U, const float *dact, void *dg
  * at once, every workgroup still runs to its end, the launch's output is invalid, and the following call of that
  * entry point returns QLMX_E_HIP once, exactly as after a real time-out. One-shot; the call after that is normal. */
 int qlmx_test_force_wait_timeout(int which);
+/* Test hook. qlmx_step takes the square roots of the second moment with a short form of the correctly rounded
+ * sqrtf() that is valid for arguments in [2^-96, +infinity] (and switches to sqrtf() itself below that). This
+ * compares the two forms on the device for the `count` consecutive bit patterns starting at first_bits and adds
+ * the number of differing results to *mismatches_dev (device memory, unsigned long long). */
+int qlmx_test_sqrt_form(unsigned first_bits, unsigned long long count, unsigned long long *mismatches_dev, void *stream);
 
 /* =====================================================================================
  * q4n wire format (host only, no device needed): quantize_params / dequantize_params with qtype 3

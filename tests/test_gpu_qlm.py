@@ -248,6 +248,43 @@ def test_sqsum_gnorm_and_clipped_step(q, orc, golden):
         assert beq(got, want), nm
 
 
+def test_short_sqrt_form_equals_sqrtf_on_every_float_it_serves(q):
+    """The step's square root of the second moment is v_sqrt_f32 plus the two neighbour tests of the compiler's own
+    sqrtf expansion, without that expansion's subnormal rescaling; it is used for arguments >= 2^-96. Exhaustive:
+    all 1,879,048,193 bit patterns from 2^-96 to +infinity give the bits sqrtf gives."""
+    import torch
+    bad = torch.zeros(1, dtype=torch.int64, device="cuda")
+    first, last = 0x0F800000, 0x7F800000
+    q.call("qlmx_test_sqrt_form", first, last - first + 1, bad, None)
+    torch.cuda.synchronize()
+    assert int(bad.item()) == 0
+
+
+def test_step_zero_and_tiny_second_moments_take_the_general_square_root(q, orc):
+    """Groups whose gradient and second moment are exactly zero, or so small that the new second moment is a
+    subnormal number, sit below the short form's bound; whole wavefronts then take sqrtf. Bytes equal the oracle."""
+    import torch
+    group, dmax = 128, 7
+    tab, nq, ng = make_spans([128 * 64], group)
+    tab["sref"] = [0.0086]
+    hd = orc.digits(nq, 9, 20); hr = orc.int8(nq, 9, 21, -64, 64); hm8 = orc.int8(nq, 9, 22, -127, 127)
+    hv8 = orc.u8(nq, 9, 23, 0, 255)
+    hs = orc.uniform(ng, 9, 24, 0.5, 1.5) * f32(0.02 * 3 / 7)
+    hm8s = orc.uniform(ng, 9, 25, 0.5, 1.5) * f32(3e-3 / 127); hv8s = orc.uniform(ng, 9, 26, 0.5, 1.5) * f32(3e-3 / 255)
+    hG = orc.normal(nq, 9, 27, 1e-3)
+    hG[:128 * 8] = 0.0; hv8[:128 * 8] = 0                      # exact zeros: vv = 0
+    hG[128 * 8:128 * 16] *= f32(1e-22); hv8[128 * 8:128 * 16] = 0    # gr^2 * 0.05 ~ 1e-51: subnormal / underflowing
+    hG[128 * 16:128 * 17] *= f32(1e-18); hv8s[16] = f32(1e-20)       # tiny but mixed with a live v8
+    hv8[128 * 20 + 5] = 0; hG[128 * 20 + 5] = 0.0                    # one zero element in an ordinary group
+    d, r, m8, v8, s, m8s, v8s, G = (dev(x) for x in (hd, hr, hm8, hv8, hs, hm8s, hv8s, hG))
+    for t in (1, 2):
+        hp = (3e-4, 0.9, 0.95, 0.1, 1.0, None, 10.0, 4.4721, 0, t, 1, None, 1, 0, ng)
+        q.step(None, G, d, r, s, m8, m8s, v8, v8s, dev(tab), 1, group, dmax, *hp)
+        orc.step(None, hG, hd, hr, hs, hm8, hm8s, hv8, hv8s, tab, group, dmax, *hp)
+    for got, want, nm in [(d, hd, "d"), (r, hr, "r"), (m8, hm8, "m8"), (v8, hv8, "v8"), (m8s, hm8s, "m8s"), (v8s, hv8s, "v8s")]:
+        assert beq(got, want), nm
+
+
 def test_argument_errors(q):
     import torch
     x = torch.zeros(256, device="cuda")

@@ -39,6 +39,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train", "train5", "c5", "codec", "glue", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--fwd-math", default="f16", choices=["f16", "bf16x2"],
+                    help="train, c5: forward GEMMs on the fp16 matrix core (one MFMA per product, 2e-4 relative L2) or as bf16 hi+lo (two, 3e-6)")
     ap.add_argument("--step-only", action="store_true", help="train: skip the per-launch repetitions, so that a kernel trace holds nothing but steps")
     ap.add_argument("--adamw-weights", type=int, default=120 * 2 ** 20)
     ap.add_argument("--render-p", type=int, default=0, help="adamw: also write the fp32 view P (4 B/weight more)")
@@ -84,7 +86,8 @@ def zipf_counts(E, tokens, topk, seed=0):
 
 
 def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label="C3 train layer"):
-    from cudalm_c_amd.binding import ACT_BF16, MATH_MFMA
+    from cudalm_c_amd.binding import ACT_BF16, MATH_MFMA, MATH_MFMA_F16
+    FWD = MATH_MFMA if args.fwd_math == "bf16x2" else MATH_MFMA_F16
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev); g.manual_seed(0)
     cnt = zipf_counts(E, tokens, topk)
@@ -137,8 +140,8 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
     # the order of moe_forward / moe_backward (cudalm.cu:4211-4225, 4333-4335, 4362-4366): each backward flush
     # holds the weight gradient and the input gradient of the same operands
     calls = [
-        ("fwd w1,w3 (nn)", lambda: q.gemm_nn(d, s, group, p_w13, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream), 2),
-        ("fwd w2 (nn)", lambda: q.gemm_nn(d, s, group, p_w2, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
+        ("fwd w1,w3 (nn)", lambda: q.gemm_nn(d, s, group, p_w13, 2 * E, D, F, ACT_BF16, FWD, stream), 2),
+        ("fwd w2 (nn)", lambda: q.gemm_nn(d, s, group, p_w2, E, F, D, ACT_BF16, FWD, stream), 1),
         ("wgrad w2 (nt)", lambda: q.gemm_nt(p_g2, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
         ("dgrad w2 (tn)", lambda: q.gemm_tn(d, s, group, p_d2, E, D, F, ACT_BF16, MATH_MFMA, stream), 1),
         ("wgrad w1,w3 (nt)", lambda: q.gemm_nt(p_g13, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream), 2),
@@ -174,7 +177,8 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
         "kernel_ms": tm, "per_launch": per, "beside_the_step": extra, "gflop_per_step": flops / 1e9,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": None, "kernel": "k_gemm_nn_lds, k_gemm_tn_lds, k_gemm_nt_lds (all 6 launches; slowest: %s)" % dom,
-                     "note": "algorithmic flops only; the forward issues two MFMAs per product (bf16 hi+lo weight split)"},
+                     "note": "algorithmic flops only; forward math: " + ("bf16 hi+lo weight split, two MFMAs per product" if args.fwd_math == "bf16x2" else
+                             "fp16 matrix core, bf16 activations converted exactly, weights rounded once to fp16 (2e-4 relative L2), one MFMA per product")},
     }
 
 
@@ -187,7 +191,8 @@ def bench_c5(torch, q, args, L=8, E=64, D=2048, F=1408, tokens=32768, topk=4):
     A step of this workload is heavy (about 0.1 s), so it is timed over max(3, K // 10) steps after max(1, W // 10)
     warm-up steps; both figures are in the result."""
     import numpy as np
-    from cudalm_c_amd.binding import ACT_BF16, MATH_MFMA, SPAN_DTYPE
+    from cudalm_c_amd.binding import ACT_BF16, MATH_MFMA, MATH_MFMA_F16, SPAN_DTYPE
+    FWD = MATH_MFMA if args.fwd_math == "bf16x2" else MATH_MFMA_F16
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev); g.manual_seed(0)
     group = 128
@@ -243,8 +248,8 @@ def bench_c5(torch, q, args, L=8, E=64, D=2048, F=1408, tokens=32768, topk=4):
         p_g13 = P(items(Xp, D, dgp, F, G, 0, o1, True) + items(Xp, D, dup, F, G, 0, o3, True))
         p_d1 = P(items(dgp, F, None, 0, dXp, D, o1)); p_d3 = P(items(dup, F, None, 0, dXp, D, o3, beta=1.0))
         calls += [
-            (lambda p=p_w13: q.gemm_nn(d, s, group, p, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream)),
-            (lambda p=p_w2: q.gemm_nn(d, s, group, p, E, F, D, ACT_BF16, MATH_MFMA, stream)),
+            (lambda p=p_w13: q.gemm_nn(d, s, group, p, 2 * E, D, F, ACT_BF16, FWD, stream)),
+            (lambda p=p_w2: q.gemm_nn(d, s, group, p, E, F, D, ACT_BF16, FWD, stream)),
             (lambda p=p_g2: q.gemm_nt(p, E, F, D, ACT_BF16, MATH_MFMA, stream)),
             (lambda p=p_d2: q.gemm_tn(d, s, group, p, E, D, F, ACT_BF16, MATH_MFMA, stream)),
             (lambda p=p_g13: q.gemm_nt(p, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream)),

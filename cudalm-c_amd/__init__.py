@@ -6,5 +6,5 @@ module is a thin ctypes loader used by the tests, bench.py and __graft_entry__.p
 arithmetic of its own and has no fallback: if the library is missing or no gfx950 device is bound,
 every call raises.
 """
-from .binding import (Qlmx, QlmxError, GemmProb, SPAN_DTYPE, ACT_F32, ACT_BF16, MATH_F32, MATH_MFMA,  # noqa: F401
+from .binding import (Qlmx, QlmxError, GemmProb, SPAN_DTYPE, ACT_F32, ACT_BF16, MATH_F32, MATH_MFMA, MATH_MFMA_F16,  # noqa: F401
                       load, lib_path)

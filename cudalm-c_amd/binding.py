@@ -24,7 +24,7 @@ class GemmProb(C.Structure):
 
 
 ACT_F32, ACT_BF16 = 0, 1
-MATH_F32, MATH_MFMA = 0, 1
+MATH_F32, MATH_MFMA, MATH_MFMA_F16 = 0, 1, 2
 
 
 def lib_path():

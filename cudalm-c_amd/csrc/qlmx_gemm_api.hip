@@ -8,7 +8,7 @@ int qlmx_gemm_f32_dispatch(int mode, const signed char *d, const float *s, int g
 int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob,
                           int K, int N, hipStream_t st);
 int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int group,
-                            const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second, int nprob, int K, int N, int act_dtype, hipStream_t st);
+                            const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second, int nprob, int K, int N, int act_dtype, hipStream_t st, bool f16);
 
 static int gemm_entry(const char *who, int mode, const signed char *d, const float *s, int group,
                       const qlmx_gemm_prob *probs, int nprob, int K, int N, int act_dtype, int math, void *stream,
@@ -16,7 +16,7 @@ static int gemm_entry(const char *who, int mode, const signed char *d, const flo
     int rc = qlmx_check_ready(); if(rc) return rc;
     QLMX_REQUIRE(K > 0 && N > 0, "%s: K=%d N=%d", who, K, N);
     QLMX_REQUIRE(act_dtype == QLMX_ACT_F32 || act_dtype == QLMX_ACT_BF16, "%s: act_dtype %d", who, act_dtype);
-    QLMX_REQUIRE(math == QLMX_MATH_F32 || math == QLMX_MATH_MFMA, "%s: math %d", who, math);
+    QLMX_REQUIRE(math == QLMX_MATH_F32 || math == QLMX_MATH_MFMA || math == QLMX_MATH_MFMA_F16, "%s: math %d", who, math);
     if(mode != GEMM_NT){
         QLMX_REQUIRE(d && s, "%s: NULL digits or scales", who);
         QLMX_REQUIRE(group >= 2 && group <= 256 && (group & 1) == 0, "%s: group %d", who, group);
@@ -26,8 +26,8 @@ static int gemm_entry(const char *who, int mode, const signed char *d, const flo
             QLMX_REQUIRE(probs[i].wq % (unsigned long long)group == 0 && (!second || second[i].wq % (unsigned long long)group == 0),
                          "%s: problem %d weight offset is not group aligned", who, i);
     }
-    if(math == QLMX_MATH_MFMA)
-        return qlmx_gemm_mfma_dispatch(mode, d, s, group, probs, second, nprob, K, N, act_dtype, (hipStream_t)stream);
+    if(math != QLMX_MATH_F32)
+        return qlmx_gemm_mfma_dispatch(mode, d, s, group, probs, second, nprob, K, N, act_dtype, (hipStream_t)stream, math == QLMX_MATH_MFMA_F16);
     QLMX_REQUIRE(!second, "%s: continued contractions need the MFMA path", who);
     if(mode == GEMM_NN && act_dtype == QLMX_ACT_F32 && N % 32 == 0 && group % 32 == 0 && ((uintptr_t)d & 15) == 0){
         /* every problem has a few rows only: stream the weights once (decode shape) */
@@ -61,7 +61,7 @@ extern "C" int qlmx_moe_gemm_tn_pair(const signed char *d, const float *s, int g
     QLMX_REQUIRE(first && second && nprob >= 0, "qlmx_moe_gemm_tn_pair: NULL problem list");
     for(int i = 0; i < nprob; i++)
         QLMX_REQUIRE(second[i].M == first[i].M, "qlmx_moe_gemm_tn_pair: problem %d has %d and %d rows", i, first[i].M, second[i].M);
-    if(act_dtype == QLMX_ACT_BF16 && math == QLMX_MATH_MFMA)
+    if(act_dtype == QLMX_ACT_BF16 && math != QLMX_MATH_F32)
         return gemm_entry("qlmx_moe_gemm_tn_pair", GEMM_TN, d, s, group, first, nprob, K, N, act_dtype, math, stream, second);
     int rc = gemm_entry("qlmx_moe_gemm_tn_pair", GEMM_TN, d, s, group, first, nprob, K, N, act_dtype, math, stream);
     if(rc) return rc;

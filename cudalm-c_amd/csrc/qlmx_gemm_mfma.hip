@@ -33,6 +33,7 @@
 int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second,
                             int nprob, int K, int N, hipStream_t st);
 int qlmx_gemm_nn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
+int qlmx_gemm_nn_h_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
 int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -392,7 +393,7 @@ static int launch_mfma(const signed char *d, const float *s, int group, const ql
 
 /* `second`: tn on bf16 activations only, the continuation of every problem's contraction (else NULL) */
 int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int group,
-                            const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second, int nprob, int K, int N, int act_dtype, hipStream_t st){
+                            const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second, int nprob, int K, int N, int act_dtype, hipStream_t st, bool f16){
     QLMX_REQUIRE(!second || (mode == GEMM_TN && act_dtype == QLMX_ACT_BF16), "mfma gemm: continued contractions exist for tn on bf16 activations only");
     /* shapes the tiling assumes; anything else must use QLMX_MATH_F32 */
     QLMX_REQUIRE(N % BN == 0, "mfma gemm: N=%d is not a multiple of %d (use QLMX_MATH_F32)", N, BN);
@@ -415,6 +416,7 @@ int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int 
     /* bf16 operands take the direct-to-LDS kernels; fp32 activations need the converting ones */
     if(mode == GEMM_TN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_tn_lds_launch(d, s, group, probs, second, nprob, K, N, st);
     if(mode == GEMM_NT && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nt_lds_launch(probs, nprob, K, N, st);
+    if(mode == GEMM_NN && act_dtype == QLMX_ACT_BF16 && f16) return qlmx_gemm_nn_h_launch(d, s, group, probs, nprob, K, N, st);
     if(mode == GEMM_NN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nn_lds_launch(d, s, group, probs, nprob, K, N, st);
     if(mode == GEMM_NN) return launch_mfma<GEMM_NN, 4, true>(d, s, group, probs, nprob, K, N, act_dtype, st);
     if(mode == GEMM_TN) return launch_mfma<GEMM_TN, 2, false>(d, s, group, probs, nprob, K, N, act_dtype, st);

@@ -138,6 +138,12 @@ int qlmx_servo(signed char *d, signed char *r, float *s,
 #define QLMX_ACT_BF16  1     /* activation operands are bf16 (high half of an fp32)  */
 #define QLMX_MATH_F32  0     /* fp32 FMA on the vector ALU                           */
 #define QLMX_MATH_MFMA 1     /* bf16 MFMA, fp32 accumulate                           */
+#define QLMX_MATH_MFMA_F16 2 /* as QLMX_MATH_MFMA, except that qlmx_moe_gemm_nn on bf16 activations runs on the fp16
+                              * matrix core: the activations are converted exactly (|x| in [2^-14, 65504]; smaller ones
+                              * with an absolute error below 3e-8), every weight s*digit is rounded once to fp16
+                              * (11 significant bits, full precision for 2.4e-7 <= |w| <= 255) and a product costs one
+                              * MFMA instead of the two of the bf16 hi + lo split. Relative L2 error against the fp32
+                              * result about 2e-4 (QLMX_MATH_MFMA: 3e-6), inside the 1e-3 bar for matmul outputs. */
 #define QLMX_MAX_PROBLEMS 1024   /* like MG_MAXP, cudalm.cu:3214 */
 
 typedef struct qlmx_gemm_prob {

@@ -153,6 +153,56 @@ def test_mfma_layer_shapes(q, orc, mode, K, N):
     assert err < TOL_MFMA, err
 
 
+# ------------------------------------------------------------------ forward on the fp16 matrix core
+@pytest.mark.parametrize("K,N,rows", [(768, 2048, None), (2048, 768, None), (256, 384, [300, 0, 64, 1, 129, 517, 193, 255]),
+                                      (32, 128, [5, 700]), (64, 256, [1, 65, 130, 200, 256, 257])])
+def test_mfma_f16_forward_vs_oracle(q, orc, K, N, rows):
+    """QLMX_MATH_MFMA_F16: bf16 activations converted exactly, weights rounded once to fp16, one MFMA per product.
+    Tolerance 1e-3 relative L2 against the oracle's fp32 GEMM on the rendered weights; the rounding of s*digit to
+    11 bits predicts about 2e-4. Every last-tile height, empty experts, single-step contractions."""
+    rows = rows or zipf_rows(1100, 4, 7)
+    got, want = run_case(q, orc, "nn", len(rows), rows, K, N, pkg.ACT_BF16, pkg.MATH_MFMA_F16, seed=4)
+    err = orc.relerr(got, want)
+    print("fp16 forward K=%d N=%d: relative L2 %.2e" % (K, N, err))
+    assert err < 1e-3, err
+    assert err < 4e-4, err          # observed 1.5e-4 .. 2.5e-4
+    # rows of empty experts and everything outside the written tiles stay as they were
+    off = np.concatenate([[0], np.cumsum(rows)]).astype(int)
+    assert got.size == off[-1] * N
+
+
+def test_mfma_f16_forward_range_edges(q, orc):
+    """Where fp16 would lose bits the kernel's 2^8 range shift keeps them: weights scaled down to 1e-6 (below fp16's
+    normal range unshifted) still meet the bar; activations far below fp16's normal range change nothing measurable;
+    other orientations given QLMX_MATH_MFMA_F16 run their bf16 kernels unchanged."""
+    import torch
+    E, K, N, rows = 2, 256, 256, [200, 90]
+    n = E * K * N
+    tab, nq, ng = make_spans([n], 128)
+    for wscale, ascale in ((1e-6, 1.0), (0.02, 1e-3), (30.0, 100.0)):
+        P = orc.normal(n, 31, 1, wscale)
+        d = np.zeros(n // 2, np.int8); r = np.zeros(n, np.int8); s = np.zeros(ng, f32)
+        orc.encode(P, d, r, s, tab, 128, 7, 1, ng)
+        orc.render(P, d, s, tab, 128, 1, 0, ng)
+        off = np.concatenate([[0], np.cumsum(rows)]).astype(int)
+        A = orc.bf16_round(orc.normal(int(off[-1]) * K, 31, 2, ascale))
+        A[:64] = orc.bf16_round(orc.normal(64, 31, 3, 1e-7))          # a few values that become fp16 subnormals
+        dA, dC = dev(A), torch.zeros(int(off[-1]) * N, device="cuda")
+        pa = to_bf16_bits(dA)
+        items = [(pa.data_ptr() + int(off[e]) * K * 2, None, dC.data_ptr() + int(off[e]) * N * 4, e * K * N, e * K * N // 128, rows[e], 0.0)
+                 for e in range(E)]
+        q.gemm_nn(dev(d), dev(s), 128, q.problems(items), E, K, N, pkg.ACT_BF16, pkg.MATH_MFMA_F16)
+        torch.cuda.synchronize()
+        want = np.zeros(int(off[-1]) * N, f32)
+        for e in range(E):
+            orc.gemm_nn(A[off[e] * K:], P[e * K * N:(e + 1) * K * N], want[off[e] * N:off[e + 1] * N], rows[e], K, N)
+        err = orc.relerr(dC.cpu().numpy(), want)
+        assert err < 1e-3, (wscale, ascale, err)
+    got, want = run_case(q, orc, "tn", 3, [70, 0, 132], 256, 128, pkg.ACT_BF16, pkg.MATH_MFMA_F16, seed=14)
+    got2, _ = run_case(q, orc, "tn", 3, [70, 0, 132], 256, 128, pkg.ACT_BF16, pkg.MATH_MFMA, seed=14)
+    assert np.array_equal(got, got2)
+
+
 def test_mfma_f32_acts_are_rounded_once(q, orc):
     """fp32 activations on the MFMA path are rounded to bf16 on load: equal to feeding pre-rounded ones."""
     import torch

@@ -21,6 +21,7 @@
  * matrix's own order with the 16-byte units xor-swizzled, read through ds_read_b64_tr_b16.
  */
 #include "qlmx_gemm.h"
+#include <type_traits>
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -50,24 +51,18 @@ template<int OFF> __device__ __forceinline__ i32x2 nh_tr(uint32_t addr){
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
     return v;
 }
-__device__ __forceinline__ void nh_wr128(uint32_t addr, i32x4 v){
-    asm volatile("ds_write_b128 %0, %1" :: "v"(addr), "v"(v) : "memory");
+template<int OFF> __device__ __forceinline__ void nh_wr128(uint32_t addr, i32x4 v){
+    asm volatile("ds_write_b128 %0, %1 offset:%2" :: "v"(addr), "v"(v), "n"(OFF) : "memory");
 }
-__device__ __forceinline__ int nh_gld4(const void *p){
-    int v;
-    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-    return v;
-}
-__device__ __forceinline__ i32x2 nh_gld8(const void *p){
-    i32x2 v;
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-    return v;
-}
-__device__ __forceinline__ i32x4 nh_gld16(const void *p){
-    i32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-    return v;
-}
+/* Global loads are ordinary loads here: this kernel has no load-to-LDS instruction, so the compiler's own wait
+ * counts are exact (it waits, with the right count, just before the first use of a loaded value, also when that
+ * use is in the next iteration of the loop) and a tile's loads can stay in flight for a step and a half. */
+typedef const __attribute__((address_space(1))) int   g_i32;
+typedef const __attribute__((address_space(1))) i32x2 g_i32x2;
+typedef const __attribute__((address_space(1))) i32x4 g_i32x4;
+__device__ __forceinline__ int   nh_gld4(const void *p){ return *(g_i32 *)p; }
+__device__ __forceinline__ i32x2 nh_gld8(const void *p){ return *(g_i32x2 *)p; }
+__device__ __forceinline__ i32x4 nh_gld16(const void *p){ return *(g_i32x4 *)p; }
 struct NhOps { i32x4 a[4]; i32x2 b[2][2]; };
 __device__ __forceinline__ void nh_wait_lds(NhOps &o){
     asm volatile("s_waitcnt lgkmcnt(0)"
@@ -139,24 +134,30 @@ __device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, int i
         return r;
     };
 
-    /* ---- operand read offsets ---- */
-    uint32_t ra[2][NI];                                  /* [k16 slice][row tile] activations, 128-bit */
+    /* ---- LDS addresses. Which of an operand's two buffers a step reads or writes is known at compile time (the
+     * loop below is unrolled by two), so the buffer, the k16 slice and the second half of a transposing read all
+     * go into the instructions' immediate offsets and the loop computes no LDS address at all. ---- */
+    uint32_t ra[2][NI];                                  /* [k16 slice][row tile] activations, 128-bit reads */
 #pragma unroll
     for(int i = 0; i < NI; i++){
         const int r = wi + i * 32 + fr, f = (r >> 2) & 3;
 #pragma unroll
-        for(int ks = 0; ks < 2; ks++) ra[ks][i] = (uint32_t)(r * 64 + (((ks * 2 + hf) ^ f) << 4));
+        for(int ks = 0; ks < 2; ks++) ra[ks][i] = lds_base + (uint32_t)(r * 64 + (((ks * 2 + hf) ^ f) << 4));
     }
-    uint32_t rb[2];                                      /* [column tile] weights, transposing reads; slice 1 is 16 rows further */
+    uint32_t rb[2];                                      /* [column tile] weights, transposing reads */
     {
         const int g16 = lane >> 4, s16 = lane & 15, v = s16 >> 2, q = s16 & 3, khalf = g16 >> 1, chalf = g16 & 1;
         const int row0 = khalf * 8 + v, swr = (row0 & 3) << 2;
 #pragma unroll
         for(int j = 0; j < 2; j++){
             const int col = wj + j * 32 + chalf * 16 + q * 4;
-            rb[j] = NH_B_OFF + (uint32_t)(row0 * 256 + (((col >> 3) ^ swr) << 4) + (col & 7) * 2);
+            rb[j] = lds_base + (uint32_t)(row0 * 256 + (((col >> 3) ^ swr) << 4) + (col & 7) * 2);
         }
     }
+    uint32_t wpa[NI];
+#pragma unroll
+    for(int h = 0; h < NI; h++) wpa[h] = lds_base + posA[h];
+    const uint32_t wp0 = lds_base + wr0 - NH_B_OFF, wp1 = lds_base + wr1 - NH_B_OFF;
 
     f32x16 acc[NI][2];
 #pragma unroll
@@ -164,65 +165,58 @@ __device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, int i
 #pragma unroll
         for(int j = 0; j < 2; j++) acc[i][j] = (f32x16)(0.0f);
 
-    /* ---- prologue: tile 0 into buffer 0, tile 1 into registers; all requests go out before the first wait ---- */
-    NhW wcur; i32x4 acur[NI];
+    /* ---- prologue: tile 0 into buffer 0, tile 1 into registers; all requests go out before the first use ---- */
+    NhW wA, wB; i32x4 aA[NI], aB[NI];
     {
         NhW w0 = load_w(0); i32x4 a0[NI];
 #pragma unroll
         for(int h = 0; h < NI; h++) a0[h] = load_a(0, h);
-        wcur = load_w(1);
+        wB = load_w(1);
 #pragma unroll
-        for(int h = 0; h < NI; h++) acur[h] = load_a(1, h);
-        /* tile 0 is in once only tile 1's 2 + NI loads are still out */
-        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(w0.d), "+v"(w0.s) : "n"(2 + NI) : "memory");
+        for(int h = 0; h < NI; h++) aB[h] = load_a(1, h);
 #pragma unroll
-        for(int h = 0; h < NI; h++) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a0[h]) : "n"(2 + NI) : "memory");
-#pragma unroll
-        for(int h = 0; h < NI; h++) nh_wr128(lds_base + posA[h], convert_a(a0[h]));
+        for(int h = 0; h < NI; h++) nh_wr128<0>(wpa[h], convert_a(a0[h]));
         const float sc = __int_as_float(w0.s) * NH_WSCALE;
-        nh_wr128(lds_base + wr0, dequant_unit(unit_digits(w0, 0), sc));
-        nh_wr128(lds_base + wr1, dequant_unit(unit_digits(w0, 1), sc));
-        /* tile 1 has arrived as well before the loop touches it */
-#pragma unroll
-        for(int h = 0; h < NI; h++) asm volatile("s_waitcnt vmcnt(0)" : "+v"(acur[h]) :: "memory");
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(wcur.d), "+v"(wcur.s) :: "memory");
+        nh_wr128<NH_B_OFF>(wp0, dequant_unit(unit_digits(w0, 0), sc));
+        nh_wr128<NH_B_OFF>(wp1, dequant_unit(unit_digits(w0, 1), sc));
     }
 
-    /* Main loop. A wavefront issues in order and an MFMA of this shape leaves room for about four vector-ALU
-     * instructions behind it, so everything else of a step is cut into small items that are dealt evenly into
-     * the gaps after the step's MFMAs (fences keep the compiler from gathering them again):
+    /* Main loop, two steps per iteration: step `st` of parity PAR reads buffers PAR, holds tile st+1 in the
+     * register set `cur` (loaded during step st-1) and loads tile st+2 into the set `nxt`; the two sets swap
+     * roles from step to step, so no loaded value is ever copied and a tile's loads stay in flight from the first
+     * items of step st until the conversions of step st+1 need them, more than a step later (the compiler places
+     * those waits, with exact counts: this kernel has no load-to-LDS instruction to confuse it).
+     * A wavefront issues in order and an MFMA of this shape leaves room for about four vector-ALU instructions
+     * behind it, so everything else of a step is cut into small items that are dealt evenly into the gaps after
+     * the step's MFMAs (fences keep the compiler from gathering them again):
      *   the loads of tile st+2 (weights, then the NI activation pieces),
      *   the conversion of tile st+1's activation pieces (two words per item) and their LDS writes,
      *   the dequantisation of tile st+1's weights (two weights per item) and their two LDS writes,
-     * all into the buffers that were read in step st-1. The loads are waited for at the end of the step, when
-     * they have long arrived: no asynchronously loaded register is carried round the loop before its wait. */
+     * the writes going to the buffers that were read in step st-1. */
     constexpr int SLOTS = NI * 4, ITEMS = 2 + NI + 2 * NI + 8 + 2;
-    for(int st = 0; st < steps; st++){
+    auto step = [&](auto PARC, int st, const NhW &wcur, const i32x4 (&acur)[NI], NhW &wnxt, i32x4 (&anxt)[NI]){
+        constexpr int PAR = decltype(PARC)::value;
+        constexpr int RA = PAR * NH_A_BYTES, RB = NH_B_OFF + PAR * NH_B_BYTES;                 /* read  */
+        constexpr int WA = (1 - PAR) * NH_A_BYTES, WB = NH_B_OFF + (1 - PAR) * NH_B_BYTES;     /* write */
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     /* own LDS writes of tile st are done */
         __builtin_amdgcn_s_barrier();
-
-        const uint32_t sa = lds_base + (uint32_t)(st & 1) * NH_A_BYTES;
-        const uint32_t sb = lds_base + (uint32_t)(st & 1) * NH_B_BYTES;
-        const uint32_t wa = lds_base + (uint32_t)((st + 1) & 1) * NH_A_BYTES;
-        const uint32_t wb = lds_base + (uint32_t)((st + 1) & 1) * NH_B_BYTES;
-        NhW wnext; i32x4 anext[NI];
         i32x4 ah[NI], wh[2];
         QxNibs dg[2];
         const float sc = __int_as_float(wcur.s) * NH_WSCALE;
         auto item = [&](int k){
-            if(k == 0)      wnext.d = nh_gld8(pw + tile_of(st + 2) * wstep);
-            else if(k == 1) wnext.s = nh_gld4(ps + tile_of(st + 2) * sstep);
-            else if(k < 2 + NI) anext[k - 2] = nh_gld16(srcA[k - 2] + tile_of(st + 2) * (NH_BK * 2));
+            if(k == 0)      wnxt.d = nh_gld8(pw + tile_of(st + 2) * wstep);
+            else if(k == 1) wnxt.s = nh_gld4(ps + tile_of(st + 2) * sstep);
+            else if(k < 2 + NI) anxt[k - 2] = nh_gld16(srcA[k - 2] + tile_of(st + 2) * (NH_BK * 2));
             else if(k < 2 + 3 * NI){
                 const int q = k - 2 - NI, h = q >> 1;
                 if((q & 1) == 0){ ah[h][0] = nh_bf16x2_to_f16x2(acur[h][0]); ah[h][1] = nh_bf16x2_to_f16x2(acur[h][1]); }
-                else { ah[h][2] = nh_bf16x2_to_f16x2(acur[h][2]); ah[h][3] = nh_bf16x2_to_f16x2(acur[h][3]); nh_wr128(wa + posA[h], ah[h]); }
+                else { ah[h][2] = nh_bf16x2_to_f16x2(acur[h][2]); ah[h][3] = nh_bf16x2_to_f16x2(acur[h][3]); nh_wr128<WA>(wpa[h], ah[h]); }
             } else if(k < 2 + 3 * NI + 8){
                 const int q = k - 2 - 3 * NI, r = q >> 2, j = q & 3;
                 if(q == 0){ dg[0] = qx_nibs(unit_digits(wcur, 0)); dg[1] = qx_nibs(unit_digits(wcur, 1)); }
                 wh[r][j] = nh_pk(sc * qx_nib16(dg[r], 2 * j), sc * qx_nib16(dg[r], 2 * j + 1));
             } else {
-                if(k - 2 - 3 * NI - 8 == 0) nh_wr128(wb + wr0, wh[0]); else nh_wr128(wb + wr1, wh[1]);
+                if(k - 2 - 3 * NI - 8 == 0) nh_wr128<WB>(wp0, wh[0]); else nh_wr128<WB>(wp1, wh[1]);
             }
         };
         NhOps o0, o1;
@@ -232,11 +226,11 @@ __device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, int i
         }
 #define NH_READ(O, KS)                                                                                    \
         _Pragma("unroll")                                                                                 \
-        for(int i = 0; i < NI; i++) O.a[i] = nh_rd128<0>(sa + ra[KS][i]);                                 \
+        for(int i = 0; i < NI; i++) O.a[i] = nh_rd128<RA>(ra[KS][i]);                                     \
         _Pragma("unroll")                                                                                 \
         for(int j = 0; j < 2; j++){                                                                       \
-            O.b[j][0] = nh_tr<KS * 16 * 256>(sb + rb[j]);                                                 \
-            O.b[j][1] = nh_tr<KS * 16 * 256 + 4 * 256>(sb + rb[j]);                                       \
+            O.b[j][0] = nh_tr<RB + KS * 16 * 256>(rb[j]);                                                 \
+            O.b[j][1] = nh_tr<RB + KS * 16 * 256 + 4 * 256>(rb[j]);                                       \
         }
 #define NH_MMA(O, BLOCK)                                                                                  \
         _Pragma("unroll")                                                                                 \
@@ -259,13 +253,14 @@ __device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, int i
         NH_MMA(o1, 1)
 #undef NH_READ
 #undef NH_MMA
-        /* tile st+2 has arrived */
-#pragma unroll
-        for(int h = 0; h < NI; h++) asm volatile("s_waitcnt vmcnt(0)" : "+v"(anext[h]) :: "memory");
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(wnext.d), "+v"(wnext.s) :: "memory");
-        wcur = wnext;
-#pragma unroll
-        for(int h = 0; h < NI; h++) acur[h] = anext[h];
+    };
+    {
+        int st = 0;
+        for(; st + 1 < steps; st += 2){
+            step(std::integral_constant<int, 0>(), st, wB, aB, wA, aA);
+            step(std::integral_constant<int, 1>(), st + 1, wA, aA, wB, aB);
+        }
+        if(st < steps) step(std::integral_constant<int, 0>(), st, wB, aB, wA, aA);
     }
 
     /* ---- epilogue: undo the range shift, then the lane holds column lane%32 of each 32x32 tile, four-row band lane/32 ---- */

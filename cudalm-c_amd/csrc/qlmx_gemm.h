@@ -193,7 +193,8 @@ typedef uint32_t DevUnit;                 /* prob:10 | tile row:6 | (8 spare) | 
 #define QLMX_MAX_UNITS 16384
 #define QX_CHAIN_SPINS (1 << 22)
 struct UnitUpload { DevProb *hprob; DevUnit *hunit; const DevProb *dprob; const DevUnit *dunit; int *flags; unsigned *status; };
-int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot);                         /* tables to fill (pinned, read by the kernel); waits for the slot's last user */
+int qlmx_unit_slot(int nprob, UnitUpload *out, int *slot);                         /* tables to fill (host staging) and where the kernel will read them; waits for the slot's last user */
+void qlmx_unit_commit(const UnitUpload *u, int nprob, int nunits);                 /* staging copy -> the slot the kernel reads; before the launch */
 int qlmx_unit_done(int slot, hipStream_t stream);                                  /* after the kernel launch */
 int qlmx_chain_reserve(int nflags, int *first, unsigned *epoch);                   /* flags for one launch */
 /* one-shot switches of the time-out tests (qlmx_test_force_wait_timeout): true once after being armed */

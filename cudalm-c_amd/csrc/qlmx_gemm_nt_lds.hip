@@ -319,6 +319,7 @@ int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N
                 a.wait_epoch = a.epoch; a.wait_limit = QX_CHAIN_SPINS;
                 if(nflags && qlmx_test_take_forced_timeout(2)){ a.wait_epoch = a.epoch ^ 0x00A5A5A5u; a.wait_limit = 1; }
                 for(int p = 0; p < n; p++) uu.hprob[p].flag0 += first;
+                qlmx_unit_commit(&uu, n, nent);
                 hipLaunchKernelGGL(k_gemm_nt_lds, dim3(grid), dim3(256), 0, st, a);
                 QLMX_LAUNCH_CHECK("grouped gemm nt (scheduled) launch");
                 return qlmx_unit_done(uslot, st);

@@ -72,6 +72,9 @@ SIGNATURES = {
     "qlmx_moe_gemm_tn": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_tn_pair": (c_i, [c_vp, c_vp, c_i, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_nn_swiglu": (c_i, [c_vp, c_vp, c_i, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_moe_gemm_nn_gather": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_vp, c_vp]),
+    "qlmx_moe_gemm_nn_scatter": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_vp, c_vp, c_vp]),
+    "qlmx_moe_gemm_tn_pair_scatter": (c_i, [c_vp, c_vp, c_i, c_vp, c_vp, c_i, c_i, c_i, c_vp, c_vp]),
     "qlmx_moe_gemm_nt": (c_i, [c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_decode_forward": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_decode_forward_noalloc": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
@@ -161,6 +164,15 @@ class Qlmx:
 
     def gemm_nn_swiglu(self, d, s, group, gate, up, nprob, K, N, act=ACT_F32, math=MATH_F32, stream=None):
         self.call("qlmx_moe_gemm_nn_swiglu", d, s, group, C.addressof(gate), C.addressof(up), nprob, K, N, act, math, stream)
+
+    def gemm_nn_gather(self, d, s, group, probs, nprob, K, N, x_bf16, stream=None):
+        self.call("qlmx_moe_gemm_nn_gather", d, s, group, C.addressof(probs), nprob, K, N, x_bf16, stream)
+
+    def gemm_nn_scatter(self, d, s, group, probs, nprob, K, N, out, gate, stream=None):
+        self.call("qlmx_moe_gemm_nn_scatter", d, s, group, C.addressof(probs), nprob, K, N, out, gate, stream)
+
+    def gemm_tn_pair_scatter(self, d, s, group, first, second, nprob, K, N, dst, stream=None):
+        self.call("qlmx_moe_gemm_tn_pair_scatter", d, s, group, C.addressof(first), C.addressof(second), nprob, K, N, dst, stream)
 
     def gemm_nt(self, probs, nprob, K, N, act=ACT_F32, math=MATH_F32, stream=None):
         self.call("qlmx_moe_gemm_nt", C.addressof(probs), nprob, K, N, act, math, stream)

@@ -180,6 +180,32 @@ __device__ __forceinline__ void qx_store_tiles(const qx_f32x16 (&acc)[NI][NJ], f
     else                           qx_store_tiles_edge<NI, NJ, SYS>(acc, (qx_gfloat *)c, row, rows, ld, accumulate);
 }
 
+/* The NI x 2 accumulator tiles of one wavefront added to INDEXED output rows (the gated scatter and the
+ * scatter-add of the MoE glue, cudalm.cu:2541-2545, 2564-2567, as a GEMM epilogue): row r of the problem goes to
+ * row idx[r] of `out`, out = out + gate[idx[r]] * y (multiply, then add, as k_scatter_gate does), or out += y when
+ * gate is NULL (k_scatter_add4); idx[r] < 0 drops the row. `row` is the lane's first row, `col` its column in
+ * tile (., 0); tile (., 1) lies 32 columns further. 32 lanes cover 128 contiguous bytes of an output row. */
+template<int NI>
+__device__ __forceinline__ void qx_scatter_tiles(const qx_f32x16 (&acc)[NI][2], const int *idx, const float *gate, float *out,
+                                                 int row, int rows, size_t ld, int col){
+#pragma unroll
+    for(int i = 0; i < NI; i++)
+#pragma unroll
+        for(int e = 0; e < 16; e++){
+            const int r = row + i * 32 + (e >> 2) * 8 + (e & 3);
+            if(r < rows){
+                const int tok = idx[r];
+                if(tok >= 0){
+                    float *o = out + (size_t)tok * ld + col;
+                    if(gate){
+                        const float g = gate[tok];
+                        o[0] = o[0] + g * acc[i][0][e]; o[32] = o[32] + g * acc[i][1][e];
+                    } else { o[0] += acc[i][0][e]; o[32] += acc[i][1][e]; }
+                }
+            }
+        }
+}
+
 /* ---- scheduled launches: instead of deriving its tile from its index, a workgroup reads an entry of
  * a table the host has laid out -- which problem, which row of output tiles, which slice of the
  * contraction; the workgroups that share an entry take one column tile each, which keeps the table

@@ -112,6 +112,63 @@ extern "C" int qlmx_moe_gemm_nn_swiglu(const signed char *d, const float *s, int
     return rc;
 }
 
+/* ---- the row moves of the MoE glue folded into the GEMMs (fp16 forward kernel, bf16 input-gradient kernel) ---- */
+int qlmx_gemm_nn_h_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N,
+                          int io, const void *xsrc, float *out, const float *gate, hipStream_t st);
+int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second,
+                            int nprob, int K, int N, float *out, const float *gate, hipStream_t st);
+
+static int rows_entry_checks(const char *who, const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs,
+                             const qlmx_gemm_prob *second, int nprob, int K, int N, int bk, bool idx_in_a){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(d && s && probs && nprob >= 0 && K > 0 && N > 0, "%s: NULL or empty argument", who);
+    QLMX_REQUIRE(((uintptr_t)d & 15) == 0, "%s: digit array is not 16-byte aligned", who);
+    QLMX_REQUIRE(N % 128 == 0 && K % bk == 0, "%s: N=%d must be a multiple of 128 and K=%d of %d", who, N, K, bk);
+    QLMX_REQUIRE(group >= bk && group <= 256 && (group & (group - 1)) == 0, "%s: group %d must be a power of two in [%d, 256]", who, group, bk);
+    for(int i = 0; i < nprob; i++){
+        if(probs[i].M == 0) continue;
+        QLMX_REQUIRE(probs[i].A && probs[i].C, "%s: problem %d has a NULL pointer", who, i);
+        QLMX_REQUIRE(((uintptr_t)(idx_in_a ? (const void *)probs[i].C : probs[i].A) & 15) == 0 && ((uintptr_t)(idx_in_a ? probs[i].A : (const void *)probs[i].C) & 3) == 0,
+                     "%s: problem %d operand alignment (rows 16 bytes, index list 4)", who, i);
+        QLMX_REQUIRE(probs[i].wq % (unsigned long long)group == 0 && (probs[i].wq & 31ULL) == 0, "%s: problem %d weight offset alignment", who, i);
+        if(second){
+            QLMX_REQUIRE(second[i].M == probs[i].M && second[i].A && ((uintptr_t)second[i].A & 15) == 0, "%s: problem %d second half (rows, pointer, alignment)", who, i);
+            QLMX_REQUIRE(second[i].wq % (unsigned long long)group == 0 && (second[i].wq & 31ULL) == 0, "%s: problem %d second weight offset alignment", who, i);
+        }
+    }
+    return QLMX_OK;
+}
+
+/* k_gather + mg_ab (cudalm.cu:4209-4213) in one launch: problem i computes C = x[idx_i[0..M), :] . W, where
+ * idx_i = (const int *)probs[i].A lists the rows of the bf16 token matrix x [tokens, K] (an entry < 0 reads as a row of
+ * zeros). fp16 matrix core (QLMX_MATH_MFMA_F16 arithmetic). */
+extern "C" int qlmx_moe_gemm_nn_gather(const signed char *d, const float *s, int group,
+                                       const qlmx_gemm_prob *probs, int nprob, int K, int N, const void *x_bf16, void *stream){
+    int rc = rows_entry_checks("qlmx_moe_gemm_nn_gather", d, s, group, probs, nullptr, nprob, K, N, 32, true); if(rc) return rc;
+    QLMX_REQUIRE(x_bf16 && ((uintptr_t)x_bf16 & 15) == 0 && K % 8 == 0, "qlmx_moe_gemm_nn_gather: token matrix must be given and 16-byte aligned");
+    return qlmx_gemm_nn_h_launch(d, s, group, probs, nprob, K, N, 1, x_bf16, nullptr, nullptr, (hipStream_t)stream);
+}
+/* mg_ab + k_scatter_gate (cudalm.cu:4224-4227) in one launch: problem i computes y = A . W and adds it to indexed rows,
+ * out[idx_i[r], :] = out[idx_i[r], :] + gate[idx_i[r]] * y[r, :], idx_i = (const int *)probs[i].C (entries < 0 are dropped;
+ * gate NULL adds y itself). No output row may be named twice in one call (true of one pass of the MoE layer). */
+extern "C" int qlmx_moe_gemm_nn_scatter(const signed char *d, const float *s, int group,
+                                        const qlmx_gemm_prob *probs, int nprob, int K, int N,
+                                        float *out, const float *gate, void *stream){
+    int rc = rows_entry_checks("qlmx_moe_gemm_nn_scatter", d, s, group, probs, nullptr, nprob, K, N, 32, false); if(rc) return rc;
+    QLMX_REQUIRE(out, "qlmx_moe_gemm_nn_scatter: NULL output");
+    return qlmx_gemm_nn_h_launch(d, s, group, probs, nprob, K, N, 2, nullptr, out, gate, (hipStream_t)stream);
+}
+/* the paired mg_abt_b calls + k_scatter_add4 (cudalm.cu:4365-4367) in one launch: as qlmx_moe_gemm_tn_pair on bf16
+ * activations with MFMA math, the sum of both products added to indexed rows, dst[idx_i[r], :] += y[r, :],
+ * idx_i = (const int *)first[i].C. */
+extern "C" int qlmx_moe_gemm_tn_pair_scatter(const signed char *d, const float *s, int group,
+                                             const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int K, int N,
+                                             float *dst, void *stream){
+    int rc = rows_entry_checks("qlmx_moe_gemm_tn_pair_scatter", d, s, group, first, second, nprob, K, N, 64, false); if(rc) return rc;
+    QLMX_REQUIRE(dst && second && nprob * 2 <= QLMX_MAX_PROBLEMS, "qlmx_moe_gemm_tn_pair_scatter: NULL output or too many problems");
+    return qlmx_gemm_tn_lds_launch(d, s, group, first, second, nprob, K, N, dst, nullptr, (hipStream_t)stream);
+}
+
 /* mg_atb + mg_flush (cudalm.cu:3254-3256) */
 extern "C" int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs, int nprob, int K, int N,
                                 int act_dtype, int math, void *stream){

@@ -39,7 +39,20 @@ typedef int      i32x4 __attribute__((ext_vector_type(4)));
 #define NH_WSCALE 4096.0f                       /* 16 (the digits come as digit/16) * 2^8 (range shift) */
 #define NH_UNSCALE (1.0f / 256.0f)
 
-struct NhArgs { const DevProb *pr; int nprob, ntiles; const signed char *d; const float *s; int gshift; int K, N; };
+/* Row plumbing of a launch (the MoE glue folded into the GEMM):
+ *   NH_PLAIN    A and C of a problem are its own row-major buffers;
+ *   NH_GATHER   k_gather in front (cudalm.cu:2536-2539, 4211): a problem's A field points at its row indices
+ *               (const int *), row r of the problem is row idx[r] of `xsrc` (bf16 [tokens, K]), zeros where idx[r] < 0;
+ *   NH_SCATTER  k_scatter_gate / k_scatter_add4 behind (cudalm.cu:2541-2545, 2564-2567, 4227): a problem's C field
+ *               points at its row indices, out[idx[r], :] = out[idx[r], :] + gate[idx[r]] * y[r, :] (gate NULL: + y[r, :]),
+ *               rows with idx[r] < 0 dropped. Within one launch every output row must be named at most once. */
+enum { NH_PLAIN = 0, NH_GATHER = 1, NH_SCATTER = 2 };
+struct NhArgs { const DevProb *pr; int nprob, ntiles; const signed char *d; const float *s; int gshift; int K, N;
+                const char *xsrc; float *out; const float *gate; };
+
+/* a row of zeros as long as the longest contraction a gathering launch accepts: what a dropped row reads */
+#define NH_ZERO_BYTES 32768
+static __device__ __align__(16) unsigned char nh_zero_row[NH_ZERO_BYTES];
 
 template<int OFF> __device__ __forceinline__ i32x4 nh_rd128(uint32_t addr){
     i32x4 v;
@@ -87,7 +100,7 @@ struct NhW { i32x2 d; int s; };
 
 /* One output tile of NI*64 rows (NI = 4: the full 256; the last tile of a problem takes the smallest NI that
  * holds its rows). */
-template<int NI>
+template<int NI, int IO>
 __device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, int i0, int j0, unsigned char *lds){
     const int rows = P.M;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -102,7 +115,10 @@ __device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, int i
     for(int h = 0; h < NI; h++){
         const int p = h * 256 + tid, r = p >> 2, ko = (p & 3) ^ ((r >> 2) & 3);
         const int rr = (i0 + r < rows) ? i0 + r : rows - 1;               /* clamp: feeds unstored rows only */
-        srcA[h] = (const char *)P.A + ((size_t)rr * a.K + ko * 8) * 2;
+        if(IO == NH_GATHER){
+            const int tok = ((const int *)P.A)[rr];
+            srcA[h] = (tok >= 0 ? a.xsrc + (size_t)tok * a.K * 2 : (const char *)nh_zero_row) + ko * 16;
+        } else srcA[h] = (const char *)P.A + ((size_t)rr * a.K + ko * 8) * 2;
         posA[h] = (uint32_t)p * 16;
     }
     /* ---- weights: thread = (contraction row kr, columns oc*16 .. +15): one 8-byte load of digits and one scale
@@ -269,9 +285,11 @@ __device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, int i
 #pragma unroll
         for(int j = 0; j < 2; j++) acc[i][j] = acc[i][j] * NH_UNSCALE;
     const int row = i0 + wi + hf * 4;
-    qx_store_tiles<NI, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, false);
+    if(IO == NH_SCATTER) qx_scatter_tiles<NI>(acc, (const int *)P.C, a.gate, a.out, row, rows, (size_t)a.N, j0 + wj + fr);
+    else qx_store_tiles<NI, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, false);
 }
 
+template<int IO>
 __global__ void __launch_bounds__(256, 2) k_gemm_nn_h(NhArgs a){
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * NH_A_BYTES + 2 * NH_B_BYTES];
     const int t = qx_xcd_tile(blockIdx.x, gridDim.x);
@@ -280,22 +298,28 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nn_h(NhArgs a){
     const int lt = t - P.tile0;
     const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
     const int i0 = ti * NH_BM, j0 = tj * NH_BN, left = P.M - i0;
-    if(left > 192)      nh_tile<4>(a, P, i0, j0, lds);
-    else if(left > 128) nh_tile<3>(a, P, i0, j0, lds);
-    else if(left > 64)  nh_tile<2>(a, P, i0, j0, lds);
-    else                nh_tile<1>(a, P, i0, j0, lds);
+    if(left > 192)      nh_tile<4, IO>(a, P, i0, j0, lds);
+    else if(left > 128) nh_tile<3, IO>(a, P, i0, j0, lds);
+    else if(left > 64)  nh_tile<2, IO>(a, P, i0, j0, lds);
+    else                nh_tile<1, IO>(a, P, i0, j0, lds);
 }
 
-/* bf16 activations only; N % 128 == 0, K % 32 == 0, group a power of two >= 32 (checked by the caller) */
+/* bf16 activations only; N % 128 == 0, K % 32 == 0, group a power of two >= 32 (checked by the caller).
+ * io = NH_GATHER: xsrc is the bf16 token matrix and the problems' A fields are row-index lists;
+ * io = NH_SCATTER: out (and gate, may be NULL) is the destination and the problems' C fields are row-index lists. */
 int qlmx_gemm_nn_h_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob,
-                          int K, int N, hipStream_t st){
+                          int K, int N, int io, const void *xsrc, float *out, const float *gate, hipStream_t st){
+    QLMX_REQUIRE(io != NH_GATHER || (size_t)K * 2 <= NH_ZERO_BYTES, "grouped gemm nn with gather: K=%d exceeds %d", K, NH_ZERO_BYTES / 2);
     ProbUpload up; int slot;
     int rc = qlmx_upload_problems(probs, nprob, GEMM_NN, K, N, NH_BM, NH_BN, st, &up, &slot); if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;
     NhArgs a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.d = d; a.s = s; a.K = K; a.N = N;
+    a.xsrc = (const char *)xsrc; a.out = out; a.gate = gate;
     a.gshift = 0; while((1 << a.gshift) < group) a.gshift++;
     const int grid = (up.ntiles + 7) / 8 * 8;
-    hipLaunchKernelGGL(k_gemm_nn_h, dim3(grid), dim3(256), 0, st, a);
+    if(io == NH_GATHER)       hipLaunchKernelGGL(k_gemm_nn_h<NH_GATHER>,  dim3(grid), dim3(256), 0, st, a);
+    else if(io == NH_SCATTER) hipLaunchKernelGGL(k_gemm_nn_h<NH_SCATTER>, dim3(grid), dim3(256), 0, st, a);
+    else                      hipLaunchKernelGGL(k_gemm_nn_h<NH_PLAIN>,   dim3(grid), dim3(256), 0, st, a);
     QLMX_LAUNCH_CHECK("grouped gemm nn (fp16 matrix core) launch");
     return qlmx_upload_done(slot, st);
 }

@@ -187,6 +187,25 @@ int qlmx_moe_gemm_tn_pair(const signed char *d, const float *s, int group,
 int qlmx_moe_gemm_nn_swiglu(const signed char *d, const float *s, int group,
                             const qlmx_gemm_prob *gate_host, const qlmx_gemm_prob *up_host, int nprob,
                             int K, int N, int act_dtype, int math, void *stream);
+/* The row moves of the MoE layer folded into the expert GEMMs, so that the permuted copies never exist in memory
+ * (cudalm.cu:4209-4213 gather + mg_ab; 4224-4227 mg_ab + k_scatter_gate; 4365-4367 paired mg_abt_b + k_scatter_add4).
+ * bf16 activations, matrix-core math (fp16 forward as QLMX_MATH_MFMA_F16, bf16 input gradient as QLMX_MATH_MFMA),
+ * N % 128 == 0, K % 32 == 0 (64 for the input gradient), group a power of two >= that. An index list is int32 in
+ * device memory, entry r of problem i naming a token row; an entry < 0 reads as zeros (gather) or is dropped
+ * (scatter). Moves are exact: results equal the separate gather / GEMM / scatter kernels bit for bit.
+ *   gather:  probs[i].A = index list; C[r, :] = x[idx[r], :] . W                     x: bf16 [tokens, K]
+ *   scatter: probs[i].C = index list; out[idx[r], :] = out[idx[r], :] + gate[idx[r]] * (A . W)[r, :]   (gate NULL: + (A . W)[r, :])
+ *   tn_pair_scatter: first[i].C = index list; dst[idx[r], :] += (first.A . W1^T + second.A . W3^T)[r, :]
+ * A scatter call must not name an output row twice (one pass of the layer never does); calls on one stream are
+ * ordered, so the passes of a layer add up in pass order as in the reference. */
+int qlmx_moe_gemm_nn_gather(const signed char *d, const float *s, int group,
+                            const qlmx_gemm_prob *probs_host, int nprob, int K, int N, const void *x_bf16, void *stream);
+int qlmx_moe_gemm_nn_scatter(const signed char *d, const float *s, int group,
+                             const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
+                             float *out, const float *gate, void *stream);
+int qlmx_moe_gemm_tn_pair_scatter(const signed char *d, const float *s, int group,
+                                  const qlmx_gemm_prob *first_host, const qlmx_gemm_prob *second_host, int nprob, int K, int N,
+                                  float *dst, void *stream);
 /* nt: no weight operand; both inputs are activations, fp32 result. beta = 1 reproduces the
  * reference's accumulation into a zeroed G; beta = 0 saves the read when G is known to be fresh. */
 int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs_host, int nprob, int K, int N,

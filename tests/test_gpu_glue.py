@@ -286,6 +286,76 @@ class GpuLayer:
             q.moe_scatter_add(self.dXp, prm, dx, N, D)
 
 
+def _perm_case(orc, N, E, seed, drop=()):
+    """one pass: tokens assigned to experts at random, stable counting sort, a few rows dropped (index -1)"""
+    rng = np.random.default_rng(seed)
+    asn = rng.integers(0, E, N).astype(np.int32)
+    perm = np.argsort(asn, kind="stable").astype(np.int32)
+    cnt = np.bincount(asn, minlength=E)
+    off = np.concatenate([[0], np.cumsum(cnt)]).astype(int)
+    for j in drop:
+        perm[j] = -1
+    return perm, off
+
+
+@pytest.mark.parametrize("N,E,D,F", [(700, 5, 256, 384), (1500, 8, 768, 2048)])
+def test_fused_row_moves_equal_the_separate_kernels(q, orc, N, E, D, F):
+    """qlmx_moe_gemm_nn_gather == gather + GEMM, qlmx_moe_gemm_nn_scatter == GEMM + gated scatter,
+    qlmx_moe_gemm_tn_pair_scatter == paired input-gradient GEMM + scatter-add: bit for bit (pure moves around the
+    same arithmetic), with dropped rows, empty experts and every last-tile height; the separate path is itself
+    checked against the oracle in the layer tests below."""
+    import torch
+    d, s, P, n = encode_layer(orc, 70 + N, E, D, F)
+    dd, ds = dev(d), dev(s)
+    perm, off = _perm_case(orc, N, E, N, drop=(3, N // 2, N - 1))
+    dperm = dev(perm)
+    x = orc.bf16_round(orc.normal(N * D, 71, 1))
+    dx = dev(x)
+    xb = zeros(N * D, torch.int16)
+    q.moe_gather(dx, dev(np.arange(N, dtype=np.int32)), xb, N, D, pkg.ACT_BF16)        # the token matrix as bf16, once
+    rows = [int(off[e + 1] - off[e]) for e in range(E)]
+
+    def probs(A, a_esz, a_cols, C, c_cols, wbase, idx_a=False, idx_c=False, beta=0.0):
+        items = []
+        for e in range(E):
+            a = dperm.data_ptr() + int(off[e]) * 4 if idx_a else A.data_ptr() + int(off[e]) * a_cols * a_esz
+            c = dperm.data_ptr() + int(off[e]) * 4 if idx_c else C.data_ptr() + int(off[e]) * c_cols * 4
+            items.append((a, None, c, wbase + e * D * F, (wbase + e * D * F) // 128, rows[e], beta))
+        return q.problems(items)
+
+    # (a) gather in front of w1
+    Xp = zeros(N * D, torch.int16)
+    q.moe_gather(dx, dperm, Xp, N, D, pkg.ACT_BF16)
+    g_sep, g_fus = zeros(N * F), zeros(N * F)
+    q.gemm_nn(dd, ds, 128, probs(Xp, 2, D, g_sep, F, 0), E, D, F, pkg.ACT_BF16, pkg.MATH_MFMA_F16)
+    q.gemm_nn_gather(dd, ds, 128, probs(None, 0, 0, g_fus, F, 0, idx_a=True), E, D, F, xb)
+    torch.cuda.synchronize()
+    assert torch.equal(g_sep, g_fus)
+    # (b) gated scatter behind w2
+    ap = zeros(N * F, torch.int16)
+    q.moe_gather(dev(orc.bf16_round(orc.normal(N * F, 71, 2))), dev(np.arange(N, dtype=np.int32)), ap, N, F, pkg.ACT_BF16)
+    gate = dev(orc.uniform(N, 71, 3, 0.1, 0.6))
+    res = orc.normal(N * D, 71, 4)
+    yp, o_sep, o_fus = zeros(N * D), dev(res), dev(res)
+    q.gemm_nn(dd, ds, 128, probs(ap, 2, F, yp, D, 2 * n), E, F, D, pkg.ACT_BF16, pkg.MATH_MFMA_F16)
+    q.moe_scatter_gate(yp, dperm, gate, o_sep, N, D)
+    q.gemm_nn_scatter(dd, ds, 128, probs(ap, 2, F, None, 0, 2 * n, idx_c=True), E, F, D, o_fus, gate)
+    torch.cuda.synchronize()
+    assert torch.equal(o_sep, o_fus)
+    assert not torch.equal(o_fus, dev(res))
+    # (c) scatter-add behind the paired input gradient
+    dgp, dup = zeros(N * F, torch.int16), zeros(N * F, torch.int16)
+    ident = dev(np.arange(N, dtype=np.int32))
+    q.moe_gather(dev(orc.bf16_round(orc.normal(N * F, 71, 5))), ident, dgp, N, F, pkg.ACT_BF16)
+    q.moe_gather(dev(orc.bf16_round(orc.normal(N * F, 71, 6))), ident, dup, N, F, pkg.ACT_BF16)
+    dXp, x_sep, x_fus = zeros(N * D), dev(res), dev(res)
+    q.gemm_tn_pair(dd, ds, 128, probs(dgp, 2, F, dXp, D, 0), probs(dup, 2, F, dXp, D, n), E, F, D, pkg.ACT_BF16, pkg.MATH_MFMA)
+    q.moe_scatter_add(dXp, dperm, x_sep, N, D)
+    q.gemm_tn_pair_scatter(dd, ds, 128, probs(dgp, 2, F, None, 0, 0, idx_c=True), probs(dup, 2, F, None, 0, n, idx_c=True), E, F, D, x_fus)
+    torch.cuda.synchronize()
+    assert torch.equal(x_sep, x_fus)
+
+
 @pytest.mark.parametrize("math,N,E,D,F,K", [("f32", 96, 4, 128, 256, 2), ("f32", 300, 8, 256, 384, 2),
                                             ("mfma", 512, 4, 256, 384, 2), ("mfma", 1024, 8, 768, 2048, 2)])
 def test_layer_forward_backward_vs_oracle(q, orc, math, N, E, D, F, K):

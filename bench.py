@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=30)
-    ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train", "train5", "c5", "codec", "glue", "copy"])
+    ap.add_argument("--workload", default="all", choices=["all", "adamw", "decode", "train", "train5", "c5", "layer", "codec", "glue", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--fwd-math", default="f16", choices=["f16", "bf16x2"],
                     help="train, c5: forward GEMMs on the fp16 matrix core (one MFMA per product, 2e-4 relative L2) or as bf16 hi+lo (two, 3e-6)")
@@ -180,6 +180,150 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
                      "note": "algorithmic flops only; forward math: " + ("bf16 hi+lo weight split, two MFMAs per product" if args.fwd_math == "bf16x2" else
                              "fp16 matrix core, bf16 activations converted exactly, weights rounded once to fp16 (2e-4 relative L2), one MFMA per product")},
     }
+
+
+# --------------------------------------------------------------------------------------------- layer
+def bench_layer(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2):
+    """One whole MoE expert layer at config 3's shape, forward + backward with the recomputed forward (stash off), router
+    outputs given, grouping on the device. Three ways:
+      separate  the reference's call order pass by pass (moe_forward / moe_backward, cudalm.cu:4193-4228, 4299-4371),
+                every glue step a kernel of its own;
+      fused     the same passes with the glue folded into the GEMMs (gather -> w1|w3 -> SwiGLU, w2 -> gated scatter,
+                dgrad w2 -> SwiGLU gradient, paired dgrad -> scatter-add);
+      merged    all K passes as one expert-grouped list of K*N rows (the reference's merged top-K, cudalm.cu:3532-3561,
+                4048-4110): every GEMM once per layer, the passes combined per token in pass order, glue folded in
+                where one launch may still name a token once.
+    What stays a kernel of its own when fused: the token matrix to bf16 once, the gather that feeds the weight gradient,
+    the gate gradient and (merged) the two combines."""
+    import numpy as np
+    from cudalm_c_amd.binding import ACT_BF16, MATH_MFMA, MATH_MFMA_F16
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev); g.manual_seed(0)
+    N, K, group = tokens, topk, 128
+    nw = E * D * F
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def packed():
+        b = torch.randint(0, 256, (nw // 2,), dtype=torch.int16, device=dev, generator=g).to(torch.uint8)
+        lo = b & 15; hi = b >> 4
+        lo = torch.where(lo == 8, torch.zeros_like(lo), lo); hi = torch.where(hi == 8, torch.zeros_like(hi), hi)
+        return (lo | (hi << 4)).view(torch.int8)
+    d = torch.cat([packed(), packed(), packed()])
+    s = (0.02 * 3 / 7) * (0.5 + torch.rand(3 * nw // group, device=dev, generator=g))
+    # Zipf(1.1) routing without replacement, pass-major assignment, gates U(0.1, 0.6)
+    logp = -1.1 * np.log(np.arange(E) + 1.0)
+    keys = logp[None, :] + np.random.default_rng(0).gumbel(size=(N, E))
+    top = np.argsort(-keys, axis=1)[:, :K]
+    assign = torch.from_numpy(np.ascontiguousarray(top.T).astype(np.int32).reshape(-1)).to(dev)
+    gate = 0.1 + 0.5 * torch.rand(K * N, device=dev, generator=g)
+    x = torch.randn(N * D, device=dev, generator=g).to(torch.bfloat16).float()
+    dout = torch.randn(N * D, device=dev, generator=g).to(torch.bfloat16).float()
+    bf = torch.bfloat16
+    KN = K * N
+    xb = torch.empty(N * D, dtype=bf, device=dev)
+    Xp, ap = torch.empty(KN * D, dtype=bf, device=dev), torch.empty(KN * F, dtype=bf, device=dev)
+    gp, up, yp = torch.empty(KN * F, device=dev), torch.empty(KN * F, device=dev), torch.empty(KN * D, device=dev)
+    dyp, dgp, dup = torch.empty(KN * D, dtype=bf, device=dev), torch.empty(KN * F, dtype=bf, device=dev), torch.empty(KN * F, dtype=bf, device=dev)
+    dap, dXp = torch.empty(KN * F, device=dev), torch.empty(KN * D, device=dev)
+    out, dx, dgate = torch.zeros(N * D, device=dev), torch.zeros(N * D, device=dev), torch.zeros(KN, device=dev)
+    G = torch.zeros(3 * nw, device=dev)
+    ident = torch.arange(N, dtype=torch.int32, device=dev)
+    P = q.problems
+
+    class Lists:
+        """the grouped lists of one way of running the layer: K lists of N rows, or one of K*N"""
+        def __init__(self, merged):
+            self.R, self.n = (KN, 1) if merged else (N, K)
+            self.perm = torch.empty(KN, dtype=torch.int32, device=dev); self.off = torch.empty(self.n * (E + 1), dtype=torch.int32, device=dev)
+            ws = torch.empty(q.moe_perm_workspace(self.R, E, self.n), dtype=torch.uint8, device=dev)
+            q.moe_perm(assign, self.R, E, self.n, self.perm, self.off, ws, stream)
+            self.offh = self.off.cpu().numpy().reshape(self.n, E + 1)
+            self.tok, self.inv = self.perm, None
+            if merged:
+                self.tok, self.inv = torch.empty(KN, dtype=torch.int32, device=dev), torch.empty(KN, dtype=torch.int32, device=dev)
+                q.moe_merge_rows(self.perm, N, K, self.tok, self.inv, stream)
+            self.T = [self.tables(k) for k in range(self.n)]
+
+        def probs(self, k, A, a_cols, C, c_cols, wbase, B=None, b_cols=0, beta=0.0, out_expert=False, idx_a=False, idx_c=False):
+            o = self.offh[k]; items = []
+            for e in range(E):
+                ne, oe = int(o[e + 1] - o[e]), int(o[e])
+                a = self.tok.data_ptr() + (k * self.R + oe) * 4 if idx_a else A.data_ptr() + oe * a_cols * 2
+                b = None if B is None else B.data_ptr() + oe * b_cols * 2
+                if idx_c:       c = self.tok.data_ptr() + (k * self.R + oe) * 4
+                elif C is None: c = None
+                else:           c = C.data_ptr() + ((wbase + e * D * F) * 4 if out_expert else oe * c_cols * 4)
+                items.append((a, b, c, wbase + e * D * F, (wbase + e * D * F) // group, ne, beta))
+            return items
+
+        def tables(self, k):
+            pr = self.probs
+            return dict(
+                w13=P(pr(k, Xp, D, gp, F, 0) + pr(k, Xp, D, up, F, nw)),
+                w1=P(pr(k, Xp, D, gp, F, 0)), w3=P(pr(k, Xp, D, up, F, nw, B=ap, b_cols=F)),
+                w1g=P(pr(k, None, 0, None, F, 0, idx_a=True)), w3o=P(pr(k, Xp, D, None, F, nw, B=ap, b_cols=F)),
+                w2=P(pr(k, ap, F, yp, D, 2 * nw)), w2s=P(pr(k, ap, F, None, 0, 2 * nw, idx_c=True)),
+                g2=P(pr(k, ap, F, G, 0, 2 * nw, B=dyp, b_cols=D, beta=1.0, out_expert=True)),
+                d2=P(pr(k, dyp, D, dap, F, 2 * nw)), d2s=P(pr(k, dyp, D, gp, F, 2 * nw)),
+                g13=P(pr(k, Xp, D, G, 0, 0, B=dgp, b_cols=F, beta=1.0, out_expert=True) + pr(k, Xp, D, G, 0, nw, B=dup, b_cols=F, beta=1.0, out_expert=True)),
+                d1=P(pr(k, dgp, F, dXp, D, 0)), d3=P(pr(k, dup, F, dXp, D, nw)),
+                d1s=P(pr(k, dgp, F, None, 0, 0, idx_c=True)), d3s=P(pr(k, dup, F, None, 0, nw, idx_c=True)))
+
+    def layer(L, fused, merged):
+        R = L.R
+        if fused: q.moe_gather(x, ident, xb, N, D, ACT_BF16, stream)               # the token matrix as bf16, once per layer
+        for k in range(L.n):                                                          # forward
+            T, tok, gk = L.T[k], L.tok[k * R:(k + 1) * R], gate[k * N:(k + 1) * N]
+            if fused: q.gemm_nn_gather_swiglu(d, s, group, T["w1g"], T["w3o"], E, D, F, xb, stream)
+            else:
+                q.moe_gather(x, tok, Xp, R, D, ACT_BF16, stream)
+                q.gemm_nn(d, s, group, T["w13"], 2 * E, D, F, ACT_BF16, MATH_MFMA_F16, stream)
+                q.swiglu(gp, up, ap, R * F, ACT_BF16, stream)
+            if merged:
+                q.gemm_nn(d, s, group, T["w2"], E, F, D, ACT_BF16, MATH_MFMA_F16, stream)
+                q.moe_combine(yp, L.inv, gate, out, N, K, D, stream)
+            elif fused: q.gemm_nn_scatter(d, s, group, T["w2s"], E, F, D, out, gk, stream)
+            else:
+                q.gemm_nn(d, s, group, T["w2"], E, F, D, ACT_BF16, MATH_MFMA_F16, stream)
+                q.moe_scatter_gate(yp, tok, gk, out, N, D, stream)
+        for k in range(L.n):                                                          # backward
+            T, tok, gk = L.T[k], L.tok[k * R:(k + 1) * R], gate[k * N:(k + 1) * N]
+            q.moe_gather(x, tok, Xp, R, D, ACT_BF16, stream)                          # the weight gradient reads the grouped rows
+            if fused: q.gemm_nn_swiglu(d, s, group, T["w1"], T["w3"], E, D, F, ACT_BF16, MATH_MFMA_F16, stream)
+            else:
+                q.gemm_nn(d, s, group, T["w13"], 2 * E, D, F, ACT_BF16, MATH_MFMA_F16, stream)
+                q.swiglu(gp, up, ap, R * F, ACT_BF16, stream)
+            q.gemm_nn(d, s, group, T["w2"], E, F, D, ACT_BF16, MATH_MFMA_F16, stream)
+            if merged: q.moe_dgate_merged(dout, yp, L.perm, gate, dgate, dyp, N, K, D, ACT_BF16, stream)
+            else:      q.moe_dgate(dout, yp, tok, gk, dgate[k * N:(k + 1) * N], dyp, N, D, ACT_BF16, stream)
+            q.gemm_nt(T["g2"], E, F, D, ACT_BF16, MATH_MFMA, stream)
+            if fused: q.gemm_tn_swiglu_bwd(d, s, group, T["d2s"], E, D, F, gp, up, dgp, dup, stream)
+            else:
+                q.gemm_tn(d, s, group, T["d2"], E, D, F, ACT_BF16, MATH_MFMA, stream)
+                q.swiglu_bwd(gp, up, dap, dgp, dup, R * F, ACT_BF16, stream)
+            q.gemm_nt(T["g13"], 2 * E, D, F, ACT_BF16, MATH_MFMA, stream)
+            if merged:
+                q.gemm_tn_pair(d, s, group, T["d1"], T["d3"], E, F, D, ACT_BF16, MATH_MFMA, stream)
+                q.moe_combine(dXp, L.inv, None, dx, N, K, D, stream)
+            elif fused: q.gemm_tn_pair_scatter(d, s, group, T["d1s"], T["d3s"], E, F, D, dx, stream)
+            else:
+                q.gemm_tn_pair(d, s, group, T["d1"], T["d3"], E, F, D, ACT_BF16, MATH_MFMA, stream)
+                q.moe_scatter_add(dXp, tok, dx, N, D, stream)
+
+    steps, warmup = max(5, args.steps // 4), max(2, args.warmup // 4)
+    per_pass, one_list = Lists(False), Lists(True)
+    t_sep = timed(torch, lambda: layer(per_pass, False, False), steps, warmup)
+    t_fus = timed(torch, lambda: layer(per_pass, True, False), steps, warmup)
+    t_mrg = timed(torch, lambda: layer(one_list, True, True), steps, warmup)
+    flops = K * 12 * 2.0 * N * D * F                       # per pass: 3 forward GEMMs, 3 recomputed in the backward, 3 dgrad, 3 wgrad
+    tf = flops / (t_mrg["event_ms_avg"] * 1e-3) / 1e12
+    return {"workload": "C3 whole expert layer, forward + backward with the recomputed forward (%d tokens top-%d, E=%d D=%d F=%d): GEMMs and glue" % (N, K, E, D, F),
+            "metric": "layer TFLOP/s (12 GEMMs per token and pass incl. the recomputed forward; all passes as one grouped list, glue folded in)",
+            "value": tf, "unit": "TFLOP/s", "ms_per_step": t_mrg["wall_ms"], "dtype": "bf16", "steps": steps, "warmup": warmup,
+            "layer_ms": {"pass by pass, glue as separate kernels": t_sep["event_ms_avg"], "pass by pass, glue folded into the GEMMs": t_fus["event_ms_avg"],
+                         "all passes as one list, glue folded in": t_mrg["event_ms_avg"]},
+            "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                         "kernel": "whole layer: grouped GEMMs + router-independent glue"}}
 
 
 # --------------------------------------------------------------------------------------------- c5
@@ -682,13 +826,13 @@ def main():
     q = pkg.load()           # raises if libqlmx.so is missing or no gfx950 device
     torch.cuda.set_device(0)
     want = ["train", "decode", "adamw", "c5"] if args.workload == "all" else [args.workload]
-    runners = {"adamw": bench_adamw, "train": bench_train, "decode": bench_decode, "copy": bench_copy, "codec": bench_codec, "glue": bench_glue, "c5": bench_c5,
+    runners = {"adamw": bench_adamw, "train": bench_train, "decode": bench_decode, "copy": bench_copy, "codec": bench_codec, "glue": bench_glue, "c5": bench_c5, "layer": bench_layer,
                "train5": lambda t, qq, a: bench_train(t, qq, a, E=64, D=2048, F=1408, tokens=32768, topk=4, label="C5 train layer (one of 8)")}
     results = {}
     for w in want:
         if w in runners:
             results[w] = runners[w](torch, q, args)
-    first = next(results[w] for w in ["train", "train5", "c5", "decode", "adamw", "codec", "glue", "copy"] if w in results)
+    first = next(results[w] for w in ["train", "train5", "c5", "layer", "decode", "adamw", "codec", "glue", "copy"] if w in results)
     line = {
         "metric": "QLM expert dequant-GEMM TFLOP/s & GB/s (% roofline); int-AdamW GB/s",
         "value": first["value"], "unit": first["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

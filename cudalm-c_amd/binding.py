@@ -73,6 +73,8 @@ SIGNATURES = {
     "qlmx_moe_gemm_tn_pair": (c_i, [c_vp, c_vp, c_i, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_nn_swiglu": (c_i, [c_vp, c_vp, c_i, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_gemm_nn_gather": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_vp, c_vp]),
+    "qlmx_moe_gemm_nn_gather_swiglu": (c_i, [c_vp, c_vp, c_i, c_vp, c_vp, c_i, c_i, c_i, c_vp, c_vp]),
+    "qlmx_moe_gemm_tn_swiglu_bwd": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "qlmx_moe_gemm_nn_scatter": (c_i, [c_vp, c_vp, c_i, c_vp, c_i, c_i, c_i, c_vp, c_vp, c_vp]),
     "qlmx_moe_gemm_tn_pair_scatter": (c_i, [c_vp, c_vp, c_i, c_vp, c_vp, c_i, c_i, c_i, c_vp, c_vp]),
     "qlmx_moe_gemm_nt": (c_i, [c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
@@ -91,6 +93,9 @@ SIGNATURES = {
     "qlmx_moe_scatter_gate": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_vp]),
     "qlmx_moe_scatter_add": (c_i, [c_vp, c_vp, c_vp, c_i, c_i, c_vp]),
     "qlmx_moe_dgate": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_vp]),
+    "qlmx_moe_dgate_merged": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_moe_merge_rows": (c_i, [c_vp, c_i, c_i, c_vp, c_vp, c_vp]),
+    "qlmx_moe_combine": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_vp]),
     "qlmx_swiglu": (c_i, [c_vp, c_vp, c_vp, c_sz, c_i, c_vp]),
     "qlmx_swiglu_bwd": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_i, c_vp]),
     "qlmx_q4n_bound": (c_sz, [c_sz, c_i]),
@@ -168,6 +173,12 @@ class Qlmx:
     def gemm_nn_gather(self, d, s, group, probs, nprob, K, N, x_bf16, stream=None):
         self.call("qlmx_moe_gemm_nn_gather", d, s, group, C.addressof(probs), nprob, K, N, x_bf16, stream)
 
+    def gemm_nn_gather_swiglu(self, d, s, group, gate, up, nprob, K, N, x_bf16, stream=None):
+        self.call("qlmx_moe_gemm_nn_gather_swiglu", d, s, group, C.addressof(gate), C.addressof(up), nprob, K, N, x_bf16, stream)
+
+    def gemm_tn_swiglu_bwd(self, d, s, group, probs, nprob, K, N, gp, up, dgp, dup, stream=None):
+        self.call("qlmx_moe_gemm_tn_swiglu_bwd", d, s, group, C.addressof(probs), nprob, K, N, gp, up, dgp, dup, stream)
+
     def gemm_nn_scatter(self, d, s, group, probs, nprob, K, N, out, gate, stream=None):
         self.call("qlmx_moe_gemm_nn_scatter", d, s, group, C.addressof(probs), nprob, K, N, out, gate, stream)
 
@@ -215,6 +226,15 @@ class Qlmx:
 
     def moe_scatter_add(self, dXp, perm, dst, N, D, stream=None):
         self.call("qlmx_moe_scatter_add", dXp, perm, dst, N, D, stream)
+
+    def moe_dgate_merged(self, dout, yp, perm, gate, d_gate, dyp, N, K, D, out_dtype=ACT_F32, stream=None):
+        self.call("qlmx_moe_dgate_merged", dout, yp, perm, gate, d_gate, dyp, N, K, D, out_dtype, stream)
+
+    def moe_merge_rows(self, perm, N, K, tok, inv, stream=None):
+        self.call("qlmx_moe_merge_rows", perm, N, K, tok, inv, stream)
+
+    def moe_combine(self, y, inv, gate, out, N, K, D, stream=None):
+        self.call("qlmx_moe_combine", y, inv, gate, out, N, K, D, stream)
 
     def moe_dgate(self, dout, yp, perm, gate, d_gate, dyp, N, D, out_dtype=ACT_F32, stream=None):
         self.call("qlmx_moe_dgate", dout, yp, perm, gate, d_gate, dyp, N, D, out_dtype, stream)

@@ -77,6 +77,11 @@ __device__ __forceinline__ int qx_xcd_tile_rows(int b, int g){
 }
 
 typedef float qx_f32x16 __attribute__((ext_vector_type(16)));
+/* round to nearest even, as cudalm.cu:334-338 */
+__device__ __forceinline__ unsigned short qx_f32_to_bf16(float f){
+    uint32_t x = __float_as_uint(f);
+    return (unsigned short)((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16);
+}
 typedef __attribute__((address_space(1))) float qx_gfloat;      /* known to be global memory: loads and stores complete in order */
 
 /* Writes the NI x NJ accumulator tiles (32x32 each, as v_mfma_f32_32x32x16 leaves them) of one
@@ -180,30 +185,94 @@ __device__ __forceinline__ void qx_store_tiles(const qx_f32x16 (&acc)[NI][NJ], f
     else                           qx_store_tiles_edge<NI, NJ, SYS>(acc, (qx_gfloat *)c, row, rows, ld, accumulate);
 }
 
+/* k_swiglu_bwd (cudalm.cu:2440-2453; cpu_kern.h:385-394) for one element: z, u the forward's gate and up
+ * pre-activations, da the gradient of their SwiGLU */
+template<bool HW = false>
+__device__ __forceinline__ void qx_swiglu_bwd1(float z, float u, float da, float &dg, float &du){
+    const float sg = HW ? qx_fsig_hw(z) : qx_fsig(z), silu = z * sg, ds = sg + z * sg * (1.0f - sg);
+    dg = da * u * ds; du = da * silu;
+}
+/* The SwiGLU gradient as the epilogue of the GEMM that produces its input: the NI x 2 accumulator tiles hold
+ * da = d(act); gp, up (fp32) are read at the same positions and bf16(dg), bf16(du) written there, so that da
+ * itself never reaches memory; the sigmoid is qx_fsig_hw. All four pointers are at the lane's first element (row `row`, its column in
+ * tile (., 0)); neighbouring columns are paired into 4-byte stores as in qx_store_swiglu. */
+template<int NI>
+__device__ __forceinline__ void qx_store_swiglu_bwd(const qx_f32x16 (&acc)[NI][2], const float *gp, const float *up,
+                                                    unsigned short *dg, unsigned short *du, int row, int rows, size_t ld){
+    typedef const __attribute__((address_space(1))) float gfloat;
+    typedef __attribute__((address_space(1))) uint32_t guint;
+    const bool oddl = threadIdx.x & 1;
+#pragma unroll
+    for(int i = 0; i < NI; i++){
+        float z[2][16], u[2][16];
+#pragma unroll
+        for(int e = 0; e < 16; e++){
+            const int ro = i * 32 + (e >> 2) * 8 + (e & 3);
+            const bool in = row + ro < rows;
+#pragma unroll
+            for(int j = 0; j < 2; j++){
+                const size_t o = (size_t)ro * ld + j * 32;
+                z[j][e] = in ? *((gfloat *)gp + o) : 0.0f;
+                u[j][e] = in ? *((gfloat *)up + o) : 0.0f;
+            }
+        }
+#pragma unroll
+        for(int j = 0; j < 2; j++){
+            uint32_t a[16];                                  /* bf16(dg) | bf16(du) << 16 of the lane's 16 rows */
+#pragma unroll
+            for(int e = 0; e < 16; e++){
+                float x, y;
+                qx_swiglu_bwd1<true>(z[j][e], u[j][e], acc[i][j][e], x, y);
+                a[e] = (uint32_t)qx_f32_to_bf16(x) | ((uint32_t)qx_f32_to_bf16(y) << 16);
+            }
+            /* the even lane of a pair of columns stores the first eight of its rows for both, the odd lane the rest */
+#pragma unroll
+            for(int e = 0; e < 8; e++){
+                const uint32_t mine = oddl ? a[e + 8] : a[e];
+                const uint32_t got = (uint32_t)__shfl_xor((int)(oddl ? a[e] : a[e + 8]), 1, 64);
+                const uint32_t lo = oddl ? got : mine, hi = oddl ? mine : got;          /* even column, odd column */
+                const int e2 = oddl ? e + 8 : e;
+                const int ro = i * 32 + (e2 >> 2) * 8 + (e2 & 3);
+                if(row + ro < rows){
+                    const size_t o = (size_t)ro * ld + j * 32 - (oddl ? 1 : 0);
+                    *(guint *)(dg + o) = (lo & 0xFFFFu) | (hi << 16);
+                    *(guint *)(du + o) = (lo >> 16) | (hi & 0xFFFF0000u);
+                }
+            }
+        }
+    }
+}
+
 /* The NI x 2 accumulator tiles of one wavefront added to INDEXED output rows (the gated scatter and the
  * scatter-add of the MoE glue, cudalm.cu:2541-2545, 2564-2567, as a GEMM epilogue): row r of the problem goes to
  * row idx[r] of `out`, out = out + gate[idx[r]] * y (multiply, then add, as k_scatter_gate does), or out += y when
  * gate is NULL (k_scatter_add4); idx[r] < 0 drops the row. `row` is the lane's first row, `col` its column in
- * tile (., 0); tile (., 1) lies 32 columns further. 32 lanes cover 128 contiguous bytes of an output row. */
+ * tile (., 0); tile (., 1) lies 32 columns further. 32 lanes cover 128 contiguous bytes of an output row.
+ * The additions are float atomics without a return value, sent off behind each other: a row index occurs
+ * once in a launch's lists, so each element receives exactly one addition and the result is the one rounded
+ * sum that a load, an add and a store would give, without the wavefront waiting a memory round trip per row. */
 template<int NI>
 __device__ __forceinline__ void qx_scatter_tiles(const qx_f32x16 (&acc)[NI][2], const int *idx, const float *gate, float *out,
                                                  int row, int rows, size_t ld, int col){
 #pragma unroll
-    for(int i = 0; i < NI; i++)
+    for(int i = 0; i < NI; i++){
+        int tok[16]; float g[16];
 #pragma unroll
         for(int e = 0; e < 16; e++){
             const int r = row + i * 32 + (e >> 2) * 8 + (e & 3);
-            if(r < rows){
-                const int tok = idx[r];
-                if(tok >= 0){
-                    float *o = out + (size_t)tok * ld + col;
-                    if(gate){
-                        const float g = gate[tok];
-                        o[0] = o[0] + g * acc[i][0][e]; o[32] = o[32] + g * acc[i][1][e];
-                    } else { o[0] += acc[i][0][e]; o[32] += acc[i][1][e]; }
-                }
-            }
+            tok[e] = r < rows ? idx[r] : -1;
         }
+#pragma unroll
+        for(int e = 0; e < 16; e++) g[e] = (gate && tok[e] >= 0) ? gate[tok[e]] : 1.0f;
+#pragma unroll
+        for(int e = 0; e < 16; e++)
+            if(tok[e] >= 0){
+                qx_gfloat *o = (qx_gfloat *)(out + (size_t)tok[e] * ld + col);
+                const float y0 = gate ? g[e] * acc[i][0][e] : acc[i][0][e], y1 = gate ? g[e] * acc[i][1][e] : acc[i][1][e];
+                (void)__builtin_amdgcn_global_atomic_fadd_f32(o, y0);
+                (void)__builtin_amdgcn_global_atomic_fadd_f32(o + 32, y1);
+            }
+    }
 }
 
 /* ---- scheduled launches: instead of deriving its tile from its index, a workgroup reads an entry of
@@ -245,10 +314,43 @@ __device__ __forceinline__ void qx_chain_publish(int *flags, int flag, unsigned 
 }
 
 __device__ __forceinline__ float qx_bf16_to_f32(unsigned short h){ return __uint_as_float((uint32_t)h << 16); }
-/* round to nearest even, as cudalm.cu:334-338 */
-__device__ __forceinline__ unsigned short qx_f32_to_bf16(float f){
-    uint32_t x = __float_as_uint(f);
-    return (unsigned short)((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16);
+
+/* gate, up (fp32; both skipped when gp is NULL) and bf16(gate * sigmoid(gate) * up) of a gate|up tile (HW: the
+ * sigmoid is qx_fsig_hw instead of the SwiGLU kernel's qx_fsig). The tile's 128 LDS columns are
+ * [gate 0-31 | up 0-31 | gate 32-63 | up 32-63] of the problem's columns j0 .. j0+63, so a wavefront's first
+ * accumulator column holds gate and its second holds up of the same 32 columns, element for element. */
+template<int NI, bool HW = false>
+__device__ __forceinline__ void qx_store_swiglu(const qx_f32x16 (&acc)[NI][2], float *gp, float *up, unsigned short *act,
+                                                 int row, int rows, size_t ld){
+    typedef __attribute__((address_space(1))) float gfloat;
+    typedef __attribute__((address_space(1))) uint32_t guint;
+    const bool oddl = threadIdx.x & 1;
+#pragma unroll
+    for(int i = 0; i < NI; i++){
+        uint32_t a[16];
+#pragma unroll
+        for(int e = 0; e < 16; e++){
+            const int ro = i * 32 + (e >> 2) * 8 + (e & 3);
+            const float g = acc[i][0][e], u = acc[i][1][e];
+            a[e] = qx_f32_to_bf16(g * (HW ? qx_fsig_hw(g) : qx_fsig(g)) * u);
+            if(gp && row + ro < rows){
+                const size_t o = (size_t)ro * ld;
+                __builtin_nontemporal_store(g, (gfloat *)gp + o);
+                __builtin_nontemporal_store(u, (gfloat *)up + o);
+            }
+        }
+        /* two neighbouring columns per 4-byte store: the even lane of a pair writes the first eight of its
+         * rows for both, the odd lane the other eight */
+#pragma unroll
+        for(int e = 0; e < 8; e++){
+            const uint32_t got = (uint32_t)__shfl_xor((int)(oddl ? a[e] : a[e + 8]), 1, 64);
+            const int e2 = oddl ? e + 8 : e;
+            const int ro = i * 32 + (e2 >> 2) * 8 + (e2 & 3);
+            const uint32_t v = oddl ? (got | (a[e + 8] << 16)) : (a[e] | (got << 16));
+            if(row + ro < rows) *(guint *)(act + (size_t)ro * ld - (oddl ? 1 : 0)) = v;
+        }
+    }
 }
+
 
 #endif

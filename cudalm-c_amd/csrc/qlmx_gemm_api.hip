@@ -74,6 +74,8 @@ extern "C" int qlmx_moe_gemm_tn_pair(const signed char *d, const float *s, int g
 }
 int qlmx_gemm_nn_swiglu_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *gate,
                                    const qlmx_gemm_prob *up, int nprob, int K, int N, hipStream_t st);
+int qlmx_gemm_nn_h_swiglu_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *gate, const qlmx_gemm_prob *up_,
+                                 int nprob, int K, int N, const void *xsrc, hipStream_t st);
 extern "C" int qlmx_swiglu(const float *G, const float *U, void *O, size_t n, int out_dtype, void *stream);
 
 /* The gate and up GEMMs of moe_forward and the SwiGLU between them and the down GEMM (cudalm.cu:4211-4215:
@@ -89,9 +91,10 @@ extern "C" int qlmx_moe_gemm_nn_swiglu(const signed char *d, const float *s, int
     QLMX_REQUIRE(gate && up && nprob >= 0, "qlmx_moe_gemm_nn_swiglu: NULL problem list");
     for(int i = 0; i < nprob; i++){
         QLMX_REQUIRE(up[i].M == gate[i].M, "qlmx_moe_gemm_nn_swiglu: problem %d has %d and %d rows", i, gate[i].M, up[i].M);
-        QLMX_REQUIRE(gate[i].M == 0 || (gate[i].A && gate[i].C && up[i].C && up[i].B), "qlmx_moe_gemm_nn_swiglu: problem %d has a NULL pointer", i);
+        const bool both_or_none = math == QLMX_MATH_MFMA_F16 && !gate[i].C && !up[i].C;       /* bf16 output only */
+        QLMX_REQUIRE(gate[i].M == 0 || (gate[i].A && ((gate[i].C && up[i].C) || both_or_none) && up[i].B), "qlmx_moe_gemm_nn_swiglu: problem %d has a NULL pointer", i);
     }
-    if(act_dtype == QLMX_ACT_BF16 && math == QLMX_MATH_MFMA && N % 64 == 0 && K % 32 == 0 && group >= 64 && (group & (group - 1)) == 0 &&
+    if(act_dtype == QLMX_ACT_BF16 && (math == QLMX_MATH_MFMA || math == QLMX_MATH_MFMA_F16) && N % 64 == 0 && K % 32 == 0 && group >= 64 && (group & (group - 1)) == 0 &&
        nprob * 2 <= QLMX_MAX_PROBLEMS){
         QLMX_REQUIRE(d && s && ((uintptr_t)d & 15) == 0, "qlmx_moe_gemm_nn_swiglu: digits and scales must be given, digits 16-byte aligned");
         for(int i = 0; i < nprob; i++){
@@ -99,8 +102,11 @@ extern "C" int qlmx_moe_gemm_nn_swiglu(const signed char *d, const float *s, int
             QLMX_REQUIRE(gate[i].wq % (unsigned long long)group == 0 && up[i].wq % (unsigned long long)group == 0 &&
                          (gate[i].wq & 31ULL) == 0 && (up[i].wq & 31ULL) == 0, "qlmx_moe_gemm_nn_swiglu: problem %d weight offset alignment", i);
         }
+        if(math == QLMX_MATH_MFMA_F16) return qlmx_gemm_nn_h_swiglu_launch(d, s, group, gate, up, nprob, K, N, nullptr, (hipStream_t)stream);
         return qlmx_gemm_nn_swiglu_lds_launch(d, s, group, gate, up, nprob, K, N, (hipStream_t)stream);
     }
+    for(int i = 0; i < nprob; i++)
+        QLMX_REQUIRE(gate[i].M == 0 || (gate[i].C && up[i].C), "qlmx_moe_gemm_nn_swiglu: problem %d has no fp32 outputs and the shape is not one the fused kernel takes", i);
     rc = gemm_entry("qlmx_moe_gemm_nn_swiglu", GEMM_NN, d, s, group, gate, nprob, K, N, act_dtype, math, stream); if(rc) return rc;
     qlmx_gemm_prob *tmp = (qlmx_gemm_prob *)malloc(sizeof(qlmx_gemm_prob) * (size_t)(nprob > 0 ? nprob : 1));
     QLMX_REQUIRE(tmp, "qlmx_moe_gemm_nn_swiglu: out of host memory");
@@ -116,7 +122,8 @@ extern "C" int qlmx_moe_gemm_nn_swiglu(const signed char *d, const float *s, int
 int qlmx_gemm_nn_h_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N,
                           int io, const void *xsrc, float *out, const float *gate, hipStream_t st);
 int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second,
-                            int nprob, int K, int N, float *out, const float *gate, hipStream_t st);
+                            int nprob, int K, int N, float *out, const float *gate,
+                            const float *gp, const float *up_, void *dg, void *du, hipStream_t st);
 
 static int rows_entry_checks(const char *who, const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs,
                              const qlmx_gemm_prob *second, int nprob, int K, int N, int bk, bool idx_in_a){
@@ -148,6 +155,27 @@ extern "C" int qlmx_moe_gemm_nn_gather(const signed char *d, const float *s, int
     QLMX_REQUIRE(x_bf16 && ((uintptr_t)x_bf16 & 15) == 0 && K % 8 == 0, "qlmx_moe_gemm_nn_gather: token matrix must be given and 16-byte aligned");
     return qlmx_gemm_nn_h_launch(d, s, group, probs, nprob, K, N, 1, x_bf16, nullptr, nullptr, (hipStream_t)stream);
 }
+/* k_gather + mg_ab w1 + mg_ab w3 + e_swig (cudalm.cu:4209-4215) in one launch: qlmx_moe_gemm_nn_swiglu with
+ * QLMX_MATH_MFMA_F16 whose gate[i].A are row-index lists into the bf16 token matrix x, as in qlmx_moe_gemm_nn_gather.
+ * gate[i].C and up[i].C may both be NULL: only the bf16 SwiGLU output up[i].B is written then. */
+extern "C" int qlmx_moe_gemm_nn_gather_swiglu(const signed char *d, const float *s, int group,
+                                              const qlmx_gemm_prob *gate, const qlmx_gemm_prob *up, int nprob, int K, int N,
+                                              const void *x_bf16, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(d && s && gate && up && nprob >= 0 && K > 0 && N > 0 && nprob * 2 <= QLMX_MAX_PROBLEMS, "qlmx_moe_gemm_nn_gather_swiglu: NULL or empty argument, or too many problems");
+    QLMX_REQUIRE(((uintptr_t)d & 15) == 0 && x_bf16 && ((uintptr_t)x_bf16 & 15) == 0, "qlmx_moe_gemm_nn_gather_swiglu: digits and token matrix must be 16-byte aligned");
+    QLMX_REQUIRE(N % 64 == 0 && K % 32 == 0, "qlmx_moe_gemm_nn_gather_swiglu: N=%d must be a multiple of 64 and K=%d of 32", N, K);
+    QLMX_REQUIRE(group >= 64 && group <= 256 && (group & (group - 1)) == 0, "qlmx_moe_gemm_nn_gather_swiglu: group %d must be 64, 128 or 256", group);
+    for(int i = 0; i < nprob; i++){
+        QLMX_REQUIRE(up[i].M == gate[i].M, "qlmx_moe_gemm_nn_gather_swiglu: problem %d has %d and %d rows", i, gate[i].M, up[i].M);
+        if(gate[i].M == 0) continue;
+        QLMX_REQUIRE(gate[i].A && up[i].B && (gate[i].C != nullptr) == (up[i].C != nullptr), "qlmx_moe_gemm_nn_gather_swiglu: problem %d has a NULL pointer (the fp32 outputs: both or none)", i);
+        QLMX_REQUIRE(((uintptr_t)gate[i].A & 3) == 0 && ((uintptr_t)up[i].B & 3) == 0, "qlmx_moe_gemm_nn_gather_swiglu: problem %d operand alignment", i);
+        QLMX_REQUIRE(gate[i].wq % (unsigned long long)group == 0 && up[i].wq % (unsigned long long)group == 0 &&
+                     (gate[i].wq & 31ULL) == 0 && (up[i].wq & 31ULL) == 0, "qlmx_moe_gemm_nn_gather_swiglu: problem %d weight offset alignment", i);
+    }
+    return qlmx_gemm_nn_h_swiglu_launch(d, s, group, gate, up, nprob, K, N, x_bf16, (hipStream_t)stream);
+}
 /* mg_ab + k_scatter_gate (cudalm.cu:4224-4227) in one launch: problem i computes y = A . W and adds it to indexed rows,
  * out[idx_i[r], :] = out[idx_i[r], :] + gate[idx_i[r]] * y[r, :], idx_i = (const int *)probs[i].C (entries < 0 are dropped;
  * gate NULL adds y itself). No output row may be named twice in one call (true of one pass of the MoE layer). */
@@ -166,7 +194,21 @@ extern "C" int qlmx_moe_gemm_tn_pair_scatter(const signed char *d, const float *
                                              float *dst, void *stream){
     int rc = rows_entry_checks("qlmx_moe_gemm_tn_pair_scatter", d, s, group, first, second, nprob, K, N, 64, false); if(rc) return rc;
     QLMX_REQUIRE(dst && second && nprob * 2 <= QLMX_MAX_PROBLEMS, "qlmx_moe_gemm_tn_pair_scatter: NULL output or too many problems");
-    return qlmx_gemm_tn_lds_launch(d, s, group, first, second, nprob, K, N, dst, nullptr, (hipStream_t)stream);
+    return qlmx_gemm_tn_lds_launch(d, s, group, first, second, nprob, K, N, dst, nullptr, nullptr, nullptr, nullptr, nullptr, (hipStream_t)stream);
+}
+/* mg_abt (the down projection's input gradient) + e_swigb (cudalm.cu:4340-4346) in one launch: problem i computes
+ * d(act) = A . W^T [M, N] and, instead of storing it, applies k_swiglu_bwd to it: with o the element offset of
+ * probs[i].C inside gp (probs[i].C points at the problem's rows of the forward's gate pre-activations),
+ * dgp[o ..] and dup[o ..] (bf16) receive the gradients computed from gp[o ..], up[o ..] (fp32). Element for
+ * element the operations of qlmx_swiglu_bwd on the stored product: bit-identical to the two separate calls. */
+extern "C" int qlmx_moe_gemm_tn_swiglu_bwd(const signed char *d, const float *s, int group,
+                                           const qlmx_gemm_prob *probs, int nprob, int K, int N,
+                                           const float *gp, const float *up, void *dgp, void *dup, void *stream){
+    int rc = rows_entry_checks("qlmx_moe_gemm_tn_swiglu_bwd", d, s, group, probs, nullptr, nprob, K, N, 64, false); if(rc) return rc;
+    QLMX_REQUIRE(gp && up && dgp && dup && (((uintptr_t)gp | (uintptr_t)up | (uintptr_t)dgp | (uintptr_t)dup) & 3) == 0, "qlmx_moe_gemm_tn_swiglu_bwd: NULL or misaligned buffer");
+    for(int i = 0; i < nprob; i++)
+        QLMX_REQUIRE(probs[i].M == 0 || (probs[i].C >= gp && (probs[i].C - gp) % 2 == 0), "qlmx_moe_gemm_tn_swiglu_bwd: problem %d: C must point into gp at an even element", i);
+    return qlmx_gemm_tn_lds_launch(d, s, group, probs, nullptr, nprob, K, N, nullptr, nullptr, gp, up, dgp, dup, (hipStream_t)stream);
 }
 
 /* mg_atb + mg_flush (cudalm.cu:3254-3256) */

@@ -127,7 +127,7 @@ static int upload_problems(const qlmx_gemm_prob *probs, const qlmx_gemm_prob *se
         const qlmx_gemm_prob &p = probs[i];
         QLMX_REQUIRE(p.M >= 0, "grouped gemm: problem %d has M=%d", i, p.M);
         if(p.M == 0) continue;
-        QLMX_REQUIRE(p.A && p.C, "grouped gemm: problem %d has a NULL operand", i);
+        QLMX_REQUIRE(p.A && (p.C || (second && mode == GEMM_NN)), "grouped gemm: problem %d has a NULL operand", i);
         QLMX_REQUIRE(mode != GEMM_NT || p.B, "grouped gemm nt: problem %d has no B operand", i);
         QLMX_REQUIRE(p.beta == 0.0f || p.beta == 1.0f, "grouped gemm: beta must be 0 or 1");
         const int rows = mode == GEMM_NT ? K : p.M;
@@ -140,7 +140,7 @@ static int upload_problems(const qlmx_gemm_prob *probs, const qlmx_gemm_prob *se
         if(second){
             const qlmx_gemm_prob &p2 = second[i];
             QLMX_REQUIRE(p2.M == p.M, "grouped gemm: problem %d and its second half differ in rows (%d, %d)", i, p.M, p2.M);
-            QLMX_REQUIRE(mode == GEMM_TN ? p2.A != nullptr : (p2.B != nullptr && p2.C != nullptr), "grouped gemm: the second half of problem %d lacks a pointer", i);
+            QLMX_REQUIRE(mode == GEMM_TN ? p2.A != nullptr : (p2.B != nullptr && (p2.C != nullptr) == (p.C != nullptr)), "grouped gemm: the second half of problem %d lacks a pointer", i);
             DevProb &c = h[n++];
             c = q; c.A = p2.A; c.B = p2.B; c.C = p2.C; c.wq = p2.wq; c.wg = p2.wg; c.tile0 = (int)tiles; c.chunk = 0;
         }

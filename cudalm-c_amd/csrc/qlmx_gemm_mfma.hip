@@ -31,7 +31,8 @@
  */
 #include "qlmx_gemm.h"
 int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second,
-                            int nprob, int K, int N, float *out, const float *gate, hipStream_t st);
+                            int nprob, int K, int N, float *out, const float *gate,
+                            const float *gp, const float *up_, void *dg, void *du, hipStream_t st);
 int qlmx_gemm_nn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st);
 int qlmx_gemm_nn_h_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs, int nprob, int K, int N,
                           int io, const void *xsrc, float *out, const float *gate, hipStream_t st);
@@ -415,7 +416,7 @@ int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int 
     }
     QLMX_REQUIRE(mode == GEMM_NT || ((uintptr_t)d & 15) == 0, "mfma gemm: digit array is not 16-byte aligned");
     /* bf16 operands take the direct-to-LDS kernels; fp32 activations need the converting ones */
-    if(mode == GEMM_TN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_tn_lds_launch(d, s, group, probs, second, nprob, K, N, nullptr, nullptr, st);
+    if(mode == GEMM_TN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_tn_lds_launch(d, s, group, probs, second, nprob, K, N, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, st);
     if(mode == GEMM_NT && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nt_lds_launch(probs, nprob, K, N, st);
     if(mode == GEMM_NN && act_dtype == QLMX_ACT_BF16 && f16) return qlmx_gemm_nn_h_launch(d, s, group, probs, nprob, K, N, 0, nullptr, nullptr, nullptr, st);
     if(mode == GEMM_NN && act_dtype == QLMX_ACT_BF16) return qlmx_gemm_nn_lds_launch(d, s, group, probs, nprob, K, N, st);

@@ -100,8 +100,13 @@ struct NhW { i32x2 d; int s; };
 
 /* One output tile of NI*64 rows (NI = 4: the full 256; the last tile of a problem takes the smallest NI that
  * holds its rows). */
-template<int NI, int IO>
-__device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, int i0, int j0, unsigned char *lds){
+/* The second half of a gate|up problem (DUAL): the other weight matrix, its fp32 output, the SwiGLU output. The
+ * tile's 128 LDS columns are then [gate 0-31 | up 0-31 | gate 32-63 | up 32-63] of the problem's columns
+ * j0 .. j0+63: a wavefront's first accumulator column holds gate and its second up of the same 32 columns. */
+struct NhDual { unsigned long long wq, wg; float *C; unsigned short *act; };
+
+template<int NI, int IO, bool DUAL = false>
+__device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, const NhDual &Q, int i0, int j0, unsigned char *lds){
     const int rows = P.M;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wi = (wave >> 1) * (NI * 32), wj = (wave & 1) * 64;
@@ -125,9 +130,10 @@ __device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, int i
      * per step; its two 16-byte units are taken in opposite order by even and odd rows, so that the 16 lanes of
      * a write phase (two rows) hit 16 different units ---- */
     const int oc = tid & 7, kr = tid >> 3, odd = kr & 1;
-    const size_t e0 = (size_t)kr * a.N + j0 + oc * 16;
-    const signed char *pw = a.d + ((P.wq + e0) >> 1);
-    const float *ps = a.s + P.wg + (e0 >> a.gshift);
+    const bool second = DUAL && ((oc >> 1) & 1);
+    const size_t e0 = (size_t)kr * a.N + j0 + (DUAL ? ((oc & 1) + ((oc >> 2) << 1)) * 16 : oc * 16);
+    const signed char *pw = a.d + (((second ? Q.wq : P.wq) + e0) >> 1);
+    const float *ps = a.s + (second ? Q.wg : P.wg) + (e0 >> a.gshift);
     const size_t wstep = (size_t)NH_BK * a.N >> 1, sstep = (size_t)NH_BK * a.N >> a.gshift;
     const int sw = (kr & 3) << 2;
     const uint32_t wr0 = NH_B_OFF + (uint32_t)(kr * 256 + (((2 * oc + odd) ^ sw) << 4));         /* written first  */
@@ -285,7 +291,10 @@ __device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, int i
 #pragma unroll
         for(int j = 0; j < 2; j++) acc[i][j] = acc[i][j] * NH_UNSCALE;
     const int row = i0 + wi + hf * 4;
-    if(IO == NH_SCATTER) qx_scatter_tiles<NI>(acc, (const int *)P.C, a.gate, a.out, row, rows, (size_t)a.N, j0 + wj + fr);
+    if(DUAL){
+        const size_t o = (size_t)row * a.N + (j0 + (wj >> 1) + fr);
+        qx_store_swiglu<NI, true>(acc, P.C ? P.C + o : nullptr, Q.C + o, Q.act + o, row, rows, (size_t)a.N);
+    } else if(IO == NH_SCATTER) qx_scatter_tiles<NI>(acc, (const int *)P.C, a.gate, a.out, row, rows, (size_t)a.N, j0 + wj + fr);
     else qx_store_tiles<NI, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, false);
 }
 
@@ -298,10 +307,32 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nn_h(NhArgs a){
     const int lt = t - P.tile0;
     const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
     const int i0 = ti * NH_BM, j0 = tj * NH_BN, left = P.M - i0;
-    if(left > 192)      nh_tile<4, IO>(a, P, i0, j0, lds);
-    else if(left > 128) nh_tile<3, IO>(a, P, i0, j0, lds);
-    else if(left > 64)  nh_tile<2, IO>(a, P, i0, j0, lds);
-    else                nh_tile<1, IO>(a, P, i0, j0, lds);
+    const NhDual none = {0, 0, nullptr, nullptr};
+    if(left > 192)      nh_tile<4, IO>(a, P, none, i0, j0, lds);
+    else if(left > 128) nh_tile<3, IO>(a, P, none, i0, j0, lds);
+    else if(left > 64)  nh_tile<2, IO>(a, P, none, i0, j0, lds);
+    else                nh_tile<1, IO>(a, P, none, i0, j0, lds);
+}
+
+/* gate|up problems with the SwiGLU in the epilogue (mg_ab w1, mg_ab w3, e_swig; cudalm.cu:4211-4215): tiles of 256
+ * rows x 64 columns of both matrices; the table entry after the problem's holds the second matrix, the up output
+ * and the bf16 SwiGLU output. The fp32 gate / up outputs are skipped when the problem's C is NULL. */
+template<int IO>
+__global__ void __launch_bounds__(256, 2) k_gemm_nn_h_swiglu(NhArgs a){
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * NH_A_BYTES + 2 * NH_B_BYTES];
+    const int t = qx_xcd_tile(blockIdx.x, gridDim.x);
+    if(t >= a.ntiles) return;
+    const int pi = qx_find_problem(a.pr, a.nprob, t);
+    const DevProb P = a.pr[pi];
+    const DevProb P2 = a.pr[pi + 1];
+    const NhDual Q = {P2.wq, P2.wg, P2.C, (unsigned short *)P2.B};
+    const int lt = t - P.tile0;
+    const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
+    const int i0 = ti * NH_BM, j0 = tj * (NH_BN / 2), left = P.M - i0;
+    if(left > 192)      nh_tile<4, IO, true>(a, P, Q, i0, j0, lds);
+    else if(left > 128) nh_tile<3, IO, true>(a, P, Q, i0, j0, lds);
+    else if(left > 64)  nh_tile<2, IO, true>(a, P, Q, i0, j0, lds);
+    else                nh_tile<1, IO, true>(a, P, Q, i0, j0, lds);
 }
 
 /* bf16 activations only; N % 128 == 0, K % 32 == 0, group a power of two >= 32 (checked by the caller).
@@ -321,5 +352,24 @@ int qlmx_gemm_nn_h_launch(const signed char *d, const float *s, int group, const
     else if(io == NH_SCATTER) hipLaunchKernelGGL(k_gemm_nn_h<NH_SCATTER>, dim3(grid), dim3(256), 0, st, a);
     else                      hipLaunchKernelGGL(k_gemm_nn_h<NH_PLAIN>,   dim3(grid), dim3(256), 0, st, a);
     QLMX_LAUNCH_CHECK("grouped gemm nn (fp16 matrix core) launch");
+    return qlmx_upload_done(slot, st);
+}
+
+/* gate|up pairs with the SwiGLU in the epilogue: N % 64 == 0, K % 32 == 0, group a power of two >= 64 (a tile's 64
+ * columns of a matrix share a scale per contraction row). xsrc != NULL: the gate problems' A fields are row-index
+ * lists into the bf16 token matrix xsrc (NH_GATHER). Problems whose gate C is NULL store the bf16 output only. */
+int qlmx_gemm_nn_h_swiglu_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *gate, const qlmx_gemm_prob *up_,
+                                 int nprob, int K, int N, const void *xsrc, hipStream_t st){
+    QLMX_REQUIRE(!xsrc || (size_t)K * 2 <= NH_ZERO_BYTES, "grouped gemm nn + swiglu with gather: K=%d exceeds %d", K, NH_ZERO_BYTES / 2);
+    ProbUpload up; int slot;
+    int rc = qlmx_upload_problem_pairs(gate, up_, nprob, GEMM_NN, K, N, NH_BM, NH_BN / 2, st, &up, &slot); if(rc) return rc;
+    if(up.ntiles == 0) return QLMX_OK;
+    NhArgs a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.d = d; a.s = s; a.K = K; a.N = N;
+    a.xsrc = (const char *)xsrc; a.out = nullptr; a.gate = nullptr;
+    a.gshift = 0; while((1 << a.gshift) < group) a.gshift++;
+    const int grid = (up.ntiles + 7) / 8 * 8;
+    if(xsrc) hipLaunchKernelGGL(k_gemm_nn_h_swiglu<NH_GATHER>, dim3(grid), dim3(256), 0, st, a);
+    else     hipLaunchKernelGGL(k_gemm_nn_h_swiglu<NH_PLAIN>,  dim3(grid), dim3(256), 0, st, a);
+    QLMX_LAUNCH_CHECK("grouped gemm nn + swiglu (fp16 matrix core) launch");
     return qlmx_upload_done(slot, st);
 }

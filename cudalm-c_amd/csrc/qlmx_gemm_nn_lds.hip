@@ -91,42 +91,6 @@ __device__ __forceinline__ bf16x8 nn3_pack(const i32x2 lo, const i32x2 hi){
 /* The second half of a gate|up problem: the other weight matrix, its output, the SwiGLU output. */
 struct Nn3Dual { unsigned long long wq, wg; float *C; unsigned short *act; };
 
-/* gate, up and bf16(gate * sigmoid(gate) * up) of a gate|up tile. The tile's 128 LDS columns are
- * [gate 0-31 | up 0-31 | gate 32-63 | up 32-63] of the problem's columns j0 .. j0+63, so a wavefront's first
- * accumulator column holds gate and its second holds up of the same 32 columns, element for element. */
-template<int NI>
-__device__ __forceinline__ void nn3_store_swiglu(const f32x16 (&acc)[NI][2], float *gp, float *up, unsigned short *act,
-                                                 int row, int rows, size_t ld){
-    typedef __attribute__((address_space(1))) float gfloat;
-    typedef __attribute__((address_space(1))) uint32_t guint;
-    const bool oddl = threadIdx.x & 1;
-#pragma unroll
-    for(int i = 0; i < NI; i++){
-        uint32_t a[16];
-#pragma unroll
-        for(int e = 0; e < 16; e++){
-            const int ro = i * 32 + (e >> 2) * 8 + (e & 3);
-            const float g = acc[i][0][e], u = acc[i][1][e];
-            a[e] = qx_f32_to_bf16(g * qx_fsig(g) * u);
-            if(row + ro < rows){
-                const size_t o = (size_t)ro * ld;
-                __builtin_nontemporal_store(g, (gfloat *)gp + o);
-                __builtin_nontemporal_store(u, (gfloat *)up + o);
-            }
-        }
-        /* two neighbouring columns per 4-byte store: the even lane of a pair writes the first eight of its
-         * rows for both, the odd lane the other eight */
-#pragma unroll
-        for(int e = 0; e < 8; e++){
-            const uint32_t got = (uint32_t)__shfl_xor((int)(oddl ? a[e] : a[e + 8]), 1, 64);
-            const int e2 = oddl ? e + 8 : e;
-            const int ro = i * 32 + (e2 >> 2) * 8 + (e2 & 3);
-            const uint32_t v = oddl ? (got | (a[e + 8] << 16)) : (a[e] | (got << 16));
-            if(row + ro < rows) *(guint *)(act + (size_t)ro * ld - (oddl ? 1 : 0)) = v;
-        }
-    }
-}
-
 template<int NI, bool DUAL = false>
 __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, const Nn3Dual &Q, int i0, int j0, unsigned char *lds){
     const int rows = P.M;
@@ -334,7 +298,7 @@ __device__ __forceinline__ void nn3_tile(const Nn3Args &a, const DevProb &P, con
     const int row = i0 + wi + hf * 4;
     if(DUAL){
         const size_t o = (size_t)row * a.N + (j0 + (wj >> 1) + fr);
-        nn3_store_swiglu<NI>(acc, P.C + o, Q.C + o, Q.act + o, row, rows, (size_t)a.N);
+        qx_store_swiglu<NI>(acc, P.C + o, Q.C + o, Q.act + o, row, rows, (size_t)a.N);
     } else
         qx_store_tiles<NI, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
 }

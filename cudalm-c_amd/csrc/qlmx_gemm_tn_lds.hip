@@ -37,7 +37,10 @@ typedef int    i32x4  __attribute__((ext_vector_type(4)));
 struct Tn3Seg { int nseg; long long dA, dW, dS; };
 /* out != NULL: the problems' C fields are row-index lists and the result is added to the indexed rows of `out`
  * (k_scatter_add4 behind the paired input-gradient GEMMs, cudalm.cu:4365-4367), see qx_scatter_tiles */
-struct Tn3Args { const DevProb *pr; int nprob, ntiles; const signed char *d; const float *s; int gshift; int K, N; float *out; const float *gate; };
+/* gp != NULL: k_swiglu_bwd behind the down projection's input gradient (cudalm.cu:4340-4346): the product is d(act);
+ * a problem's C field points at its rows of gp, and up, dg, du hold the same rows at the same element offset */
+struct Tn3Args { const DevProb *pr; int nprob, ntiles; const signed char *d; const float *s; int gshift; int K, N; float *out; const float *gate;
+                 const float *gp, *up; unsigned short *dg, *du; };
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void glb_void;
@@ -285,7 +288,10 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, con
     /* ---- epilogue: the lane holds column lane%32 of each 32x32 tile, four-row band lane/32 ---- */
     const int row = i0 + wi + hf * 4;
     if(a.out) qx_scatter_tiles<NI>(acc, (const int *)P.C, a.gate, a.out, row, rows, (size_t)a.N, j0 + wj + fr);
-    else qx_store_tiles<NI, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
+    else if(a.gp){
+        const size_t o = (size_t)(P.C - a.gp) + (size_t)row * a.N + (j0 + wj + fr);
+        qx_store_swiglu_bwd<NI>(acc, a.gp + o, a.up + o, a.dg + o, a.du + o, row, rows, (size_t)a.N);
+    } else qx_store_tiles<NI, 2>(acc, P.C + (size_t)row * a.N + (j0 + wj + fr), row, i0 + wi, rows, (size_t)a.N, P.beta != 0.0f);
 }
 
 __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
@@ -311,13 +317,15 @@ __global__ void __launch_bounds__(256, 2) k_gemm_tn_lds(Tn3Args a){
 
 /* bf16 activations only; N % 128 == 0, K % 64 == 0, group a power of two >= 64 (checked by the caller) */
 int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs,
-                            const qlmx_gemm_prob *second, int nprob, int K, int N, float *out, const float *gate, hipStream_t st){
+                            const qlmx_gemm_prob *second, int nprob, int K, int N, float *out, const float *gate,
+                            const float *gp, const float *up_, void *dg, void *du, hipStream_t st){
     ProbUpload up; int slot;
     int rc = second ? qlmx_upload_problem_pairs(probs, second, nprob, GEMM_TN, K, N, TN3_BM, TN3_BN, st, &up, &slot)
                     : qlmx_upload_problems(probs, nprob, GEMM_TN, K, N, TN3_BM, TN3_BN, st, &up, &slot);
     if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;
     Tn3Args a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.d = d; a.s = s; a.K = K; a.N = N; a.out = out; a.gate = gate;
+    a.gp = gp; a.up = up_; a.dg = (unsigned short *)dg; a.du = (unsigned short *)du;
     a.gshift = 0; while((1 << a.gshift) < group) a.gshift++;
     const int grid = (up.ntiles + 7) / 8 * 8;
     hipLaunchKernelGGL(k_gemm_tn_lds, dim3(grid), dim3(256), 0, st, a);

@@ -219,6 +219,11 @@ __global__ void __launch_bounds__(GP_CHUNK) k_gp_scatter(const int *asn, int N, 
     }
 }
 
+__global__ void __launch_bounds__(256) k_fill_i32(int *p, int v, int n){
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if(i < n) p[i] = v;
+}
+
 /* ---- row movers. One workgroup per row; D % 4 == 0. ---- */
 template<bool OUT_BF16>
 __global__ void __launch_bounds__(256) k_gather_rows(const float4 *src, const int *perm, void *Xp, int D4){
@@ -261,9 +266,11 @@ __global__ void __launch_bounds__(256) k_scatter_add(const float4 *dXp, const in
 /* d_gate[n] = dout[n,:] . yp[j,:];  dyp[j,:] = gate[n] * dout[n,:] */
 template<bool OUT_BF16>
 __global__ void __launch_bounds__(256) k_moe_dgate(const float4 *dout, const float4 *yp, const int *perm, const float *gate,
-                                                   float *d_gate, void *dyp, int D4){
+                                                   float *d_gate, void *dyp, int D4, int tokens){
     __shared__ float red[4];
-    const int j = blockIdx.x, n = perm[j];
+    /* one pass (tokens = 0): perm names the token, which also indexes gate and d_gate; all passes as one grouped
+     * list: perm names pass * tokens + token, which indexes gate and d_gate, and the token is the remainder */
+    const int j = blockIdx.x, m = perm[j], n = (tokens && m >= 0) ? m % tokens : m;
     if(n < 0){
         for(int d = threadIdx.x; d < D4; d += 256){
             if(OUT_BF16) ((uint2 *)dyp)[(size_t)j * D4 + d] = make_uint2(0u, 0u);
@@ -272,7 +279,7 @@ __global__ void __launch_bounds__(256) k_moe_dgate(const float4 *dout, const flo
         return;
     }
     const float4 *dr = dout + (size_t)n * D4, *y = yp + (size_t)j * D4;
-    const float g = gate[n];
+    const float g = gate[m];
     float acc = 0.0f;
     for(int d = threadIdx.x; d < D4; d += 256){
         const float4 a = dr[d], b = y[d];
@@ -288,7 +295,36 @@ __global__ void __launch_bounds__(256) k_moe_dgate(const float4 *dout, const flo
     acc = qx_wave_sum(acc);
     if((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
     __syncthreads();
-    if(threadIdx.x == 0) d_gate[n] = (red[0] + red[1]) + (red[2] + red[3]);
+    if(threadIdx.x == 0) d_gate[m] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+/* ---- all K passes as ONE expert-grouped list of K*N rows (the reference's merged top-K, cudalm.cu:3532-3561,
+ * 4022-4034): the grouping permutation of the K*N assignments names entries m = pass * N + token; row p of the
+ * grouped buffers holds token perm[p] % N, and inv[m] is the row that holds entry m. ---- */
+__global__ void __launch_bounds__(256) k_merge_rows(const int *perm, int KN, int N, int *tok, int *inv){
+    const int p = blockIdx.x * 256 + threadIdx.x;
+    if(p >= KN) return;
+    const int m = perm[p];
+    tok[p] = m < 0 ? -1 : m % N;
+    if(m >= 0) inv[m] = p;
+}
+/* out[n,:] = (..(out[n,:] + g[0*N+n] * y[inv[0*N+n],:]) + ..) + g[(K-1)*N+n] * y[inv[(K-1)*N+n],:], pass after pass:
+ * the sums the per-pass scatters build, in their order (g NULL: plain additions; inv < 0: the pass dropped the token) */
+__global__ void __launch_bounds__(256) k_combine(const float4 *y, const int *inv, const float *g, float4 *out, int N, int K, int D4){
+    const int n = blockIdx.x;
+    float4 *o = out + (size_t)n * D4;
+    for(int d = threadIdx.x; d < D4; d += 256){
+        float4 a = o[d];
+        for(int k = 0; k < K; k++){
+            const size_t i = (size_t)k * N + n;
+            const int p = inv[i];
+            if(p < 0) continue;
+            const float4 b = y[(size_t)p * D4 + d];
+            if(g){ const float w = g[i]; a.x = a.x + w * b.x; a.y = a.y + w * b.y; a.z = a.z + w * b.z; a.w = a.w + w * b.w; }
+            else { a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w; }
+        }
+        o[d] = a;
+    }
 }
 
 /* ---- SwiGLU between the GEMMs: O = g * sigmoid(g) * u with the polynomial sigmoid ---- */
@@ -307,18 +343,14 @@ __global__ void __launch_bounds__(256) k_swiglu(const float4 *G, const float4 *U
         ((uint2 *)O)[i] = p;
     } else ((float4 *)O)[i] = o;
 }
-__device__ __forceinline__ void swiglu_bwd1(float z, float u, float da, float &dg, float &du){
-    const float sg = qx_fsig(z), silu = z * sg, ds = sg + z * sg * (1.0f - sg);
-    dg = da * u * ds; du = da * silu;
-}
 template<bool OUT_BF16>
 __global__ void __launch_bounds__(256) k_swiglu_bwd(const float4 *Gg, const float4 *U, const float4 *dact, void *dg, void *du, size_t n4){
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if(i >= n4) return;
     const float4 g = Gg[i], u = U[i], a = dact[i];
     float4 x, y;
-    swiglu_bwd1(g.x, u.x, a.x, x.x, y.x); swiglu_bwd1(g.y, u.y, a.y, x.y, y.y);
-    swiglu_bwd1(g.z, u.z, a.z, x.z, y.z); swiglu_bwd1(g.w, u.w, a.w, x.w, y.w);
+    qx_swiglu_bwd1(g.x, u.x, a.x, x.x, y.x); qx_swiglu_bwd1(g.y, u.y, a.y, x.y, y.y);
+    qx_swiglu_bwd1(g.z, u.z, a.z, x.z, y.z); qx_swiglu_bwd1(g.w, u.w, a.w, x.w, y.w);
     if(OUT_BF16){
         uint2 p, q;
         p.x = (uint32_t)qx_f32_to_bf16(x.x) | ((uint32_t)qx_f32_to_bf16(x.y) << 16);
@@ -438,9 +470,50 @@ extern "C" int qlmx_moe_dgate(const float *dout, const float *yp, const int *per
     QLMX_REQUIRE(GLUE_ALIGN16(dout) && GLUE_ALIGN16(yp) && GLUE_ALIGN16(dyp), "qlmx_moe_dgate: buffers must be 16-byte aligned");
     QLMX_REQUIRE(out_dtype == QLMX_ACT_F32 || out_dtype == QLMX_ACT_BF16, "qlmx_moe_dgate: unknown output type %d", out_dtype);
     if(N <= 0) return QLMX_OK;
-    if(out_dtype == QLMX_ACT_BF16) hipLaunchKernelGGL(k_moe_dgate<true>, dim3(N), dim3(256), 0, (hipStream_t)stream, (const float4 *)dout, (const float4 *)yp, perm, gate, d_gate, dyp, D / 4);
-    else                           hipLaunchKernelGGL(k_moe_dgate<false>, dim3(N), dim3(256), 0, (hipStream_t)stream, (const float4 *)dout, (const float4 *)yp, perm, gate, d_gate, dyp, D / 4);
+    if(out_dtype == QLMX_ACT_BF16) hipLaunchKernelGGL(k_moe_dgate<true>, dim3(N), dim3(256), 0, (hipStream_t)stream, (const float4 *)dout, (const float4 *)yp, perm, gate, d_gate, dyp, D / 4, 0);
+    else                           hipLaunchKernelGGL(k_moe_dgate<false>, dim3(N), dim3(256), 0, (hipStream_t)stream, (const float4 *)dout, (const float4 *)yp, perm, gate, d_gate, dyp, D / 4, 0);
     QLMX_LAUNCH_CHECK("dgate launch");
+    return QLMX_OK;
+}
+
+/* ---- merged passes ---- */
+extern "C" int qlmx_moe_merge_rows(const int *perm, int N, int K, int *tok, int *inv, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(perm && tok && inv, "qlmx_moe_merge_rows: NULL buffer");
+    QLMX_REQUIRE(N > 0 && K > 0 && (long long)N * K < (1LL << 31), "qlmx_moe_merge_rows: N=%d K=%d", N, K);
+    const int KN = N * K;
+    /* rows a caller dropped (perm < 0) leave no inverse: -1 everywhere first, by a kernel so that a capture holds no memset node */
+    hipLaunchKernelGGL(k_fill_i32, dim3((KN + 255) / 256), dim3(256), 0, (hipStream_t)stream, inv, -1, KN);
+    QLMX_LAUNCH_CHECK("merge rows: inverse fill");
+    hipLaunchKernelGGL(k_merge_rows, dim3((KN + 255) / 256), dim3(256), 0, (hipStream_t)stream, perm, KN, N, tok, inv);
+    QLMX_LAUNCH_CHECK("merge rows launch");
+    return QLMX_OK;
+}
+
+extern "C" int qlmx_moe_combine(const float *y, const int *inv, const float *gate, float *out, int N, int K, int D, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(y && inv && out, "qlmx_moe_combine: NULL buffer");
+    GLUE_ROWS_CHECK("qlmx_moe_combine", D);
+    QLMX_REQUIRE(K > 0 && GLUE_ALIGN16(y) && GLUE_ALIGN16(out), "qlmx_moe_combine: K=%d, buffers must be 16-byte aligned", K);
+    if(N <= 0) return QLMX_OK;
+    hipLaunchKernelGGL(k_combine, dim3(N), dim3(256), 0, (hipStream_t)stream, (const float4 *)y, inv, gate, (float4 *)out, N, K, D / 4);
+    QLMX_LAUNCH_CHECK("combine launch");
+    return QLMX_OK;
+}
+
+extern "C" int qlmx_moe_dgate_merged(const float *dout, const float *yp, const int *perm, const float *gate,
+                                     float *d_gate, void *dyp, int N, int K, int D, int out_dtype, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(dout && yp && perm && gate && d_gate && dyp, "qlmx_moe_dgate_merged: NULL buffer");
+    GLUE_ROWS_CHECK("qlmx_moe_dgate_merged", D);
+    QLMX_REQUIRE(GLUE_ALIGN16(dout) && GLUE_ALIGN16(yp) && GLUE_ALIGN16(dyp), "qlmx_moe_dgate_merged: buffers must be 16-byte aligned");
+    QLMX_REQUIRE(out_dtype == QLMX_ACT_F32 || out_dtype == QLMX_ACT_BF16, "qlmx_moe_dgate_merged: unknown output type %d", out_dtype);
+    QLMX_REQUIRE(K > 0 && (long long)N * K < (1LL << 31), "qlmx_moe_dgate_merged: N=%d K=%d", N, K);
+    if(N <= 0) return QLMX_OK;
+    const int KN = N * K;
+    if(out_dtype == QLMX_ACT_BF16) hipLaunchKernelGGL(k_moe_dgate<true>, dim3(KN), dim3(256), 0, (hipStream_t)stream, (const float4 *)dout, (const float4 *)yp, perm, gate, d_gate, dyp, D / 4, N);
+    else                           hipLaunchKernelGGL(k_moe_dgate<false>, dim3(KN), dim3(256), 0, (hipStream_t)stream, (const float4 *)dout, (const float4 *)yp, perm, gate, d_gate, dyp, D / 4, N);
+    QLMX_LAUNCH_CHECK("merged dgate launch");
     return QLMX_OK;
 }
 

@@ -206,6 +206,24 @@ int qlmx_moe_gemm_nn_scatter(const signed char *d, const float *s, int group,
 int qlmx_moe_gemm_tn_pair_scatter(const signed char *d, const float *s, int group,
                                   const qlmx_gemm_prob *first_host, const qlmx_gemm_prob *second_host, int nprob, int K, int N,
                                   float *dst, void *stream);
+/* The SwiGLU and its gradient folded into the GEMMs next to them (fp16 forward kernel, bf16 input-gradient kernel;
+ * element for element the operations of qlmx_swiglu / qlmx_swiglu_bwd, so results equal the separate calls bit for bit):
+ *   qlmx_moe_gemm_nn_swiglu with QLMX_MATH_MFMA_F16: as documented above on the fp16 matrix core; gate[i].C and
+ *     up[i].C may then both be NULL, and only the bf16 SwiGLU output up[i].B is written (a forward pass that does
+ *     not keep gp / up for the backward: cudalm.cu:4211-4215 with the stash off).
+ *   qlmx_moe_gemm_nn_gather_swiglu: the same with the gather in front (cudalm.cu:4209-4215): gate[i].A are
+ *     row-index lists into the bf16 token matrix x, as in qlmx_moe_gemm_nn_gather. N % 64 == 0, K % 32 == 0,
+ *     group 64, 128 or 256, at most QLMX_MAX_PROBLEMS / 2 problems.
+ *   qlmx_moe_gemm_tn_swiglu_bwd: mg_abt of the down projection + e_swigb (cudalm.cu:4340-4346): the product
+ *     d(act) = A . W^T is not stored; probs[i].C points at the problem's rows INSIDE gp (the forward's fp32 gate
+ *     pre-activations), and with o = probs[i].C - gp the kernel reads gp[o ..], up[o ..] and writes the bf16
+ *     gradients dgp[o ..], dup[o ..] ([rows, N] each, the four buffers laid out alike). */
+int qlmx_moe_gemm_nn_gather_swiglu(const signed char *d, const float *s, int group,
+                                   const qlmx_gemm_prob *gate_host, const qlmx_gemm_prob *up_host, int nprob, int K, int N,
+                                   const void *x_bf16, void *stream);
+int qlmx_moe_gemm_tn_swiglu_bwd(const signed char *d, const float *s, int group,
+                                const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
+                                const float *gp, const float *up, void *dgp_bf16, void *dup_bf16, void *stream);
 /* nt: no weight operand; both inputs are activations, fp32 result. beta = 1 reproduces the
  * reference's accumulation into a zeroed G; beta = 0 saves the read when G is known to be fresh. */
 int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
@@ -288,6 +306,21 @@ int qlmx_moe_scatter_add(const float *dXp, const int *perm, float *dst, int N, i
 /* k_moe_dgate (cudalm.cu:2591; cpu_kern.h:454-468): d_gate[n] = dout[n,:] . yp[j,:], dyp[j,:] = gate[n] * dout[n,:], n = perm[j] */
 int qlmx_moe_dgate(const float *dout, const float *yp, const int *perm, const float *gate,
                    float *d_gate, void *dyp, int N, int D, int out_dtype, void *stream);
+/* All K passes of a layer as ONE expert-grouped list of K*N rows (the reference's merged top-K: moe_gperm with
+ * mrg, k_gather_bfm, k_combine_bf, k_moe_dgate_bfm; cudalm.cu:3532-3561, 4022-4047), so that every grouped GEMM
+ * runs once per layer on K times the rows instead of once per pass. The grouping itself is qlmx_moe_perm over the
+ * K*N assignments as a single pass (N' = K*N, K' = 1): its perm names entries m = pass * N + token.
+ *   qlmx_moe_merge_rows: tok[p] = perm[p] % N (the token row p holds; what a gather or a gathering GEMM takes as
+ *     its index list) and inv[m] = the row that holds entry m (-1 if none), both int32 [K*N].
+ *   qlmx_moe_combine: out[n,:] = (..(out[n,:] + gate[0*N+n] * y[inv[0*N+n],:]) ..) + gate[(K-1)*N+n] * y[inv[(K-1)*N+n],:]
+ *     -- the sums that K calls of qlmx_moe_scatter_gate build, in their order and to their bits; gate NULL adds
+ *     the rows themselves (K calls of qlmx_moe_scatter_add). y fp32 [K*N, D].
+ *   qlmx_moe_dgate_merged: qlmx_moe_dgate over the grouped list: row j holds entry m = perm[j], token n = m % N;
+ *     d_gate[m] = dout[n,:] . yp[j,:], dyp[j,:] = gate[m] * dout[n,:]. */
+int qlmx_moe_merge_rows(const int *perm, int N, int K, int *tok, int *inv, void *stream);
+int qlmx_moe_combine(const float *y, const int *inv, const float *gate, float *out, int N, int K, int D, void *stream);
+int qlmx_moe_dgate_merged(const float *dout, const float *yp, const int *perm, const float *gate,
+                          float *d_gate, void *dyp, int N, int K, int D, int out_dtype, void *stream);
 /* k_swiglu / k_swiglu_bwd (cudalm.cu:2430-2453; cpu_kern.h:376-394): O = g*sigmoid(g)*u and its
  * gradient (dg, du) from dact, with the CPU build's polynomial sigmoid. n % 4 == 0. */
 int qlmx_swiglu(const float *G, const float *U, void *O, size_t n, int out_dtype, void *stream);

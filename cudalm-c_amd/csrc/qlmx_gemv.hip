@@ -340,8 +340,7 @@ __device__ __forceinline__ void df_st(u64 *p, float v, unsigned epoch){
 /* Sums of S tagged partial sums `stride` words apart from each of NSRC sources, in slice order;
  * re-reads until every word carries `epoch`. All loads of a pass are issued before the first is
  * looked at. */
-#define DF_SLICE_STEP 4
-template<int NSRC>
+template<int NSRC, int DF_SLICE_STEP>
 __device__ __forceinline__ void df_sum_wait(const u64 *const (&src)[NSRC], size_t stride, int S, unsigned epoch, int limit,
                                             volatile int *giveup, unsigned *status, float (&v)[NSRC]){
     int spins = 0;
@@ -509,28 +508,27 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
     __shared__ __align__(16) float xs[DF_NG][DF_RMAX][DF_MB];   /* x[m][r] * scale(r, g), the four m side by side */
     __shared__ float red[4 * DF_MB * DF_CW];
     __shared__ int giveup;
-    __shared__ unsigned tag;
     const int tid = threadIdx.x;
     /* The tag of this call's partial sums is one more than the last finished call's, which lives in
      * device memory: the host passes no counter, so a launch recorded in a graph tags every replay
      * afresh. Every workgroup reads the word here; the last workgroup to finish moves it on (end of
      * the kernel), which cannot happen before all of them have read it. 0 is the cleared state. */
-    if(tid == 0){
-        giveup = 0;
-        const unsigned last = __hip_atomic_load(a.ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        tag = last == 0xFFFFFFFFu ? 1u : last + 1u;
-    }
     const int npair = a.T * a.K;
     const int ng = a.group >= DF_CW ? 1 : DF_CW / a.group;
+    /* the two first loads -- the pairs' experts and the tag -- are both on their way before either is used
+     * (under branches they went one after the other, a memory round trip each) */
+    const int e_in = a.assign[min(tid, npair - 1)];
+    const unsigned last = __hip_atomic_load(a.ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if(tid == 0) giveup = 0;
 
     /* ---- problem table (identical in every workgroup): rank of pair j among (expert, j) ---- */
     if(tid < DEC_MAXPAIR){
-        int e = 0x7FFFFFFF;
-        if(tid < npair){ e = a.assign[tid]; if((unsigned)e >= (unsigned)a.E) e = 0x7FFFFFFE; }   /* invalid: sorts after every valid expert */
+        int e = tid < npair ? e_in : 0x7FFFFFFF;
+        if(tid < npair && (unsigned)e >= (unsigned)a.E) e = 0x7FFFFFFE;   /* invalid: sorts after every valid expert */
         mt.ein[tid] = e;
     }
     __syncthreads();
-    a.epoch = __builtin_amdgcn_readfirstlane(tag);
+    a.epoch = __builtin_amdgcn_readfirstlane(last == 0xFFFFFFFFu ? 1u : last + 1u);
     {
         const int j = tid & 63, part = tid >> 6, e = mt.ein[j];
         int rank = 0;
@@ -633,41 +631,41 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
         auto prep = [&](){
             if(cur.list == 1){
                 __syncthreads();                             /* the previous task is done with xs */
-                if(tid < rows){
+                for(int r = tid; r < rows; r += DF_THREADS){
                     float sc[DF_NG], xv[DF_MB];
 #pragma unroll
-                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = gg < ng ? df_scale(a, srow0, gpr, a.F, tid, chunk, gg) : 0.0f;
+                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = gg < ng ? df_scale(a, srow0, gpr, a.F, r, chunk, gg) : 0.0f;
 #pragma unroll
                     for(int m = 0; m < DF_MB; m++)
-                        xv[m] = m < M ? a.x[(size_t)(mt.rowpair[mt.p_row0[prob] + m] % a.T) * a.D + k0 + tid] : 0.0f;
+                        xv[m] = m < M ? a.x[(size_t)(mt.rowpair[mt.p_row0[prob] + m] % a.T) * a.D + k0 + r] : 0.0f;
 #pragma unroll
                     for(int gg = 0; gg < DF_NG; gg++)
-                        *(float4 *)&xs[gg][tid][0] = make_float4(xv[0] * sc[gg], xv[1] * sc[gg], xv[2] * sc[gg], xv[3] * sc[gg]);
+                        *(float4 *)&xs[gg][r][0] = make_float4(xv[0] * sc[gg], xv[1] * sc[gg], xv[2] * sc[gg], xv[3] * sc[gg]);
                 }
                 __syncthreads();
             } else {
                 const u64 *p1 = a.part1 + (((size_t)prob * 2) * a.S1 * DF_MB) * a.F + k0;
                 const size_t sstride = (size_t)DF_MB * a.F;
                 df_wait_first(2 * a.S1, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, [=](int i){ return p1 + (size_t)i * sstride; });
-                if(tid < rows){
+                for(int r = tid; r < rows; r += DF_THREADS){
                     float sc[DF_NG];
 #pragma unroll
-                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = gg < ng ? df_scale(a, srow0, gpr, a.D, tid, chunk, gg) : 0.0f;
+                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = gg < ng ? df_scale(a, srow0, gpr, a.D, r, chunk, gg) : 0.0f;
                     float hv[DF_MB];
 #pragma unroll
                     for(int m = 0; m < DF_MB; m++){
                         hv[m] = 0.0f;
                         if(m < M){
                             /* h = silu(gate) * up (k_swiglu, cudalm.cu:2430-2432), both summed over the K slices in order */
-                            const u64 *const src[2] = { p1 + (size_t)m * a.F + tid, p1 + (size_t)a.S1 * sstride + (size_t)m * a.F + tid };
+                            const u64 *const src[2] = { p1 + (size_t)m * a.F + r, p1 + (size_t)a.S1 * sstride + (size_t)m * a.F + r };
                             float gu[2];
-                            df_sum_wait<2>(src, sstride, a.S1, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, gu);
+                            df_sum_wait<2, 6>(src, sstride, a.S1, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, gu);
                             hv[m] = (gu[0] / (1.0f + expf(-gu[0]))) * gu[1];
                         }
                     }
 #pragma unroll
                     for(int gg = 0; gg < DF_NG; gg++)
-                        *(float4 *)&xs[gg][tid][0] = make_float4(hv[0] * sc[gg], hv[1] * sc[gg], hv[2] * sc[gg], hv[3] * sc[gg]);
+                        *(float4 *)&xs[gg][r][0] = make_float4(hv[0] * sc[gg], hv[1] * sc[gg], hv[2] * sc[gg], hv[3] * sc[gg]);
                 }
                 __syncthreads();
             }
@@ -699,7 +697,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
                     if(prob < 0) continue;
                     const u64 *const src[1] = { a.part2 + (((size_t)prob * a.S2) * DF_MB + mt.pair_m[j]) * a.D + col };
                     float y[1];
-                    df_sum_wait<1>(src, (size_t)DF_MB * a.D, a.S2, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, y);
+                    df_sum_wait<1, 12>(src, (size_t)DF_MB * a.D, a.S2, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, y);
                     o = o + a.gate[j] * y[0];
                 }
                 a.out[(size_t)n * a.D + col] = o;
@@ -780,7 +778,7 @@ static int df_reserve(DfSpace &ws, int which, size_t words, hipStream_t st){
     return QLMX_OK;
 }
 
-/* rows per task: 256 keeps the per-task fixed cost (staging, reduction, hand-over) small against
+/* Rows per task of list 1: 256 keeps the per-task fixed cost (staging, reduction, hand-over) small against
  * the streaming part; only when even that leaves most of the grid without a gate|up task (a single
  * token) are the slices halved. The number of problems is only known on the device; the host uses
  * the expected number of distinct experts hit by `npair` uniform picks out of E. */
@@ -788,6 +786,19 @@ static int df_rows(int Kdim, double tasks_per_slice, int grid){
     int R = DF_RMAX;
     while(R > 64 && tasks_per_slice * ((Kdim + R - 1) / R) < 0.25 * grid) R >>= 1;
     while((Kdim + R - 1) / R > 32 && R < DF_RMAX) R <<= 1;
+    return R;
+}
+/* Rows per task of list 2 (a multiple of 32): as many slices of the contraction as still leave one task per
+ * resident workgroup -- a second round of tasks would double the list's time -- but at most 12, which is what
+ * the combine reads in one round trip, and none shorter than 64 rows. */
+static int df_rows_down(int Kdim, double tasks_per_slice, int grid){
+    int S = tasks_per_slice > 0.0 ? (int)(0.95 * grid / tasks_per_slice) : 1;
+    const int smin = (Kdim + DF_RMAX - 1) / DF_RMAX, smax = Kdim >= 64 ? Kdim / 64 : 1;
+    if(S > 12) S = 12;
+    if(S > smax) S = smax;
+    if(S < smin) S = smin;
+    int R = ((Kdim + S - 1) / S + 31) & ~31;
+    if(R > DF_RMAX) R = DF_RMAX;
     return R;
 }
 
@@ -821,7 +832,7 @@ static int df_forward(bool fixed, const char *who, const float *x, const int *as
     a.NC1 = (F + DF_CW - 1) / DF_CW; a.NC2 = (D + DF_CW - 1) / DF_CW;
     const double hits = E * (1.0 - pow(1.0 - 1.0 / E, (double)npair));
     a.R1 = df_rows(D, 2.0 * hits * a.NC1, dv.grid); a.S1 = (D + a.R1 - 1) / a.R1;
-    a.R2 = DF_RMAX;                                  a.S2 = (F + a.R2 - 1) / a.R2;
+    a.R2 = df_rows_down(F, hits * a.NC2, dv.grid);   a.S2 = (F + a.R2 - 1) / a.R2;
     const size_t words1 = (size_t)npair * 2 * a.S1 * DF_MB * F, words2 = (size_t)npair * a.S2 * DF_MB * D;
     if(fixed){
         if((words1 + words2) * sizeof(u64) > (size_t)QLMX_DECODE_SCRATCH_BYTES){

@@ -21,19 +21,32 @@
  */
 #include "qlmx_gemm.h"
 #include <algorithm>
+#include <stdlib.h>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short  s16x4  __attribute__((ext_vector_type(4)));
 typedef short  s16x8  __attribute__((ext_vector_type(8)));
 typedef float  f32x16 __attribute__((ext_vector_type(16)));
 
+/* Two tile shapes, one kernel body (template parameter BN = columns of dY per tile):
+ *   256 x 128: four wavefronts of 128 x 64, two workgroups per CU (256 registers each);
+ *   256 x 256: four wavefronts of 128 x 128, one workgroup per CU, the 256 accumulator registers of a
+ *              wavefront in the accumulation half of its 512: a third fewer LDS bytes read and a third fewer
+ *              bytes brought into LDS per multiplication, but nothing else resident on the CU to cover a
+ *              workgroup's waits, prologue and epilogue. Not faster as measured (see nt3_pick_bn); opt-in. */
 #define NT3_BM 256
-#define NT3_BN 128
 #define NT3_BK 32
 #define NT3_STAGES 3
 #define NT3_A_BYTES (NT3_BK * NT3_BM * 2)      /* 16384 */
-#define NT3_B_BYTES (NT3_BK * NT3_BN * 2)      /*  8192 */
-#define NT3_STAGE_BYTES (NT3_A_BYTES + NT3_B_BYTES)
+template<int BN> struct Nt3Shape {
+    static constexpr int NJ = BN / 64;                       /* 32-column accumulator tiles per wavefront */
+    static constexpr int NB = BN / 64;                       /* 16-byte pieces of dY a thread fetches per tile */
+    static constexpr int B_BYTES = NT3_BK * BN * 2;
+    static constexpr int STAGE_BYTES = NT3_A_BYTES + B_BYTES;
+    static constexpr int NREQ = 4 + NB;                      /* requests per thread and tile */
+    static constexpr int LDS_BYTES = NT3_STAGES * STAGE_BYTES;
+    static constexpr int WG_PER_CU = BN == 128 ? 2 : 1;
+};
 
 struct Nt3Args { const DevProb *pr; const DevUnit *units; int *flags; unsigned *status; unsigned epoch;
                  unsigned wait_epoch; int wait_limit;      /* what a slice waits for (= epoch) and for how many polls */
@@ -55,23 +68,29 @@ template<int OFF> __device__ __forceinline__ i32x2 nt3_tr(uint32_t addr){
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
     return v;
 }
-struct Nt3Ops { i32x2 a[4][2], b[2][2]; };
-template<int KS> __device__ __forceinline__ void nt3_read(Nt3Ops &o, const uint32_t (&adA)[4], const uint32_t (&adB)[2]){
+template<int NJ> struct Nt3Ops { i32x2 a[4][2], b[NJ][2]; };
+template<int KS, int BN, int NJ> __device__ __forceinline__ void nt3_read(Nt3Ops<NJ> &o, const uint32_t (&adA)[4], const uint32_t (&adB)[NJ]){
 #pragma unroll
     for(int i = 0; i < 4; i++){
         o.a[i][0] = nt3_tr<KS * 16 * NT3_BM * 2>(adA[i]);
         o.a[i][1] = nt3_tr<KS * 16 * NT3_BM * 2 + 4 * NT3_BM * 2>(adA[i]);
     }
 #pragma unroll
-    for(int j = 0; j < 2; j++){
-        o.b[j][0] = nt3_tr<KS * 16 * NT3_BN * 2>(adB[j]);
-        o.b[j][1] = nt3_tr<KS * 16 * NT3_BN * 2 + 4 * NT3_BN * 2>(adB[j]);
+    for(int j = 0; j < NJ; j++){
+        o.b[j][0] = nt3_tr<KS * 16 * BN * 2>(adB[j]);
+        o.b[j][1] = nt3_tr<KS * 16 * BN * 2 + 4 * BN * 2>(adB[j]);
     }
 }
-__device__ __forceinline__ void nt3_wait_reads(Nt3Ops &o){
+__device__ __forceinline__ void nt3_wait_reads(Nt3Ops<2> &o){
     asm volatile("s_waitcnt lgkmcnt(0)"
         : "+v"(o.a[0][0]), "+v"(o.a[0][1]), "+v"(o.a[1][0]), "+v"(o.a[1][1]), "+v"(o.a[2][0]), "+v"(o.a[2][1]),
           "+v"(o.a[3][0]), "+v"(o.a[3][1]), "+v"(o.b[0][0]), "+v"(o.b[0][1]), "+v"(o.b[1][0]), "+v"(o.b[1][1]));
+}
+__device__ __forceinline__ void nt3_wait_reads(Nt3Ops<4> &o){
+    asm volatile("s_waitcnt lgkmcnt(0)"
+        : "+v"(o.a[0][0]), "+v"(o.a[0][1]), "+v"(o.a[1][0]), "+v"(o.a[1][1]), "+v"(o.a[2][0]), "+v"(o.a[2][1]),
+          "+v"(o.a[3][0]), "+v"(o.a[3][1]), "+v"(o.b[0][0]), "+v"(o.b[0][1]), "+v"(o.b[1][0]), "+v"(o.b[1][1]),
+          "+v"(o.b[2][0]), "+v"(o.b[2][1]), "+v"(o.b[3][0]), "+v"(o.b[3][1]));
 }
 __device__ __forceinline__ bf16x8 nt3_pack(const i32x2 lo, const i32x2 hi){
     const i32x4 v = {lo[0], lo[1], hi[0], hi[1]};
@@ -82,8 +101,11 @@ __device__ __forceinline__ int t_of(int b, const Nt3Args &a){
     return (a.rows_p & 7) ? qx_xcd_tile_probs(b, a.tiles_n, a.rows_p) : qx_xcd_tile_rows(b, a.tiles_n);
 }
 
-__global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
-    __shared__ __attribute__((aligned(16))) unsigned char lds[NT3_STAGES * NT3_STAGE_BYTES];
+template<int BN>
+__global__ void __launch_bounds__(256, Nt3Shape<BN>::WG_PER_CU) k_gemm_nt_lds(Nt3Args a){
+    typedef Nt3Shape<BN> SH;
+    constexpr int NJ = SH::NJ, NB = SH::NB;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     /* scheduled launch: the unit table says what to do; otherwise the tile follows from the index */
     int pi, i0, j0, k0 = 0, depth = -1, seq = 0, nseq = 1, flag = 0;
     DevUnit u = QX_UNIT_NONE;
@@ -102,20 +124,20 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
     if(a.units){
         const int ti = (u >> 16) & 63, tj = (int)(blockIdx.x >> 3) % a.tiles_n;
         seq = (u >> 4) & 15; nseq = u & 15;
-        i0 = ti * NT3_BM; j0 = tj * NT3_BN; k0 = seq * P.chunk;
+        i0 = ti * NT3_BM; j0 = tj * BN; k0 = seq * P.chunk;
         depth = P.M - k0 < P.chunk ? P.M - k0 : P.chunk;
         flag = P.flag0 + ti * P.tiles_n + tj;
     } else {
         const int lt = t_of(blockIdx.x, a) - P.tile0;
         const int ti = lt / P.tiles_n, tj = lt - ti * P.tiles_n;
-        i0 = ti * NT3_BM; j0 = tj * NT3_BN; depth = P.M;
+        i0 = ti * NT3_BM; j0 = tj * BN; depth = P.M;
     }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wi = (wave >> 1) * 128, wj = (wave & 1) * 64;
+    const int wi = (wave >> 1) * 128, wj = (wave & 1) * (BN / 2);
 
     /* ---- what this thread fetches per tile: four 16-byte pieces of X, two of dY. Piece p of a tile
      * (LDS position 16*p) is row p/32 (p/16 for dY), stored unit p%32 = logical unit ^ swizzle. ---- */
-    const char *srcA[4]; const char *srcB[2]; int rowA[4], rowB[2];
+    const char *srcA[4]; const char *srcB[NB]; int rowA[4], rowB[NB];
 #pragma unroll
     for(int h = 0; h < 4; h++){
         const int p = h * 256 + tid, row = p >> 5, lu = (p & 31) ^ ((row & 3) << 2);
@@ -124,8 +146,8 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
         srcA[h] = (const char *)P.A + ((size_t)(k0 + row) * a.K + (col < a.K ? col : 0)) * 2;   /* columns past K feed rows that are never stored */
     }
 #pragma unroll
-    for(int h = 0; h < 2; h++){
-        const int p = h * 256 + tid, row = p >> 4, lu = (p & 15) ^ ((row & 3) << 2);
+    for(int h = 0; h < NB; h++){
+        const int p = h * 256 + tid, row = p / (BN / 8), lu = (p & (BN / 8 - 1)) ^ ((row & 3) << 2);
         rowB[h] = row;
         srcB[h] = (const char *)P.B + ((size_t)(k0 + row) * a.N + j0 + lu * 8) * 2;
     }
@@ -135,7 +157,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
     /* request h of a tile: 0..3 are the X pieces, 4..5 the dY pieces */
     auto issue_one = [&](int tile, int stage, int h){
         const int kt = tile * NT3_BK;
-        unsigned char *base = lds + stage * NT3_STAGE_BYTES + wave_off;
+        unsigned char *base = lds + stage * SH::STAGE_BYTES + wave_off;
         if(h < 4){
             const char *g = (kt + rowA[h] < depth) ? srcA[h] + (size_t)tile * stepA : (const char *)a.zeros;
             __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(base + h * 4096), 16, 0, 0);
@@ -146,68 +168,71 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
     };
     auto issue = [&](int tile, int stage){
 #pragma unroll
-        for(int h = 0; h < 6; h++) issue_one(tile, stage, h);
+        for(int h = 0; h < SH::NREQ; h++) issue_one(tile, stage, h);
     };
 
     /* ---- operand read addresses inside a stage (k16 slice 0; slice 1 is 16 rows further) ---- */
     const int g16 = lane >> 4, s16 = lane & 15, v = s16 >> 2, q = s16 & 3, khalf = g16 >> 1, chalf = g16 & 1;
     const int row0 = khalf * 8 + v;                         /* + 4 for the second read, + 16 for slice 1: row & 3 unchanged */
     const int sw = (row0 & 3) << 2;
-    uint32_t offA[4], offB[2];
+    uint32_t offA[4], offB[NJ];
 #pragma unroll
     for(int i = 0; i < 4; i++){
         const int col = wi + i * 32 + chalf * 16 + q * 4;
         offA[i] = row0 * (NT3_BM * 2) + ((((col >> 3) ^ sw)) << 4) + (col & 7) * 2;
     }
 #pragma unroll
-    for(int j = 0; j < 2; j++){
+    for(int j = 0; j < NJ; j++){
         const int col = wj + j * 32 + chalf * 16 + q * 4;
-        offB[j] = NT3_A_BYTES + row0 * (NT3_BN * 2) + ((((col >> 3) ^ sw)) << 4) + (col & 7) * 2;
+        offB[j] = NT3_A_BYTES + row0 * (BN * 2) + ((((col >> 3) ^ sw)) << 4) + (col & 7) * 2;
     }
 
-    f32x16 acc[4][2];
+    f32x16 acc[4][NJ];
 #pragma unroll
     for(int i = 0; i < 4; i++)
 #pragma unroll
-        for(int j = 0; j < 2; j++) acc[i][j] = (f32x16)(0.0f);
+        for(int j = 0; j < NJ; j++) acc[i][j] = (f32x16)(0.0f);
 
     const int steps = (depth + NT3_BK - 1) / NT3_BK;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
-    issue(0, 0);
-    issue(1, 1);
-    for(int st = 0; st < steps; st++){
-        /* tile st has landed once at most the 6 requests of tile st+1 are still in flight */
-        asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-        __builtin_amdgcn_s_barrier();                       /* everybody's pieces are in; stage (st+2)%3 is free again */
-        const uint32_t sb = lds_base + (uint32_t)(st % NT3_STAGES) * NT3_STAGE_BYTES;
-        uint32_t adA[4], adB[2];
+    constexpr int R0 = SH::NREQ / 2;                        /* requests issued behind the first slice's multiplications */
+    auto addrs = [&](int st, uint32_t (&adA)[4], uint32_t (&adB)[NJ]){
+        const uint32_t sb = lds_base + (uint32_t)(st % NT3_STAGES) * SH::STAGE_BYTES;
 #pragma unroll
         for(int i = 0; i < 4; i++) adA[i] = sb + offA[i];
 #pragma unroll
-        for(int j = 0; j < 2; j++) adB[j] = sb + offB[j];
-        Nt3Ops o0, o1;
-        nt3_read<0>(o0, adA, adB);
+        for(int j = 0; j < NJ; j++) adB[j] = sb + offB[j];
+    };
+    issue(0, 0);
+    issue(1, 1);
+    for(int st = 0; st < steps; st++){
+        /* tile st has landed once at most the requests of tile st+1 are still in flight */
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(SH::NREQ) : "memory");
+        __builtin_amdgcn_s_barrier();                       /* everybody's pieces are in; stage (st+2)%3 is free again */
+        uint32_t adA[4], adB[NJ];
+        addrs(st, adA, adB);
+        Nt3Ops<NJ> o0, o1;
+        nt3_read<0, BN, NJ>(o0, adA, adB);
         nt3_wait_reads(o0);
-        nt3_read<1>(o1, adA, adB);                          /* in flight while slice 0 multiplies */
-        /* The six requests of tile st+2 go out between the multiplications, one after every other
-         * MFMA: a request can wait a hundred cycles for the address unit when eight wavefronts ask at
-         * once, and behind an MFMA that wait costs nothing. The fences keep the compiler from
-         * gathering them again. */
+        nt3_read<1, BN, NJ>(o1, adA, adB);                  /* in flight while slice 0 multiplies */
+        /* The requests of tile st+2 go out between the multiplications, one after every row of them:
+         * a request can wait a hundred cycles for the address unit when eight wavefronts ask at once, and
+         * behind an MFMA that wait costs nothing. The fences keep the compiler from gathering them again. */
         const int nt = st + 2, ns = (st + 2) % NT3_STAGES;
 #pragma unroll
         for(int i = 0; i < 4; i++){
 #pragma unroll
-            for(int j = 0; j < 2; j++)
+            for(int j = 0; j < NJ; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nt3_pack(o0.a[i][0], o0.a[i][1]), nt3_pack(o0.b[j][0], o0.b[j][1]), acc[i][j], 0, 0, 0);
-            if(i < 3){ __builtin_amdgcn_sched_barrier(0); issue_one(nt, ns, i); __builtin_amdgcn_sched_barrier(0); }
+            if(i < R0){ __builtin_amdgcn_sched_barrier(0); issue_one(nt, ns, i); __builtin_amdgcn_sched_barrier(0); }
         }
         nt3_wait_reads(o1);
 #pragma unroll
         for(int i = 0; i < 4; i++){
 #pragma unroll
-            for(int j = 0; j < 2; j++)
+            for(int j = 0; j < NJ; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nt3_pack(o1.a[i][0], o1.a[i][1]), nt3_pack(o1.b[j][0], o1.b[j][1]), acc[i][j], 0, 0, 0);
-            if(i < 3){ __builtin_amdgcn_sched_barrier(0); issue_one(nt, ns, 3 + i); __builtin_amdgcn_sched_barrier(0); }
+            if(R0 + i < SH::NREQ){ __builtin_amdgcn_sched_barrier(0); issue_one(nt, ns, R0 + i); __builtin_amdgcn_sched_barrier(0); }
         }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);                    /* vmcnt(0), as a builtin so that the compiler knows it: no request may outlive the workgroup's LDS */
@@ -216,12 +241,12 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nt_lds(Nt3Args a){
     const int fr = lane & 31, hf = lane >> 5, row = i0 + wi + hf * 4;
     float *c = P.C + (size_t)row * a.N + (j0 + wj + fr);
     if(nseq == 1){
-        qx_store_tiles<4, 2>(acc, c, row, i0 + wi, a.K, (size_t)a.N, P.beta != 0.0f);
+        qx_store_tiles<4, NJ>(acc, c, row, i0 + wi, a.K, (size_t)a.N, P.beta != 0.0f);
         return;
     }
     /* one slice of a split contraction: add to what the slices before have left, past the caches */
     if(seq > 0) qx_chain_wait(a.flags, flag, a.wait_epoch, seq, a.status, a.wait_limit);
-    qx_store_tiles<4, 2, true>(acc, c, row, i0 + wi, a.K, (size_t)a.N, seq > 0 || P.beta != 0.0f);
+    qx_store_tiles<4, NJ, true>(acc, c, row, i0 + wi, a.K, (size_t)a.N, seq > 0 || P.beta != 0.0f);
     if(seq + 1 < nseq) qx_chain_publish(a.flags, flag, a.epoch, seq);
 }
 
@@ -235,12 +260,12 @@ static void *g_nt3_zeros = nullptr;
  * column tiles of one (problem, tile row, slice); XCD x runs its entries in order, g workgroups each.
  * Returns the grid size, or 0 when the launch does not fit the table. */
 struct Nt3Group { int prob, ti, cost; };
-static int nt3_schedule(DevProb *pr, int n, int K, int N, int cus, DevUnit *units, int *nflags_out, int *nent_out){
-    const int g = N / NT3_BN, rp = (K + NT3_BM - 1) / NT3_BM;
+static int nt3_schedule(DevProb *pr, int n, int K, int N, int BN, int slots_per_cu, int cus, DevUnit *units, int *nflags_out, int *nent_out){
+    const int g = N / BN, rp = (K + NT3_BM - 1) / NT3_BM;
     if(rp > 64) return 0;                                              /* the packed entry has 6 bits for the tile row */
     long long work = 0;
     for(int p = 0; p < n; p++) work += (long long)pr[p].M * rp * g;
-    const long long slots = 2LL * cus;
+    const long long slots = (long long)slots_per_cu * cus;
     long long mean = (work + slots - 1) / slots;                       /* rows of contraction per workgroup slot */
     if(mean < 256) mean = 256;
     static int nchunk[QLMX_MAX_PROBLEMS], chunk[QLMX_MAX_PROBLEMS];
@@ -285,8 +310,34 @@ static int nt3_schedule(DevProb *pr, int n, int K, int N, int cus, DevUnit *unit
     return nent * g;
 }
 
+template<int BN> static int nt3_launch(const Nt3Args &a, int grid, hipStream_t st){
+    static bool attr_set = false;
+    if(!attr_set){
+        QLMX_HIP(hipFuncSetAttribute((const void *)k_gemm_nt_lds<BN>, hipFuncAttributeMaxDynamicSharedMemorySize, Nt3Shape<BN>::LDS_BYTES), "nt LDS size");
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k_gemm_nt_lds<BN>, dim3(grid), dim3(256), Nt3Shape<BN>::LDS_BYTES, st, a);
+    return QLMX_OK;
+}
+
+/* Which tile. The wide one is built and correct but not faster on this GPU (uniform 2048-row experts,
+ * K=768 N=2048: 873 against 861 TFLOP/s; 8192 rows: 841 against 943; with the operand reads issued a slice
+ * ahead and the barrier between the slices: 807), so it is only taken on request: QLMX_NT_TILE=256 in the
+ * environment (read at the first call), or qlmx_nt_tile(256). */
+static int g_nt3_forced = -1;
+static int nt3_pick_bn(int N){
+    if(g_nt3_forced < 0){ const char *e = getenv("QLMX_NT_TILE"); g_nt3_forced = e ? atoi(e) : 0; }
+    return (g_nt3_forced == 256 && N % 256 == 0) ? 256 : 128;
+}
+extern "C" int qlmx_nt_tile(int tile){
+    QLMX_REQUIRE(tile == 128 || tile == 256, "qlmx_nt_tile: 128 or 256, not %d", tile);
+    g_nt3_forced = tile;
+    return QLMX_OK;
+}
+
 /* bf16 operands only; N % 128 == 0, K % 8 == 0, operands 16-byte aligned (checked by the caller) */
 int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N, hipStream_t st){
+    const int BN = nt3_pick_bn(N);
     if(!g_nt3_zeros){
         QLMX_HIP(hipMalloc(&g_nt3_zeros, 256), "nt zero block");
         QLMX_HIP(hipMemset(g_nt3_zeros, 0, 256), "nt zero block clear");
@@ -307,34 +358,34 @@ int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N
                 QLMX_REQUIRE(p.A && p.B && p.C, "grouped gemm nt: problem %d has a NULL operand", i);
                 QLMX_REQUIRE(p.beta == 0.0f || p.beta == 1.0f, "grouped gemm: beta must be 0 or 1");
                 DevProb &q = uu.hprob[n++];
-                q.A = p.A; q.B = p.B; q.C = p.C; q.wq = 0; q.wg = 0; q.M = p.M; q.beta = p.beta; q.tile0 = 0; q.tiles_n = N / NT3_BN;
+                q.A = p.A; q.B = p.B; q.C = p.C; q.wq = 0; q.wg = 0; q.M = p.M; q.beta = p.beta; q.tile0 = 0; q.tiles_n = N / BN;
             }
             int nflags = 0, nent = 0;
-            const int grid = nt3_schedule(uu.hprob, n, K, N, qlmx_cu_count(), uu.hunit, &nflags, &nent);
+            const int grid = nt3_schedule(uu.hprob, n, K, N, BN, BN == 128 ? 2 : 1, qlmx_cu_count(), uu.hunit, &nflags, &nent);
             if(grid > 0){
                 Nt3Args a; a.pr = uu.dprob; a.units = uu.dunit; a.flags = uu.flags; a.status = uu.status;
-                a.nprob = n; a.ntiles = grid; a.tiles_n = N / NT3_BN; a.rows_p = 1; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
+                a.nprob = n; a.ntiles = grid; a.tiles_n = N / BN; a.rows_p = 1; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
                 int first = 0; a.epoch = 0;
                 if(nflags){ rc = qlmx_chain_reserve(nflags, &first, &a.epoch); if(rc) return rc; }
                 a.wait_epoch = a.epoch; a.wait_limit = QX_CHAIN_SPINS;
                 if(nflags && qlmx_test_take_forced_timeout(2)){ a.wait_epoch = a.epoch ^ 0x00A5A5A5u; a.wait_limit = 1; }
                 for(int p = 0; p < n; p++) uu.hprob[p].flag0 += first;
                 qlmx_unit_commit(&uu, n, nent);
-                hipLaunchKernelGGL(k_gemm_nt_lds, dim3(grid), dim3(256), 0, st, a);
+                rc = BN == 128 ? nt3_launch<128>(a, grid, st) : nt3_launch<256>(a, grid, st); if(rc) return rc;
                 QLMX_LAUNCH_CHECK("grouped gemm nt (scheduled) launch");
                 return qlmx_unit_done(uslot, st);
             }
         }
     }
     ProbUpload up; int slot;
-    int rc = qlmx_upload_problems(probs, nprob, GEMM_NT, K, N, NT3_BM, NT3_BN, st, &up, &slot); if(rc) return rc;
+    int rc = qlmx_upload_problems(probs, nprob, GEMM_NT, K, N, NT3_BM, BN, st, &up, &slot); if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;
-    Nt3Args a; a.units = nullptr; a.flags = nullptr; a.status = nullptr; a.epoch = 0; a.wait_epoch = 0; a.wait_limit = 0; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.tiles_n = N / NT3_BN; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
+    Nt3Args a; a.units = nullptr; a.flags = nullptr; a.status = nullptr; a.epoch = 0; a.wait_epoch = 0; a.wait_limit = 0; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.tiles_n = N / BN; a.K = K; a.N = N; a.zeros = g_nt3_zeros;
     a.rows_p = up.ntiles / (a.tiles_n * up.nprob);
     int grid;
     if(a.rows_p & 7) grid = 8 * a.tiles_n * a.rows_p * ((up.nprob + 7) / 8);
     else             grid = 8 * a.tiles_n * ((up.ntiles / a.tiles_n + 7) / 8);
-    hipLaunchKernelGGL(k_gemm_nt_lds, dim3(grid), dim3(256), 0, st, a);
+    rc = BN == 128 ? nt3_launch<128>(a, grid, st) : nt3_launch<256>(a, grid, st); if(rc) return rc;
     QLMX_LAUNCH_CHECK("grouped gemm nt (direct-to-LDS) launch");
     return qlmx_upload_done(slot, st);
 }

@@ -474,3 +474,22 @@ def test_mfma_rejects_unsupported_shapes(q):
     pr = q.problems([(x, None, x, 0, 0, 4, 0.0)])
     with pytest.raises(pkg.QlmxError, match="multiple"):
         q.gemm_nn(x, x, 128, pr, 1, 32, 100, pkg.ACT_F32, pkg.MATH_MFMA)
+
+
+def test_mfma_nt_wide_tile(q, orc):
+    """The opt-in 256 x 256 weight-gradient tile (qlmx_nt_tile): overwriting and accumulating, ragged, empty and
+    sliced experts, a K that is not a multiple of the tile; bit-equal to the 256 x 128 tile where no contraction
+    is sliced (same products, same order of additions)."""
+    q.call("qlmx_nt_tile", 256)
+    try:
+        for beta in (0.0, 1.0):
+            for (E, rows, K, N, seed) in [(4, [1700, 40, 0, 333], 256, 256, 6), (3, [300, 77, 512], 320, 512, 9), (2, [3841, 10], 64, 256, 8)]:
+                got, want = run_case(q, orc, "nt", E, rows, K, N, pkg.ACT_BF16, pkg.MATH_MFMA, seed=seed, nt_beta=beta)
+                assert orc.relerr(got, want) < TOL_MFMA
+        wide, _ = run_case(q, orc, "nt", 3, [64, 200, 96], 256, 512, pkg.ACT_BF16, pkg.MATH_MFMA, seed=10, nt_beta=0.0)
+    finally:
+        q.call("qlmx_nt_tile", 128)
+    narrow, _ = run_case(q, orc, "nt", 3, [64, 200, 96], 256, 512, pkg.ACT_BF16, pkg.MATH_MFMA, seed=10, nt_beta=0.0)
+    assert np.array_equal(wide.view(np.uint32), narrow.view(np.uint32))
+    with pytest.raises(pkg.QlmxError, match="128 or 256"):
+        q.call("qlmx_nt_tile", 64)

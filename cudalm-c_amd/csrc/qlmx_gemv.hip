@@ -329,9 +329,20 @@ struct DfArgs {
 struct DfMeta {
     int nprob;
     int p_e[DEC_MAXPAIR], p_M[DEC_MAXPAIR], p_row0[DEC_MAXPAIR];
-    int rowpair[DEC_MAXPAIR], pair_prob[DEC_MAXPAIR], pair_m[DEC_MAXPAIR];
+    int rowpair[DEC_MAXPAIR], rowtok[DEC_MAXPAIR], pair_prob[DEC_MAXPAIR], pair_m[DEC_MAXPAIR];
     int se[DEC_MAXPAIR], sj[DEC_MAXPAIR], ein[DEC_MAXPAIR], rk[4][DEC_MAXPAIR];
 };
+
+/* a / b for 0 <= a < 2^22, b > 0, rb = 1/b as a float: the quotient of the floats is off by at most one,
+ * which the remainder shows. (The compiler's integer division is some fifty instructions, and the
+ * bookkeeping between two tasks is made of divisions.) */
+__device__ __forceinline__ int df_div(int a, int b, float rb){
+    int q = (int)((float)a * rb);
+    const int r = a - q * b;
+    q += (r >= b) - (r < 0);
+    return q;
+}
+__device__ __forceinline__ int df_uni(int v){ return __builtin_amdgcn_readfirstlane(v); }
 
 __device__ __forceinline__ void df_st(u64 *p, float v, unsigned epoch){
     __hip_atomic_store(p, ((u64)epoch << 32) | (u64)__float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -496,13 +507,6 @@ __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w
     }
 }
 
-/* scale of row r of the slice, column group g of the chunk; srow0 points at the slice's first row,
- * chunk's first group */
-__device__ __forceinline__ float df_scale(const DfArgs &a, const float *srow0, int gpr, int N, int r, int chunk, int g){
-    if(chunk * DF_CW + g * a.group >= N) return 0.0f;
-    return srow0[(size_t)r * gpr + g];
-}
-
 __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
     __shared__ DfMeta mt;
     __shared__ __align__(16) float xs[DF_NG][DF_RMAX][DF_MB];   /* x[m][r] * scale(r, g), the four m side by side */
@@ -565,7 +569,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
         const int prob = __popcll(sm & upto) - 1;
         if(valid){
             const int j = mt.sj[r];
-            mt.rowpair[r] = j; mt.pair_prob[j] = prob; mt.pair_m[j] = pos % DF_MB;
+            mt.rowpair[r] = j; mt.rowtok[r] = j % a.T; mt.pair_prob[j] = prob; mt.pair_m[j] = pos % DF_MB;
             if(start){ mt.p_e[prob] = er; mt.p_M[prob] = min(DF_MB, cnt - pos); mt.p_row0[prob] = r; }
         }
         if(tid == 0) mt.nprob = __popcll(sm);
@@ -579,28 +583,31 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
      * first digits of a task are already on their way while the task before it finishes ---- */
     const int tpg1 = a.NC1 * a.S1, ngrp1 = 2 * nprob, lim1 = ((ngrp1 + 7) >> 3) * tpg1;
     const int tpg2 = a.NC2 * a.S2, lim2 = ((nprob + 7) >> 3) * tpg2;
+    const float rtpg1 = 1.0f / (float)tpg1, rtpg2 = 1.0f / (float)tpg2, rS1 = 1.0f / (float)a.S1, rS2 = 1.0f / (float)a.S2;
     int list = 1, q = slot0;
     auto fetch = [&]() -> DfT {
         DfT t; t.list = 0; t.wq = 0; t.wg = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = 0;
         for(;;){
             if(list == 1){
                 if(q >= lim1){ list = 2; q = slot0; continue; }
-                const int g = (q / tpg1) * 8 + xcd, sub = q % tpg1; q += nslot;
+                const int qd = df_uni(df_div(q, tpg1, rtpg1)), g = qd * 8 + xcd, sub = q - qd * tpg1; q += nslot;
                 if(g >= ngrp1) continue;
-                t.list = 1; t.prob = g >> 1; t.mat = g & 1; t.chunk = sub / a.S1; t.sl = sub - t.chunk * a.S1;
-                t.N = a.F; t.k0 = t.sl * a.R1; t.rows = min(a.R1, a.D - t.k0); t.M = mt.p_M[t.prob];
-                t.wq = (t.mat ? a.w3q : a.w1q) + (u64)mt.p_e[t.prob] * DF;
-                t.wg = (t.mat ? a.w3g : a.w1g) + (u64)mt.p_e[t.prob] * a.dfg;
+                t.list = 1; t.prob = g >> 1; t.mat = g & 1; t.chunk = df_uni(df_div(sub, a.S1, rS1)); t.sl = sub - t.chunk * a.S1;
+                t.N = a.F; t.k0 = t.sl * a.R1; t.rows = min(a.R1, a.D - t.k0); t.M = df_uni(mt.p_M[t.prob]);
+                const int ex = df_uni(mt.p_e[t.prob]);
+                t.wq = (t.mat ? a.w3q : a.w1q) + (u64)ex * DF;
+                t.wg = (t.mat ? a.w3g : a.w1g) + (u64)ex * a.dfg;
                 return t;
             }
             if(list == 2){
                 if(q >= lim2){ list = 3; return t; }
-                const int prob = (q / tpg2) * 8 + xcd, sub = q % tpg2; q += nslot;
+                const int qd = df_uni(df_div(q, tpg2, rtpg2)), prob = qd * 8 + xcd, sub = q - qd * tpg2; q += nslot;
                 if(prob >= nprob) continue;
-                t.list = 2; t.prob = prob; t.mat = 0; t.chunk = sub / a.S2; t.sl = sub - t.chunk * a.S2;
-                t.N = a.D; t.k0 = t.sl * a.R2; t.rows = min(a.R2, a.F - t.k0); t.M = mt.p_M[prob];
-                t.wq = a.w2q + (u64)mt.p_e[prob] * DF;
-                t.wg = a.w2g + (u64)mt.p_e[prob] * a.dfg;
+                t.list = 2; t.prob = prob; t.mat = 0; t.chunk = df_uni(df_div(sub, a.S2, rS2)); t.sl = sub - t.chunk * a.S2;
+                t.N = a.D; t.k0 = t.sl * a.R2; t.rows = min(a.R2, a.F - t.k0); t.M = df_uni(mt.p_M[prob]);
+                const int ex = df_uni(mt.p_e[prob]);
+                t.wq = a.w2q + (u64)ex * DF;
+                t.wg = a.w2g + (u64)ex * a.dfg;
                 return t;
             }
             return t;
@@ -608,9 +615,26 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
     };
     uint2 w0[DF_BATCH], w1[DF_BATCH];
     const int hs1 = a.R1 >> 5, hs2 = a.R2 >> 5;               /* steps per half task */
+    const int gprF = a.F / a.group, gprD = a.D / a.group;     /* scale groups per row of w1|w3 and of w2 */
+    const int cpg = a.group >= DF_CW ? a.group / DF_CW : 1;   /* chunks per scale group when the group is wider than a chunk */
+    /* first scale of a task: its first row, its chunk's first group */
+    auto scales_of = [&](const DfT &t) -> const float * {
+        const int cg = a.group >= DF_CW ? t.chunk / cpg : t.chunk * (DF_CW / a.group);
+        return a.s + t.wg + (size_t)t.k0 * (t.list == 1 ? gprF : gprD) + cg;
+    };
+    /* The group scales of row `tid` of a task, requested together with the task's digits -- a task ahead -- so
+     * that the staging finds them in registers instead of waiting for HBM. Requested without conditions (a
+     * dead position re-reads a live one); the staging zeroes what lies outside the matrix. */
+    auto scales_ahead = [&](const DfT &t, float (&sc)[DF_NG]){
+        const float *sp = scales_of(t) + (size_t)min(tid, t.rows - 1) * (t.list == 1 ? gprF : gprD);
+#pragma unroll
+        for(int gg = 0; gg < DF_NG; gg++) sc[gg] = sp[gg < ng ? gg : 0];
+    };
+    float csc[DF_NG];
     DfT cur = fetch();
     if(cur.list){
         const signed char *dp = df_digits(a, cur); const int hs = cur.list == 1 ? hs1 : hs2;
+        scales_ahead(cur, csc);
         DF_LOAD(w0, dp, (size_t)cur.N >> 1, cur.rows, hs, 0)
         DF_LOAD(w1, dp, (size_t)cur.N >> 1, cur.rows, hs, 1)
     }
@@ -618,13 +642,15 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
         const DfT nxt = fetch();
         /* after the last task the same loads go to the current task's digits again and are dropped */
         const DfT &pre = nxt.list ? nxt : cur;
+        /* older than the digits requested below, so taking them over at the end of this task waits for nothing
+         * that is still on its way */
+        float nsc[DF_NG];
+        scales_ahead(pre, nsc);
         const signed char *ndp = df_digits(a, pre); const int nhs = pre.list == 1 ? hs1 : hs2;
         auto next0 = [&](){ DF_LOAD(w0, ndp, (size_t)pre.N >> 1, pre.rows, nhs, 0) };
         auto next1 = [&](){ DF_LOAD(w1, ndp, (size_t)pre.N >> 1, pre.rows, nhs, 1) };
         const int hs = cur.list == 1 ? hs1 : hs2;
         const int prob = cur.prob, chunk = cur.chunk, k0 = cur.k0, rows = cur.rows, M = cur.M;
-        const int gpr = cur.N / a.group;
-        const float *srow0 = a.s + cur.wg + (size_t)k0 * gpr + (chunk * DF_CW) / a.group;
         u64 *dst; size_t mstride;
         if(cur.list == 1){ dst = a.part1 + ((((size_t)prob * 2 + cur.mat) * a.S1 + cur.sl) * DF_MB) * a.F; mstride = (size_t)a.F; }
         else             { dst = a.part2 + (((size_t)prob * a.S2 + cur.sl) * DF_MB) * a.D;                  mstride = (size_t)a.D; }
@@ -634,10 +660,10 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
                 for(int r = tid; r < rows; r += DF_THREADS){
                     float sc[DF_NG], xv[DF_MB];
 #pragma unroll
-                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = gg < ng ? df_scale(a, srow0, gpr, a.F, r, chunk, gg) : 0.0f;
+                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = (gg < ng && chunk * DF_CW + gg * a.group < a.F) ? csc[gg] : 0.0f;
 #pragma unroll
                     for(int m = 0; m < DF_MB; m++)
-                        xv[m] = m < M ? a.x[(size_t)(mt.rowpair[mt.p_row0[prob] + m] % a.T) * a.D + k0 + r] : 0.0f;
+                        xv[m] = m < M ? a.x[(size_t)mt.rowtok[mt.p_row0[prob] + m] * a.D + k0 + r] : 0.0f;
 #pragma unroll
                     for(int gg = 0; gg < DF_NG; gg++)
                         *(float4 *)&xs[gg][r][0] = make_float4(xv[0] * sc[gg], xv[1] * sc[gg], xv[2] * sc[gg], xv[3] * sc[gg]);
@@ -650,7 +676,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
                 for(int r = tid; r < rows; r += DF_THREADS){
                     float sc[DF_NG];
 #pragma unroll
-                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = gg < ng ? df_scale(a, srow0, gpr, a.D, r, chunk, gg) : 0.0f;
+                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = (gg < ng && chunk * DF_CW + gg * a.group < a.D) ? csc[gg] : 0.0f;
                     float hv[DF_MB];
 #pragma unroll
                     for(int m = 0; m < DF_MB; m++){
@@ -675,6 +701,8 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
         else if(M == 2) df_task<2>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1);
         else            df_task<4>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1);
         cur = nxt;
+#pragma unroll
+        for(int gg = 0; gg < DF_NG; gg++) csc[gg] = nsc[gg];
     }
     /* ---- 3. out[n,:] += gate[k][n] * y[row(k,n),:], passes in order (cudalm.cu:4227). A pair whose
      * expert index was out of range adds nothing (the reference aborts the run, cudalm.cu:3476-3478). ---- */

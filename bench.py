@@ -809,9 +809,11 @@ def cpu_decode(args, E=32, D=768, F=2048, topk=2, T=16, layers=2):
 
 # HBM bytes from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the 1 GiB copy calibration); the runs,
 # counter values and scale factors are in profiles/*.txt. adamw: per launch. train: per step, i.e. summed over
-# the step's 6 launches (1182 MiB read + 1086 MiB written). decode: per launch = per layer at T=16
-# (56.2 MiB read + 4.5 MiB written).
-PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.38e9, "decode": 6.37e7}
+# the step's 6 launches (1177 MiB read + 1086 MiB written). decode: per launch = per layer at T=16
+# (55.8 MiB read + 5.1 MiB written). The figures are constants of the code state they were measured at; that
+# state is named in the JSON line so that a reader can tell a stale one.
+PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.373e9, "decode": 6.39e7}
+PROFILED_AT = "git e24a32b"
 
 
 def main():
@@ -846,6 +848,7 @@ def main():
     for w in results:
         if results[w]["roofline"].get("traffic") is None and PROFILED_TRAFFIC.get(w) and not (w == "adamw" and args.render_p):
             results[w]["roofline"]["traffic"] = PROFILED_TRAFFIC[w]
+            results[w]["roofline"]["traffic_source"] = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, summaries in profiles/, measured at " + PROFILED_AT
     if not args.no_cpu:
         if "adamw" in results:
             results["adamw"]["cpu_baseline"] = cpu_adamw(args)

@@ -306,13 +306,31 @@ int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const
  * ---------------------------------------------------------------------------------------- */
 #define DEC_MAXPAIR 64
 #define DF_THREADS 256
-#define DF_MB 4               /* pairs per problem */
+#define DF_MB 2               /* pairs per problem: an expert hit by more pairs is several problems (a task of four rows took
+                                 2.3 times as long as one of one row and held up everything that waited for it; its digits are
+                                 fetched by neighbouring workgroups at about the same time, mostly once from HBM) */
 #define DF_CW 256             /* columns per task */
 #define DF_NG 2               /* scale groups per task row: group 128, or one when the group is a multiple of 256 */
 #define DF_RMAX 256           /* rows per task at most */
 #define DF_BATCH 8            /* steps (of 16 rows) per half task: a task is two halves of at most 128 rows */
 #define DF_SPIN_LIMIT (1 << 17)
+#define DF_MAXTASKS 128        /* tasks of one workgroup at most (both lists); the host refuses shapes that would need more */
 typedef unsigned long long u64;
+/* Tracing build (-DQLMX_DF_TRACE): thread 0 of every workgroup stamps the 100 MHz wall clock at the phases
+ * of its tasks into a device table that qlmx_debug_trace copies out. Not part of the shipped library. */
+#ifdef QLMX_DF_TRACE
+#define DF_TRACE_WG 1024
+#define DF_TRACE_EV 64
+static __device__ u64 df_trace_tab[DF_TRACE_WG][DF_TRACE_EV];
+#define DF_STAMP(code) do{ if(threadIdx.x == 0 && blockIdx.x < DF_TRACE_WG && df_nev < DF_TRACE_EV) \
+    df_trace_tab[blockIdx.x][df_nev++] = (wall_clock64() << 8) | (u64)(code); }while(0)
+#define DF_TRACE_PARAM , int &df_nev
+#define DF_TRACE_ARG , df_nev
+#else
+#define DF_STAMP(code) do{}while(0)
+#define DF_TRACE_PARAM
+#define DF_TRACE_ARG
+#endif
 
 struct DfArgs {
     const float *x; const int *assign; const float *gate; float *out;
@@ -432,7 +450,7 @@ __device__ __forceinline__ const signed char *df_digits(const DfArgs &a, const D
 template<int MT, class PREP, class NEXT0, class NEXT1>
 __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w0)[DF_BATCH], uint2 (&w1)[DF_BATCH], int hsteps,
                                         const float (*xs)[DF_RMAX][DF_MB], float *red, u64 *dst, size_t mstride,
-                                        PREP prep, NEXT0 next0, NEXT1 next1){
+                                        PREP prep, NEXT0 next0, NEXT1 next1 DF_TRACE_PARAM){
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cl = lane & 15, rp = wave * 4 + (lane >> 4);
     const int N = t.N, rows = t.rows, M = t.M, chunk = t.chunk;
@@ -444,15 +462,15 @@ __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w
         for(int j = 0; j < 16; j++) acc[m][j] = 0.0f; }
     /* The nibble masks go through df_and so that the byte-to-float converts (one instruction per
      * digit, v_cvt_f32_ubyteN) survive: seen through, the compiler rewrites mask + byte select into a
-     * bit-field extract per digit and doubles the instruction count. The four input values of a row
+     * bit-field extract per digit and doubles the instruction count. The input values of a row
      * sit side by side in LDS and come in with one 16-byte read. */
 #define DF_COMPUTE(W, h)                                                          \
     _Pragma("unroll")                                                              \
     for(int b = 0; b < DF_BATCH; b++){                                             \
         if(b < hsteps && ((h) * hsteps + b) * 16 < rows){                          \
             const int r = ((h) * hsteps + b) * 16 + rp;                            \
-            const float4 x4 = *(const float4 *)&xs[gl][r][0];                      \
-            const float xm[DF_MB] = {x4.x, x4.y, x4.z, x4.w};                      \
+            const float2 x2 = *(const float2 *)&xs[gl][r][0];                      \
+            const float xm[DF_MB] = {x2.x, x2.y};                                  \
             float f[16];                                                           \
             const uint32_t u0 = W[b].x ^ 0x88888888u, u1 = W[b].y ^ 0x88888888u;   \
             const uint32_t l0 = df_and(u0), h0 = df_and(u0 >> 4);                  \
@@ -468,11 +486,22 @@ __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w
             }                                                                      \
         }                                                                          \
     }
+    DF_STAMP(10 + 16 * t.list);
     prep();
+    DF_STAMP(11);
+    /* The multiply loop saturates the vector ALU; everything else a workgroup does -- listing its tasks, requesting
+     * digits, staging, reducing -- is short chains of dependent instructions that other workgroups wait for. Those
+     * run at a raised wave priority, the loop at the lowest, so that a workgroup still on its way to its first
+     * task is not starved by its neighbours' loops (the fourth workgroup of a CU otherwise reached its first task
+     * 8 us after the first). */
+    __builtin_amdgcn_s_setprio(0);
     DF_COMPUTE(w0, 0)
     next0();
+    DF_STAMP(12);
     DF_COMPUTE(w1, 1)
     next1();
+    __builtin_amdgcn_s_setprio(3);
+    DF_STAMP(13);
 #undef DF_COMPUTE
     /* four row phases of a wave: reduce-scatter over lane bits 5 and 4, then the four waves via LDS */
     const bool hi32 = lane & 32, hi16 = lane & 16;
@@ -505,14 +534,23 @@ __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w
             df_st(dst + (size_t)m * mstride + col, v, a.epoch);
         }
     }
+    DF_STAMP(14);
 }
 
-__global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
+__global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
     __shared__ DfMeta mt;
-    __shared__ __align__(16) float xs[DF_NG][DF_RMAX][DF_MB];   /* x[m][r] * scale(r, g), the four m side by side */
+    __shared__ __align__(16) float xs[DF_NG][DF_RMAX][DF_MB];   /* x[m][r] * scale(r, g), the m side by side */
     __shared__ float red[4 * DF_MB * DF_CW];
     __shared__ int giveup;
+    __shared__ DfT tasks[DF_MAXTASKS];
+    __shared__ int wcount[4];
     const int tid = threadIdx.x;
+    __builtin_amdgcn_s_setprio(3);
+#ifdef QLMX_DF_TRACE
+    int df_nev = 0;
+    if(tid < DF_TRACE_EV && blockIdx.x < DF_TRACE_WG) df_trace_tab[blockIdx.x][tid] = 0;
+#endif
+    DF_STAMP(1);
     /* The tag of this call's partial sums is one more than the last finished call's, which lives in
      * device memory: the host passes no counter, so a launch recorded in a graph tags every replay
      * afresh. Every workgroup reads the word here; the last workgroup to finish moves it on (end of
@@ -576,6 +614,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
     }
     __syncthreads();
     const int nprob = mt.nprob;
+    DF_STAMP(2);
     const int G = gridDim.x, xcd = blockIdx.x & 7, slot0 = blockIdx.x >> 3, nslot = G >> 3;
     const u64 DF = (u64)a.D * a.F;
 
@@ -584,34 +623,61 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
     const int tpg1 = a.NC1 * a.S1, ngrp1 = 2 * nprob, lim1 = ((ngrp1 + 7) >> 3) * tpg1;
     const int tpg2 = a.NC2 * a.S2, lim2 = ((nprob + 7) >> 3) * tpg2;
     const float rtpg1 = 1.0f / (float)tpg1, rtpg2 = 1.0f / (float)tpg2, rS1 = 1.0f / (float)a.S1, rS2 = 1.0f / (float)a.S2;
-    int list = 1, q = slot0;
-    auto fetch = [&]() -> DfT {
+    /* The task list of this workgroup is worked out once, one candidate per thread, and kept in LDS: candidate k
+     * of list 1 is slot slot0 + k * nslot of this XCD's tasks, list 2's follow; candidates that fall behind the
+     * last group of the XCD are dropped and the rest keeps its order. (Worked out one after the other by every
+     * wavefront in front of each task, this arithmetic -- a microsecond of dependent instructions -- stood between
+     * any two tasks.) */
+    const int nc1 = nslot > 0 ? (lim1 - slot0 + nslot - 1) / nslot : 0, nc2 = nslot > 0 ? (lim2 - slot0 + nslot - 1) / nslot : 0;
+    const int c1 = nc1 > 0 ? nc1 : 0, c2 = nc2 > 0 ? nc2 : 0;           /* candidates of the two lists */
+    {
         DfT t; t.list = 0; t.wq = 0; t.wg = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = 0;
-        for(;;){
-            if(list == 1){
-                if(q >= lim1){ list = 2; q = slot0; continue; }
-                const int qd = df_uni(df_div(q, tpg1, rtpg1)), g = qd * 8 + xcd, sub = q - qd * tpg1; q += nslot;
-                if(g >= ngrp1) continue;
-                t.list = 1; t.prob = g >> 1; t.mat = g & 1; t.chunk = df_uni(df_div(sub, a.S1, rS1)); t.sl = sub - t.chunk * a.S1;
-                t.N = a.F; t.k0 = t.sl * a.R1; t.rows = min(a.R1, a.D - t.k0); t.M = df_uni(mt.p_M[t.prob]);
-                const int ex = df_uni(mt.p_e[t.prob]);
+        if(tid < c1){
+            const int q = slot0 + tid * nslot;
+            const int qd = df_div(q, tpg1, rtpg1), g = qd * 8 + xcd, sub = q - qd * tpg1;
+            if(g < ngrp1){
+                t.list = 1; t.prob = g >> 1; t.mat = g & 1; t.chunk = df_div(sub, a.S1, rS1); t.sl = sub - t.chunk * a.S1;
+                t.N = a.F; t.k0 = t.sl * a.R1; t.rows = min(a.R1, a.D - t.k0); t.M = mt.p_M[t.prob];
+                const int ex = mt.p_e[t.prob];
                 t.wq = (t.mat ? a.w3q : a.w1q) + (u64)ex * DF;
                 t.wg = (t.mat ? a.w3g : a.w1g) + (u64)ex * a.dfg;
-                return t;
             }
-            if(list == 2){
-                if(q >= lim2){ list = 3; return t; }
-                const int qd = df_uni(df_div(q, tpg2, rtpg2)), prob = qd * 8 + xcd, sub = q - qd * tpg2; q += nslot;
-                if(prob >= nprob) continue;
-                t.list = 2; t.prob = prob; t.mat = 0; t.chunk = df_uni(df_div(sub, a.S2, rS2)); t.sl = sub - t.chunk * a.S2;
-                t.N = a.D; t.k0 = t.sl * a.R2; t.rows = min(a.R2, a.F - t.k0); t.M = df_uni(mt.p_M[prob]);
-                const int ex = df_uni(mt.p_e[prob]);
+        } else if(tid < c1 + c2){
+            const int q = slot0 + (tid - c1) * nslot;
+            const int qd = df_div(q, tpg2, rtpg2), prob = qd * 8 + xcd, sub = q - qd * tpg2;
+            if(prob < nprob){
+                t.list = 2; t.prob = prob; t.mat = 0; t.chunk = df_div(sub, a.S2, rS2); t.sl = sub - t.chunk * a.S2;
+                t.N = a.D; t.k0 = t.sl * a.R2; t.rows = min(a.R2, a.F - t.k0); t.M = mt.p_M[prob];
+                const int ex = mt.p_e[prob];
                 t.wq = a.w2q + (u64)ex * DF;
                 t.wg = a.w2g + (u64)ex * a.dfg;
-                return t;
             }
-            return t;
         }
+        /* keep the live ones, in order: rank inside the wavefront by a ballot, wavefronts added up through LDS */
+        const u64 bal = __ballot(t.list != 0);
+        const int lane = tid & 63, wv = tid >> 6;
+        if(lane == 0) wcount[wv] = __popcll(bal);
+        __syncthreads();
+        int base = 0;
+        for(int w = 0; w < wv; w++) base += wcount[w];
+        if(t.list != 0){
+            const int pos = base + __popcll(bal & ((1ull << lane) - 1ull));
+            if(pos < DF_MAXTASKS) tasks[pos] = t;
+        }
+        __syncthreads();
+    }
+    const int ntasks = min(DF_MAXTASKS, wcount[0] + wcount[1] + wcount[2] + wcount[3]);
+    int ti = 0;
+    auto fetch = [&]() -> DfT {
+        DfT t; t.list = 0; t.wq = 0; t.wg = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = 0;
+        if(ti < ntasks){
+            const DfT &s = tasks[ti++];
+            t.list = df_uni(s.list); t.N = df_uni(s.N); t.k0 = df_uni(s.k0); t.rows = df_uni(s.rows); t.chunk = df_uni(s.chunk);
+            t.M = df_uni(s.M); t.prob = df_uni(s.prob); t.mat = df_uni(s.mat); t.sl = df_uni(s.sl);
+            t.wq = ((u64)(unsigned)df_uni((int)(s.wq >> 32)) << 32) | (unsigned)df_uni((int)(unsigned)s.wq);
+            t.wg = ((u64)(unsigned)df_uni((int)(s.wg >> 32)) << 32) | (unsigned)df_uni((int)(unsigned)s.wg);
+        }
+        return t;
     };
     uint2 w0[DF_BATCH], w1[DF_BATCH];
     const int hs1 = a.R1 >> 5, hs2 = a.R2 >> 5;               /* steps per half task */
@@ -631,15 +697,19 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
         for(int gg = 0; gg < DF_NG; gg++) sc[gg] = sp[gg < ng ? gg : 0];
     };
     float csc[DF_NG];
+    DF_STAMP(20);
     DfT cur = fetch();
+    DF_STAMP(21);
     if(cur.list){
         const signed char *dp = df_digits(a, cur); const int hs = cur.list == 1 ? hs1 : hs2;
         scales_ahead(cur, csc);
         DF_LOAD(w0, dp, (size_t)cur.N >> 1, cur.rows, hs, 0)
         DF_LOAD(w1, dp, (size_t)cur.N >> 1, cur.rows, hs, 1)
     }
+    DF_STAMP(22);
     while(cur.list){
         const DfT nxt = fetch();
+        DF_STAMP(23);
         /* after the last task the same loads go to the current task's digits again and are dropped */
         const DfT &pre = nxt.list ? nxt : cur;
         /* older than the digits requested below, so taking them over at the end of this task waits for nothing
@@ -666,7 +736,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
                         xv[m] = m < M ? a.x[(size_t)mt.rowtok[mt.p_row0[prob] + m] * a.D + k0 + r] : 0.0f;
 #pragma unroll
                     for(int gg = 0; gg < DF_NG; gg++)
-                        *(float4 *)&xs[gg][r][0] = make_float4(xv[0] * sc[gg], xv[1] * sc[gg], xv[2] * sc[gg], xv[3] * sc[gg]);
+                        *(float2 *)&xs[gg][r][0] = make_float2(xv[0] * sc[gg], xv[1] * sc[gg]);
                 }
                 __syncthreads();
             } else {
@@ -691,19 +761,19 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
                     }
 #pragma unroll
                     for(int gg = 0; gg < DF_NG; gg++)
-                        *(float4 *)&xs[gg][r][0] = make_float4(hv[0] * sc[gg], hv[1] * sc[gg], hv[2] * sc[gg], hv[3] * sc[gg]);
+                        *(float2 *)&xs[gg][r][0] = make_float2(hv[0] * sc[gg], hv[1] * sc[gg]);
                 }
                 __syncthreads();
             }
         };
-        /* the inner loop is compiled for 1, 2 and 4 input rows (3 runs as 4 with a zero row) */
-        if(M == 1)      df_task<1>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1);
-        else if(M == 2) df_task<2>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1);
-        else            df_task<4>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1);
+        /* the inner loop is compiled for 1 and 2 input rows */
+        if(M == 1) df_task<1>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1 DF_TRACE_ARG);
+        else       df_task<2>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1 DF_TRACE_ARG);
         cur = nxt;
 #pragma unroll
         for(int gg = 0; gg < DF_NG; gg++) csc[gg] = nsc[gg];
     }
+    DF_STAMP(3);
     /* ---- 3. out[n,:] += gate[k][n] * y[row(k,n),:], passes in order (cudalm.cu:4227). A pair whose
      * expert index was out of range adds nothing (the reference aborts the run, cudalm.cu:3476-3478). ---- */
     {
@@ -732,6 +802,7 @@ __global__ void __launch_bounds__(DF_THREADS, 3) k_decode_fused(DfArgs a){
             }
         }
     }
+    DF_STAMP(4);
     /* the last workgroup to get here closes the call: clears the count and publishes the tag */
     if(tid == 0){
         const unsigned done = __hip_atomic_fetch_add(a.ctl + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -776,7 +847,7 @@ int qlmx_decode_setup(int device){
     int nb = 0; hipDeviceProp_t pr;
     QLMX_HIP(hipGetDeviceProperties(&pr, device), "decode device properties");
     QLMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, k_decode_fused, DF_THREADS, 0), "decode occupancy");
-    if(nb > 3) nb = 3;
+    if(nb > 4) nb = 4;
     dv.grid = (nb * pr.multiProcessorCount) & ~7;
     QLMX_REQUIRE(dv.grid >= 8, "decode setup: device too small (%d resident workgroups)", dv.grid);
     /* `scratch` names the array in host code; its memory on this device is wherever the loader put it */
@@ -880,10 +951,27 @@ static int df_forward(bool fixed, const char *who, const float *x, const int *as
     if(qlmx_test_take_forced_timeout(1)){ a.wait_xor = 0x40000000u; a.spin_limit = 0; }
     const long long most = (long long)2 * npair * a.NC1 * a.S1;
     const int grid = (int)std::min<long long>(dv.grid, (most + 7) & ~7LL);
+    {   /* a workgroup lists its tasks once, one candidate per thread: bound them for the worst case (every pair its own expert) */
+        const long long nslot = grid / 8;
+        const long long lim1 = ((2LL * npair + 7) / 8) * a.NC1 * a.S1, lim2 = (((long long)npair + 7) / 8) * a.NC2 * a.S2;
+        const long long cand = (lim1 + nslot - 1) / nslot + (lim2 + nslot - 1) / nslot;
+        if(cand > DF_MAXTASKS){
+            qlmx_set_error("%s: T=%d K=%d D=%d F=%d gives a workgroup up to %lld tasks, more than the %d it can list", who, T, K, D, F, cand, DF_MAXTASKS);
+            return QLMX_E_LIMIT;
+        }
+    }
     hipLaunchKernelGGL(k_decode_fused, dim3(grid), dim3(DF_THREADS), 0, st, a);
     QLMX_LAUNCH_CHECK("decode launch");
     return QLMX_OK;
 }
+
+#ifdef QLMX_DF_TRACE
+extern "C" int qlmx_debug_trace(unsigned long long *host, int words){
+    if(words > DF_TRACE_WG * DF_TRACE_EV) words = DF_TRACE_WG * DF_TRACE_EV;
+    QLMX_HIP(hipMemcpyFromSymbol(host, HIP_SYMBOL(df_trace_tab), (size_t)words * 8), "trace copy");
+    return QLMX_OK;
+}
+#endif
 
 extern "C" int qlmx_moe_decode_forward(const float *x, const int *assign, const float *gate, float *out,
                                        const signed char *d, const float *s, int group,

@@ -245,7 +245,8 @@ int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
  *   w1q/w3q/w2q: element offsets of expert 0's matrices in d; expert e adds e*D*F. All multiples of
  *   `group`; w1, w3 are [D,F] row-major and w2 is [F,D] row-major (cudalm.cu:263-265). The scale of
  *   element q is s[q / group] (every span a multiple of the group, true of all reference presets).
- * Limits: K*T <= 64 pairs, D and F multiples of 32 and <= 8192. Uses a library-owned workspace that
+ * Limits: K*T <= 64 pairs, D and F multiples of 32 and <= 8192 (QLMX_E_LIMIT for the few shapes in that range
+ * whose task lists a workgroup cannot hold). Uses a library-owned workspace that
  * is (re)allocated on first use or growth; calls on different streams must not overlap. The tag that
  * orders the hand-over between workgroups lives in device memory and moves on by itself, so a call
  * may be recorded into a HIP graph and replayed (once the workspace has its size: a call that would
@@ -263,9 +264,9 @@ int qlmx_moe_decode_forward(const float *x, const int *assign, const float *gate
  * QLMX_DECODE_SCRATCH_BYTES that is part of the library image (each GPU the library runs on holds it
  * until the process ends), and the call makes no hipMalloc, hipFree or other allocating call.
  * qlmx_init must have run for the current device. A shape whose partial sums
- *   8 * K*T * 4 * (2 * ceil(D/R1) * F + ceil(F/256) * D)  bytes, R1 = 64..256 rows per gate|up slice
+ *   8 * K*T * 2 * (2 * ceil(D/R1) * F + ceil(F/R2) * D)  bytes, R1, R2 = 64..256 rows per gate|up / down slice
  * exceed the array fails with QLMX_E_LIMIT (the 32-expert D=768 F=2048 layer at 16 tokens top-2
- * needs 18.9 MB). Every call on a GPU shares that GPU's array: calls that overlap on one GPU,
+ * needs 10.6 MB). Every call on a GPU shares that GPU's array: calls that overlap on one GPU,
  * whatever their streams, race. */
 #define QLMX_DECODE_SCRATCH_BYTES (32u << 20)
 int qlmx_moe_decode_forward_noalloc(const float *x, const int *assign, const float *gate, float *out,

@@ -342,6 +342,8 @@ struct DfArgs {
     u64 *part1, *part2; unsigned epoch; unsigned *status;
     unsigned wait_xor; int spin_limit;   /* waits look for epoch ^ wait_xor (0) for at most spin_limit polls; the time-out test changes both */
     unsigned *ctl;            /* device words: [0] tag of the last finished call, [1] workgroups of this call that are done */
+    u64 parts1, parts2;       /* byte n: pieces a group's chunks are cut into when a list has n < 8 groups (a table in a
+                                 word: indexing an array inside the kernel arguments would move them all to scratch memory) */
 };
 
 struct DfMeta {
@@ -570,7 +572,6 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
         mt.ein[tid] = e;
     }
     __syncthreads();
-    a.epoch = __builtin_amdgcn_readfirstlane(last == 0xFFFFFFFFu ? 1u : last + 1u);
     {
         const int j = tid & 63, part = tid >> 6, e = mt.ein[j];
         int rank = 0;
@@ -620,9 +621,17 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
 
     /* ---- this workgroup's tasks, list 1 (gate|up) then list 2 (down), in one stream so that the
      * first digits of a task are already on their way while the task before it finishes ---- */
-    const int tpg1 = a.NC1 * a.S1, ngrp1 = 2 * nprob, lim1 = ((ngrp1 + 7) >> 3) * tpg1;
-    const int tpg2 = a.NC2 * a.S2, lim2 = ((nprob + 7) >> 3) * tpg2;
+    /* Groups -- (problem, matrix) in list 1, problems in list 2 -- go to the XCDs round robin, whole, so that the
+     * scale sectors that a group's column chunks share meet in one L2. With fewer than 8 groups that would leave
+     * XCDs without work (a single token: 4 groups, half the device idle and two rounds of tasks on the other
+     * half), so a group's chunks are then cut into `parts` pieces that go to different XCDs (host table). */
+    const int ngrp1 = 2 * nprob;
+    const int parts1 = ngrp1 < 8 ? (int)((a.parts1 >> (8 * ngrp1)) & 0xFFu) : 1, parts2 = nprob < 8 ? (int)((a.parts2 >> (8 * nprob)) & 0xFFu) : 1;
+    const int cpp1 = df_div(a.NC1, parts1, 1.0f / (float)parts1), cpp2 = df_div(a.NC2, parts2, 1.0f / (float)parts2);   /* chunks per piece */
+    const int tpg1 = cpp1 * a.S1, nvg1 = ngrp1 * parts1, lim1 = ((nvg1 + 7) >> 3) * tpg1;
+    const int tpg2 = cpp2 * a.S2, nvg2 = nprob * parts2, lim2 = ((nvg2 + 7) >> 3) * tpg2;
     const float rtpg1 = 1.0f / (float)tpg1, rtpg2 = 1.0f / (float)tpg2, rS1 = 1.0f / (float)a.S1, rS2 = 1.0f / (float)a.S2;
+    const float rparts1 = 1.0f / (float)parts1, rparts2 = 1.0f / (float)parts2;
     /* The task list of this workgroup is worked out once, one candidate per thread, and kept in LDS: candidate k
      * of list 1 is slot slot0 + k * nslot of this XCD's tasks, list 2's follow; candidates that fall behind the
      * last group of the XCD are dropped and the rest keeps its order. (Worked out one after the other by every
@@ -634,9 +643,10 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
         DfT t; t.list = 0; t.wq = 0; t.wg = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = 0;
         if(tid < c1){
             const int q = slot0 + tid * nslot;
-            const int qd = df_div(q, tpg1, rtpg1), g = qd * 8 + xcd, sub = q - qd * tpg1;
-            if(g < ngrp1){
-                t.list = 1; t.prob = g >> 1; t.mat = g & 1; t.chunk = df_div(sub, a.S1, rS1); t.sl = sub - t.chunk * a.S1;
+            const int qd = df_div(q, tpg1, rtpg1), vg = qd * 8 + xcd, sub = q - qd * tpg1;
+            if(vg < nvg1){
+                const int g = df_div(vg, parts1, rparts1), part = vg - g * parts1, cl = df_div(sub, a.S1, rS1);
+                t.list = 1; t.prob = g >> 1; t.mat = g & 1; t.chunk = part * cpp1 + cl; t.sl = sub - cl * a.S1;
                 t.N = a.F; t.k0 = t.sl * a.R1; t.rows = min(a.R1, a.D - t.k0); t.M = mt.p_M[t.prob];
                 const int ex = mt.p_e[t.prob];
                 t.wq = (t.mat ? a.w3q : a.w1q) + (u64)ex * DF;
@@ -644,9 +654,10 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
             }
         } else if(tid < c1 + c2){
             const int q = slot0 + (tid - c1) * nslot;
-            const int qd = df_div(q, tpg2, rtpg2), prob = qd * 8 + xcd, sub = q - qd * tpg2;
-            if(prob < nprob){
-                t.list = 2; t.prob = prob; t.mat = 0; t.chunk = df_div(sub, a.S2, rS2); t.sl = sub - t.chunk * a.S2;
+            const int qd = df_div(q, tpg2, rtpg2), vg = qd * 8 + xcd, sub = q - qd * tpg2;
+            if(vg < nvg2){
+                const int prob = df_div(vg, parts2, rparts2), part = vg - prob * parts2, cl = df_div(sub, a.S2, rS2);
+                t.list = 2; t.prob = prob; t.mat = 0; t.chunk = part * cpp2 + cl; t.sl = sub - cl * a.S2;
                 t.N = a.D; t.k0 = t.sl * a.R2; t.rows = min(a.R2, a.F - t.k0); t.M = mt.p_M[prob];
                 const int ex = mt.p_e[prob];
                 t.wq = a.w2q + (u64)ex * DF;
@@ -666,6 +677,9 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
         }
         __syncthreads();
     }
+    /* the tag is first needed when a partial sum is stored: its load (past the caches) has had the table and the
+     * task list to come back */
+    a.epoch = __builtin_amdgcn_readfirstlane(last == 0xFFFFFFFFu ? 1u : last + 1u);
     const int ntasks = min(DF_MAXTASKS, wcount[0] + wcount[1] + wcount[2] + wcount[3]);
     int ti = 0;
     auto fetch = [&]() -> DfT {
@@ -945,6 +959,12 @@ static int df_forward(bool fixed, const char *who, const float *x, const int *as
         rc = df_reserve(dv.grown, 0, words1, st); if(rc) return rc;
         rc = df_reserve(dv.grown, 1, words2, st); if(rc) return rc;
         a.ctl = dv.grown.ctl; a.part1 = dv.grown.part[0]; a.part2 = dv.grown.part[1];
+    }
+    /* fewer than 8 groups: the smallest number of pieces (a divisor of the chunk count) that gives every XCD one */
+    a.parts1 = 0; a.parts2 = 0;
+    for(int n = 0; n < 8; n++){
+        auto pieces = [&](int NC){ int pcs = NC; for(int c = 1; c <= NC; c++) if(NC % c == 0 && n * c >= 8){ pcs = c; break; } return n == 0 ? 1 : pcs; };
+        a.parts1 |= (u64)pieces(a.NC1) << (8 * n); a.parts2 |= (u64)pieces(a.NC2) << (8 * n);
     }
     a.status = dv.status; a.epoch = 0;
     a.wait_xor = 0; a.spin_limit = DF_SPIN_LIMIT;

@@ -490,6 +490,14 @@ def bench_decode(torch, q, args, E=32, D=768, F=2048, topk=2, layers=8):
         tm = timed(torch, step, args.steps, args.warmup)
         res = {"ms_8_layers": tm["event_ms_avg"], "distinct_expert_hits": hits, "bytes": hits * per_expert,
                "gbs": hits * per_expert / (tm["event_ms_avg"] * 1e-3) / 1e9}
+        # beside it: the same sequence with the layer's inputs taken as fp16 pairs (qlmx_decode_math(1); 3.7e-4
+        # against the fp32 reference instead of 4e-7); the figures of the line are the default fp32 loop's
+        q.call("qlmx_decode_math", 1)
+        try:
+            th = timed(torch, step, args.steps, args.warmup)
+            res["fp16_inputs_ms_8_layers"] = th["event_ms_avg"]
+        finally:
+            q.call("qlmx_decode_math", 0)
         # the same 8-layer sequence replayed as one HIP graph (no launch gaps from the host)
         try:
             gr = torch.cuda.CUDAGraph()

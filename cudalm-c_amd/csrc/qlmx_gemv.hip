@@ -23,6 +23,8 @@
  */
 #include "qlmx_gemm.h"
 #include <math.h>
+#include <string.h>
+#include <stdlib.h>
 #include <algorithm>
 
 #define GV_THREADS 256
@@ -312,20 +314,22 @@ int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const
 #define DF_CW 256             /* columns per task */
 #define DF_NG 2               /* scale groups per task row: group 128, or one when the group is a multiple of 256 */
 #define DF_RMAX 256           /* rows per task at most */
-#define DF_BATCH 8            /* steps (of 16 rows) per half task: a task is two halves of at most 128 rows */
+#define DF_BATCH 8            /* 8-byte digit loads per lane and half task (4 steps of 32 rows, a lane's two rows each): a task is two halves of at most 128 rows */
 #define DF_SPIN_LIMIT (1 << 17)
 #define DF_MAXTASKS 128        /* tasks of one workgroup at most (both lists); the host refuses shapes that would need more */
 typedef unsigned long long u64;
 /* Tracing build (-DQLMX_DF_TRACE): thread 0 of every workgroup stamps the 100 MHz wall clock at the phases
- * of its tasks into a device table that qlmx_debug_trace copies out. Not part of the shipped library. */
+ * of its tasks into LDS (a store to memory per stamp would be waited for with the loads it sits among and
+ * stretch the phases of a saturated launch); the workgroup copies its stamps to a device table when it is
+ * done, and qlmx_debug_trace copies that out. Not part of the shipped library. */
 #ifdef QLMX_DF_TRACE
 #define DF_TRACE_WG 1024
 #define DF_TRACE_EV 64
 static __device__ u64 df_trace_tab[DF_TRACE_WG][DF_TRACE_EV];
-#define DF_STAMP(code) do{ if(threadIdx.x == 0 && blockIdx.x < DF_TRACE_WG && df_nev < DF_TRACE_EV) \
-    df_trace_tab[blockIdx.x][df_nev++] = (wall_clock64() << 8) | (u64)(code); }while(0)
-#define DF_TRACE_PARAM , int &df_nev
-#define DF_TRACE_ARG , df_nev
+#define DF_STAMP(code) do{ if(threadIdx.x == 0 && df_nev < DF_TRACE_EV) \
+    df_ev[df_nev++] = (wall_clock64() << 8) | (u64)(code); }while(0)
+#define DF_TRACE_PARAM , int &df_nev, u64 *df_ev
+#define DF_TRACE_ARG , df_nev, df_ev
 #else
 #define DF_STAMP(code) do{}while(0)
 #define DF_TRACE_PARAM
@@ -342,7 +346,7 @@ struct DfArgs {
     u64 *part1, *part2; unsigned epoch; unsigned *status;
     unsigned wait_xor; int spin_limit;   /* waits look for epoch ^ wait_xor (0) for at most spin_limit polls; the time-out test changes both */
     unsigned *ctl;            /* device words: [0] tag of the last finished call, [1] workgroups of this call that are done */
-    u64 parts1, parts2;       /* byte n: pieces a group's chunks are cut into when a list has n < 8 groups (a table in a
+    u64 parts1, parts2;       /* byte n: pieces a group's chunks are cut into when n groups are left over after the last round of 8 (a table in a
                                  word: indexing an array inside the kernel arguments would move them all to scratch memory) */
 };
 
@@ -422,36 +426,117 @@ __device__ __forceinline__ uint32_t df_and(uint32_t v){
     uint32_t r; asm("v_and_b32 %0, %1, %2" : "=v"(r) : "s"(0x0F0F0F0Fu), "v"(v)); return r;
 }
 
+/* (v & mask) | magic in one instruction; written out because the compiler emits an and and an or */
+__device__ __forceinline__ uint32_t df_and_or(uint32_t v, uint32_t mask, uint32_t magic){
+    uint32_t r; asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "s"(mask), "v"(magic)); return r;
+}
+typedef _Float16 df_h2 __attribute__((ext_vector_type(2)));
+/* a.x * b.x + a.y * b.y + c: fp16 pairs, exact products, fp32 sum (v_dot2_f32_f16) */
+__device__ __forceinline__ float df_dot2(uint32_t a, uint32_t b, float c){
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(df_h2, a), __builtin_bit_cast(df_h2, b), c, false);
+}
+__device__ __forceinline__ uint32_t df_pack_h2(float a, float b){
+    const df_h2 h = {(_Float16)a, (_Float16)b};
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+/* Staging of a task's inputs. v[g][m] is this thread's row (thread = row of the task; zeros past its rows)
+ * times the row's scale of column group g, for the task's input rows m. The multiply loop takes them as fp16
+ * pairs of two consecutive rows, so they are first brought to [2^14, 2^15) at the task's largest magnitude by a
+ * power of two (its inverse is returned and applied to the task's sums) and stored per scale group and row
+ * pair as {pair of m = 0, pair of m = 1, the same two divided by 16}. Two barriers: the first also separates
+ * the previous task's reads of xs from the writes here. */
+__device__ __forceinline__ float df_stage(const float (&v)[DF_NG][DF_MB], bool live, uint32_t (*xs)[DF_RMAX / 2][2 * DF_MB], float *wmax){
+    const int tid = threadIdx.x;
+    float mx = 0.0f;
+#pragma unroll
+    for(int gg = 0; gg < DF_NG; gg++)
+#pragma unroll
+        for(int m = 0; m < DF_MB; m++) mx = fmaxf(mx, fabsf(v[gg][m]));
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if((tid & 63) == 0) wmax[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+    /* 2^(14 - floor(log2 mx)), kept where it and its inverse are both normal numbers */
+    const int ex = (int)((__float_as_uint(mx) >> 23) & 0xFFu);
+    int se = 268 - ex; if(se > 252) se = 252; if(se < 2) se = 2;
+    const float scale = __uint_as_float((uint32_t)se << 23), inv = __uint_as_float((uint32_t)(254 - se) << 23);
+#pragma unroll
+    for(int gg = 0; gg < DF_NG; gg++){
+        uint32_t hi[DF_MB], lo[DF_MB];
+#pragma unroll
+        for(int m = 0; m < DF_MB; m++){
+            const float p = v[gg][m] * scale, q = __shfl_xor(p, 1, 64);   /* the odd row of the pair is the next lane's */
+            hi[m] = df_pack_h2(p, q); lo[m] = df_pack_h2(p * 0.0625f, q * 0.0625f);
+        }
+        if(live && !(tid & 1)) *(uint4 *)&xs[gg][tid >> 1][0] = make_uint4(hi[0], hi[1], lo[0], lo[1]);
+    }
+    __syncthreads();
+    return inv;
+}
+
+/* The same for the fp32 loop: the values as they are, xs[g][row][m]; nothing to undo (returns 1). */
+__device__ __forceinline__ float df_stage_f32(const float (&v)[DF_NG][DF_MB], bool live, float (*xs)[DF_RMAX][DF_MB]){
+    __syncthreads();                                 /* the previous task is done with xs */
+    if(live){
+#pragma unroll
+        for(int gg = 0; gg < DF_NG; gg++) *(float2 *)&xs[gg][threadIdx.x][0] = make_float2(v[gg][0], v[gg][1]);
+    }
+    __syncthreads();
+    return 1.0f;
+}
+
 /* One task: which slice of which matrix, for which problem. list 0 = none. */
 struct DfT { u64 wq, wg; int list, N, k0, rows, chunk, M, prob, mat, sl; };
 
 /* first DF_BATCH steps of a task's digits into W (the caller keeps them in flight across the end of
  * the previous task) */
+template<bool H>
 __device__ __forceinline__ const signed char *df_digits(const DfArgs &a, const DfT &t){
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int cl = lane & 15, rp = wave * 4 + (lane >> 4);
     const int col0 = t.chunk * DF_CW + cl * 16;
-    return a.d + ((t.wq + (size_t)(t.k0 + rp) * t.N + (col0 < t.N ? col0 : 0)) >> 1);
+    return a.d + ((t.wq + (size_t)(t.k0 + (H ? 2 * rp : rp)) * t.N + (col0 < t.N ? col0 : 0)) >> 1);
 }
-/* rows is a multiple of 16, so a step is live or not for the whole workgroup. Every load is issued
- * unconditionally (a dead step re-reads step 0): loads under a branch make the compiler wait for
- * each one where the branches join, which turns a batch into a chain of memory round trips. */
-#define DF_LOAD(W, dp, rowb, rows, hsteps, h)                                      \
-    _Pragma("unroll")                                                              \
-    for(int b = 0; b < DF_BATCH; b++){                                             \
-        const int st_ = (h) * (hsteps) + b;                                        \
-        const int sc_ = (b < (hsteps) && st_ * 16 < (rows)) ? st_ : 0;             \
-        W[b] = *(const uint2 *)((dp) + (size_t)sc_ * 16 * (rowb));                 \
+/* Requests half h of a task's digits into W. fp16 loop (H): a step is 32 rows, the 16 row pairs of the
+ * workgroup's 16 lane groups, and W[2 s + par] holds row `par` of the lane's pair in step s of the half; fp32
+ * loop: a step is 16 rows, W[s] the lane's row in step s. rows is a multiple of 32, so a step is live or not
+ * for the whole workgroup. Every load is issued unconditionally (a dead step re-reads step 0): loads under a
+ * branch make the compiler wait for each one where the branches join, which turns a batch into a chain of
+ * memory round trips. */
+template<bool H>
+__device__ __forceinline__ void df_load(uint2 (&W)[DF_BATCH], const signed char *dp, size_t rowb, int rows, int hsteps, int h){
+#pragma unroll
+    for(int b = 0; b < DF_BATCH; b++){
+        if(H){
+            const int st = h * hsteps + (b >> 1);
+            const int sc = ((b >> 1) < hsteps && st * 32 < rows) ? st : 0;
+            W[b] = *(const uint2 *)(dp + (size_t)(sc * 32 + (b & 1)) * rowb);
+        } else {
+            const int st = h * hsteps + b;
+            const int sc = (b < hsteps && st * 16 < rows) ? st : 0;
+            W[b] = *(const uint2 *)(dp + (size_t)sc * 16 * rowb);
+        }
     }
+}
 
 /* dst[m*mstride + chunk*256 + c] = sum_{r<rows} x[m][r] * s * digit(k0+r, chunk*256+c), m < M, stored
- * tagged. w0, w1 hold the digits of the task's two halves, requested earlier. `prep` fills
- * xs[m][g][r] = x[m][r] * scale(k0+r, column group g) and ends with a workgroup barrier. `next0`
- * and `next1` request the following task's halves into w0 and w1 as soon as this task has consumed
- * them, so the reduction, the stores and the next task's staging overlap that trip from HBM. */
-template<int MT, class PREP, class NEXT0, class NEXT1>
+ * tagged. w0, w1 hold the digits of the task's two halves, requested earlier. `prep` stages the inputs
+ * (df_stage) and returns the power of two to apply to the sums. `next0` and `next1` request the following
+ * task's halves into w0 and w1 as soon as this task has consumed them, so the reduction, the stores and the
+ * next task's staging overlap that trip from HBM.
+ *
+ * The multiply-adds are v_dot2_f32_f16: two products per instruction, exact, summed in fp32. One operand is the
+ * pair of digits of a lane's two rows as fp16, built without a conversion: with u = digit + 8 (two's complement
+ * nibble xor 8), 0x6400 | u is the fp16 number 1024 + u (even columns, low nibble) and 0x6400 | u << 4 is
+ * 1024 + 16 u (odd columns, the nibble stays where it is), so one byte permute puts two bytes of both rows side
+ * by side and one and-or per column does the rest: 14 instructions per 16 digits. The other operand is the pair
+ * of staged inputs (divided by 16 for the odd columns). What the offsets add -- (1024 + 8) and (64 + 8) times
+ * the sum of the staged inputs -- is taken out at the end. The inputs thus carry 11 significant bits. */
+template<bool H, int MT, class PREP, class NEXT0, class NEXT1>
 __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w0)[DF_BATCH], uint2 (&w1)[DF_BATCH], int hsteps,
-                                        const float (*xs)[DF_RMAX][DF_MB], float *red, u64 *dst, size_t mstride,
+                                        const uint32_t *xs_raw, float *red, u64 *dst, size_t mstride,
                                         PREP prep, NEXT0 next0, NEXT1 next1 DF_TRACE_PARAM){
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cl = lane & 15, rp = wave * 4 + (lane >> 4);
@@ -462,16 +547,49 @@ __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w
     for(int m = 0; m < MT; m++){ corr[m] = 0.0f;
 #pragma unroll
         for(int j = 0; j < 16; j++) acc[m][j] = 0.0f; }
-    /* The nibble masks go through df_and so that the byte-to-float converts (one instruction per
-     * digit, v_cvt_f32_ubyteN) survive: seen through, the compiler rewrites mask + byte select into a
-     * bit-field extract per digit and doubles the instruction count. The input values of a row
-     * sit side by side in LDS and come in with one 16-byte read. */
-#define DF_COMPUTE(W, h)                                                          \
+    const uint32_t magic = 0x64006400u;
+    const uint32_t (*xs)[DF_RMAX / 2][2 * DF_MB] = (const uint32_t (*)[DF_RMAX / 2][2 * DF_MB])xs_raw;
+    const float (*xf)[DF_RMAX][DF_MB] = (const float (*)[DF_RMAX][DF_MB])xs_raw;
+#define DF_COMPUTE_H(W, h)                                                          \
+    _Pragma("unroll")                                                              \
+    for(int s_ = 0; s_ < DF_BATCH / 2; s_++){                                      \
+        if(s_ < hsteps && ((h) * hsteps + s_) * 32 < rows){                        \
+            const uint4 x4 = *(const uint4 *)&xs[gl][((h) * hsteps + s_) * 16 + rp][0]; \
+            const uint32_t xh[DF_MB] = {x4.x, x4.y}, xl[DF_MB] = {x4.z, x4.w};     \
+            uint32_t P[16];                                                        \
+            _Pragma("unroll")                                                      \
+            for(int hf = 0; hf < 2; hf++){                                         \
+                const uint32_t r0_ = (hf ? W[2 * s_].y : W[2 * s_].x) ^ 0x88888888u;         \
+                const uint32_t r1_ = (hf ? W[2 * s_ + 1].y : W[2 * s_ + 1].x) ^ 0x88888888u; \
+                const uint32_t E0 = __builtin_amdgcn_perm(r1_, r0_, 0x05040100u);  \
+                const uint32_t E1 = __builtin_amdgcn_perm(r1_, r0_, 0x07060302u);  \
+                const uint32_t S0 = E0 >> 8, S1 = E1 >> 8;                         \
+                P[hf * 8 + 0] = df_and_or(E0, 0x000F000Fu, magic);                 \
+                P[hf * 8 + 1] = df_and_or(E0, 0x00F000F0u, magic);                 \
+                P[hf * 8 + 2] = df_and_or(S0, 0x000F000Fu, magic);                 \
+                P[hf * 8 + 3] = df_and_or(S0, 0x00F000F0u, magic);                 \
+                P[hf * 8 + 4] = df_and_or(E1, 0x000F000Fu, magic);                 \
+                P[hf * 8 + 5] = df_and_or(E1, 0x00F000F0u, magic);                 \
+                P[hf * 8 + 6] = df_and_or(S1, 0x000F000Fu, magic);                 \
+                P[hf * 8 + 7] = df_and_or(S1, 0x00F000F0u, magic);                 \
+            }                                                                      \
+            _Pragma("unroll")                                                      \
+            for(int m = 0; m < MT; m++){                                           \
+                corr[m] = df_dot2(0x3C003C00u, xh[m], corr[m]);                    \
+                _Pragma("unroll")                                                  \
+                for(int j = 0; j < 16; j++) acc[m][j] = df_dot2(P[j], (j & 1) ? xl[m] : xh[m], acc[m][j]); \
+            }                                                                      \
+        }                                                                          \
+    }
+    /* The fp32 loop: one row per lane and step, digits to fp32 one by one (v_cvt_f32_ubyteN; the nibble masks go
+     * through df_and so that those converts survive: seen through, the compiler rewrites mask + byte select into
+     * a bit-field extract per digit and doubles the instruction count), 16 fp32 multiply-adds per input row. */
+#define DF_COMPUTE_S(W, h)                                                        \
     _Pragma("unroll")                                                              \
     for(int b = 0; b < DF_BATCH; b++){                                             \
         if(b < hsteps && ((h) * hsteps + b) * 16 < rows){                          \
             const int r = ((h) * hsteps + b) * 16 + rp;                            \
-            const float2 x2 = *(const float2 *)&xs[gl][r][0];                      \
+            const float2 x2 = *(const float2 *)&xf[gl][r][0];                      \
             const float xm[DF_MB] = {x2.x, x2.y};                                  \
             float f[16];                                                           \
             const uint32_t u0 = W[b].x ^ 0x88888888u, u1 = W[b].y ^ 0x88888888u;   \
@@ -489,7 +607,7 @@ __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w
         }                                                                          \
     }
     DF_STAMP(10 + 16 * t.list);
-    prep();
+    const float unscale = prep();
     DF_STAMP(11);
     /* The multiply loop saturates the vector ALU; everything else a workgroup does -- listing its tasks, requesting
      * digits, staging, reducing -- is short chains of dependent instructions that other workgroups wait for. Those
@@ -497,14 +615,15 @@ __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w
      * task is not starved by its neighbours' loops (the fourth workgroup of a CU otherwise reached its first task
      * 8 us after the first). */
     __builtin_amdgcn_s_setprio(0);
-    DF_COMPUTE(w0, 0)
+    if(H){ DF_COMPUTE_H(w0, 0) } else { DF_COMPUTE_S(w0, 0) }
     next0();
     DF_STAMP(12);
-    DF_COMPUTE(w1, 1)
+    if(H){ DF_COMPUTE_H(w1, 1) } else { DF_COMPUTE_S(w1, 1) }
     next1();
     __builtin_amdgcn_s_setprio(3);
     DF_STAMP(13);
-#undef DF_COMPUTE
+#undef DF_COMPUTE_H
+#undef DF_COMPUTE_S
     /* four row phases of a wave: reduce-scatter over lane bits 5 and 4, then the four waves via LDS */
     const bool hi32 = lane & 32, hi16 = lane & 16;
     __syncthreads();
@@ -512,9 +631,10 @@ __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w
     for(int m = 0; m < MT; m++){
         if(m < M){
             float k8[8], k4[4];
-            const float off = 8.0f * corr[m];
+            const float off_even = (H ? 1032.0f : 8.0f) * corr[m], off_odd = (H ? 72.0f : 8.0f) * corr[m];
 #pragma unroll
             for(int j = 0; j < 8; j++){
+                const float off = (j & 1) ? off_odd : off_even;
                 const float lo = acc[m][j] - off, hi = acc[m][8 + j] - off;
                 const float mine = hi32 ? hi : lo, send = hi32 ? lo : hi;
                 k8[j] = mine + __shfl_xor(send, 32, 64);
@@ -533,24 +653,28 @@ __device__ __forceinline__ void df_task(const DfArgs &a, const DfT &t, uint2 (&w
         for(int m = 0; m < M; m++){
             const float v = ((red[(0 * DF_MB + m) * DF_CW + tid] + red[(1 * DF_MB + m) * DF_CW + tid])
                            + red[(2 * DF_MB + m) * DF_CW + tid]) + red[(3 * DF_MB + m) * DF_CW + tid];
-            df_st(dst + (size_t)m * mstride + col, v, a.epoch);
+            df_st(dst + (size_t)m * mstride + col, v * unscale, a.epoch);
         }
     }
     DF_STAMP(14);
 }
 
+template<bool H>
 __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
     __shared__ DfMeta mt;
-    __shared__ __align__(16) float xs[DF_NG][DF_RMAX][DF_MB];   /* x[m][r] * scale(r, g), the m side by side */
-    __shared__ float red[4 * DF_MB * DF_CW];
-    __shared__ int giveup;
+    __shared__ __align__(16) uint32_t xs_raw[DF_NG * DF_RMAX * DF_MB];   /* staged inputs: df_stage (fp16 pairs) or df_stage_f32 */
+    __shared__ float wmax[4];
     __shared__ DfT tasks[DF_MAXTASKS];
     __shared__ int wcount[4];
+    __shared__ float red[4 * DF_MB * DF_CW];
+    __shared__ int giveup;
     const int tid = threadIdx.x;
     __builtin_amdgcn_s_setprio(3);
 #ifdef QLMX_DF_TRACE
     int df_nev = 0;
-    if(tid < DF_TRACE_EV && blockIdx.x < DF_TRACE_WG) df_trace_tab[blockIdx.x][tid] = 0;
+    __shared__ u64 df_ev[DF_TRACE_EV];
+    if(tid < DF_TRACE_EV) df_ev[tid] = 0;
+    __syncthreads();
 #endif
     DF_STAMP(1);
     /* The tag of this call's partial sums is one more than the last finished call's, which lives in
@@ -622,14 +746,20 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
     /* ---- this workgroup's tasks, list 1 (gate|up) then list 2 (down), in one stream so that the
      * first digits of a task are already on their way while the task before it finishes ---- */
     /* Groups -- (problem, matrix) in list 1, problems in list 2 -- go to the XCDs round robin, whole, so that the
-     * scale sectors that a group's column chunks share meet in one L2. With fewer than 8 groups that would leave
-     * XCDs without work (a single token: 4 groups, half the device idle and two rounds of tasks on the other
-     * half), so a group's chunks are then cut into `parts` pieces that go to different XCDs (host table). */
+     * scale sectors that a group's column chunks share meet in one L2. The groups left over after the last full
+     * round of 8 would give some XCDs a whole group more than others (a second task for a sixth of their
+     * workgroups while others have none; with a single token: 4 groups, half the device idle), so the chunks of
+     * each of those are cut into `parts` pieces that go to different XCDs (host table by the number left over). */
     const int ngrp1 = 2 * nprob;
-    const int parts1 = ngrp1 < 8 ? (int)((a.parts1 >> (8 * ngrp1)) & 0xFFu) : 1, parts2 = nprob < 8 ? (int)((a.parts2 >> (8 * nprob)) & 0xFFu) : 1;
+    const int rem1 = ngrp1 & 7, rem2 = nprob & 7, full1 = ngrp1 - rem1, full2 = nprob - rem2;
+    const int parts1 = (int)((a.parts1 >> (8 * rem1)) & 0xFFu), parts2 = (int)((a.parts2 >> (8 * rem2)) & 0xFFu);
     const int cpp1 = df_div(a.NC1, parts1, 1.0f / (float)parts1), cpp2 = df_div(a.NC2, parts2, 1.0f / (float)parts2);   /* chunks per piece */
-    const int tpg1 = cpp1 * a.S1, nvg1 = ngrp1 * parts1, lim1 = ((nvg1 + 7) >> 3) * tpg1;
-    const int tpg2 = cpp2 * a.S2, nvg2 = nprob * parts2, lim2 = ((nvg2 + 7) >> 3) * tpg2;
+    const int tpw1 = a.NC1 * a.S1, tpw2 = a.NC2 * a.S2;               /* tasks of a whole group */
+    const int tpg1 = cpp1 * a.S1, tpg2 = cpp2 * a.S2;                 /* tasks of a piece */
+    const int nw1 = (full1 >> 3) * tpw1, nw2 = (full2 >> 3) * tpw2;   /* tasks that whole groups give each XCD */
+    const int nvg1 = rem1 * parts1, nvg2 = rem2 * parts2;             /* pieces */
+    const int lim1 = nw1 + ((nvg1 + 7) >> 3) * tpg1, lim2 = nw2 + ((nvg2 + 7) >> 3) * tpg2;
+    const float rtpw1 = 1.0f / (float)tpw1, rtpw2 = 1.0f / (float)tpw2;
     const float rtpg1 = 1.0f / (float)tpg1, rtpg2 = 1.0f / (float)tpg2, rS1 = 1.0f / (float)a.S1, rS2 = 1.0f / (float)a.S2;
     const float rparts1 = 1.0f / (float)parts1, rparts2 = 1.0f / (float)parts2;
     /* The task list of this workgroup is worked out once, one candidate per thread, and kept in LDS: candidate k
@@ -643,9 +773,13 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
         DfT t; t.list = 0; t.wq = 0; t.wg = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = 0;
         if(tid < c1){
             const int q = slot0 + tid * nslot;
-            const int qd = df_div(q, tpg1, rtpg1), vg = qd * 8 + xcd, sub = q - qd * tpg1;
-            if(vg < nvg1){
-                const int g = df_div(vg, parts1, rparts1), part = vg - g * parts1, cl = df_div(sub, a.S1, rS1);
+            /* slot q of this XCD: first its whole groups, then its pieces of the groups left over */
+            const bool whole = q < nw1;
+            const int qq = whole ? q : q - nw1, tp = whole ? tpw1 : tpg1;
+            const int qd = df_div(qq, tp, whole ? rtpw1 : rtpg1), vg = qd * 8 + xcd, sub = qq - qd * tp;
+            if(whole || vg < nvg1){
+                const int gp = df_div(vg, parts1, rparts1);
+                const int g = whole ? vg : full1 + gp, part = whole ? 0 : vg - gp * parts1, cl = df_div(sub, a.S1, rS1);
                 t.list = 1; t.prob = g >> 1; t.mat = g & 1; t.chunk = part * cpp1 + cl; t.sl = sub - cl * a.S1;
                 t.N = a.F; t.k0 = t.sl * a.R1; t.rows = min(a.R1, a.D - t.k0); t.M = mt.p_M[t.prob];
                 const int ex = mt.p_e[t.prob];
@@ -654,9 +788,12 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
             }
         } else if(tid < c1 + c2){
             const int q = slot0 + (tid - c1) * nslot;
-            const int qd = df_div(q, tpg2, rtpg2), vg = qd * 8 + xcd, sub = q - qd * tpg2;
-            if(vg < nvg2){
-                const int prob = df_div(vg, parts2, rparts2), part = vg - prob * parts2, cl = df_div(sub, a.S2, rS2);
+            const bool whole = q < nw2;
+            const int qq = whole ? q : q - nw2, tp = whole ? tpw2 : tpg2;
+            const int qd = df_div(qq, tp, whole ? rtpw2 : rtpg2), vg = qd * 8 + xcd, sub = qq - qd * tp;
+            if(whole || vg < nvg2){
+                const int gp = df_div(vg, parts2, rparts2);
+                const int prob = whole ? vg : full2 + gp, part = whole ? 0 : vg - gp * parts2, cl = df_div(sub, a.S2, rS2);
                 t.list = 2; t.prob = prob; t.mat = 0; t.chunk = part * cpp2 + cl; t.sl = sub - cl * a.S2;
                 t.N = a.D; t.k0 = t.sl * a.R2; t.rows = min(a.R2, a.F - t.k0); t.M = mt.p_M[prob];
                 const int ex = mt.p_e[prob];
@@ -694,7 +831,7 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
         return t;
     };
     uint2 w0[DF_BATCH], w1[DF_BATCH];
-    const int hs1 = a.R1 >> 5, hs2 = a.R2 >> 5;               /* steps per half task */
+    const int hs1 = a.R1 >> (H ? 6 : 5), hs2 = a.R2 >> (H ? 6 : 5);   /* steps (of 32 rows, fp32 loop: 16) per half task */
     const int gprF = a.F / a.group, gprD = a.D / a.group;     /* scale groups per row of w1|w3 and of w2 */
     const int cpg = a.group >= DF_CW ? a.group / DF_CW : 1;   /* chunks per scale group when the group is wider than a chunk */
     /* first scale of a task: its first row, its chunk's first group */
@@ -715,10 +852,10 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
     DfT cur = fetch();
     DF_STAMP(21);
     if(cur.list){
-        const signed char *dp = df_digits(a, cur); const int hs = cur.list == 1 ? hs1 : hs2;
+        const signed char *dp = df_digits<H>(a, cur); const int hs = cur.list == 1 ? hs1 : hs2;
         scales_ahead(cur, csc);
-        DF_LOAD(w0, dp, (size_t)cur.N >> 1, cur.rows, hs, 0)
-        DF_LOAD(w1, dp, (size_t)cur.N >> 1, cur.rows, hs, 1)
+        df_load<H>(w0, dp, (size_t)cur.N >> 1, cur.rows, hs, 0);
+        df_load<H>(w1, dp, (size_t)cur.N >> 1, cur.rows, hs, 1);
     }
     DF_STAMP(22);
     while(cur.list){
@@ -730,59 +867,69 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
          * that is still on its way */
         float nsc[DF_NG];
         scales_ahead(pre, nsc);
-        const signed char *ndp = df_digits(a, pre); const int nhs = pre.list == 1 ? hs1 : hs2;
-        auto next0 = [&](){ DF_LOAD(w0, ndp, (size_t)pre.N >> 1, pre.rows, nhs, 0) };
-        auto next1 = [&](){ DF_LOAD(w1, ndp, (size_t)pre.N >> 1, pre.rows, nhs, 1) };
+        const signed char *ndp = df_digits<H>(a, pre); const int nhs = pre.list == 1 ? hs1 : hs2;
+        auto next0 = [&](){ df_load<H>(w0, ndp, (size_t)pre.N >> 1, pre.rows, nhs, 0); };
+        auto next1 = [&](){ df_load<H>(w1, ndp, (size_t)pre.N >> 1, pre.rows, nhs, 1); };
         const int hs = cur.list == 1 ? hs1 : hs2;
         const int prob = cur.prob, chunk = cur.chunk, k0 = cur.k0, rows = cur.rows, M = cur.M;
         u64 *dst; size_t mstride;
         if(cur.list == 1){ dst = a.part1 + ((((size_t)prob * 2 + cur.mat) * a.S1 + cur.sl) * DF_MB) * a.F; mstride = (size_t)a.F; }
         else             { dst = a.part2 + (((size_t)prob * a.S2 + cur.sl) * DF_MB) * a.D;                  mstride = (size_t)a.D; }
-        auto prep = [&](){
+        auto prep = [&]() -> float {
+            /* thread = row of the task (rows <= DF_RMAX = the threads) */
+            const int r = tid; const bool live = r < rows;
+            float v[DF_NG][DF_MB];
             if(cur.list == 1){
-                __syncthreads();                             /* the previous task is done with xs */
-                for(int r = tid; r < rows; r += DF_THREADS){
-                    float sc[DF_NG], xv[DF_MB];
+                float xv[DF_MB];
 #pragma unroll
-                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = (gg < ng && chunk * DF_CW + gg * a.group < a.F) ? csc[gg] : 0.0f;
+                for(int m = 0; m < DF_MB; m++)
+                    xv[m] = (live && m < M) ? a.x[(size_t)mt.rowtok[mt.p_row0[prob] + m] * a.D + k0 + r] : 0.0f;
 #pragma unroll
-                    for(int m = 0; m < DF_MB; m++)
-                        xv[m] = m < M ? a.x[(size_t)mt.rowtok[mt.p_row0[prob] + m] * a.D + k0 + r] : 0.0f;
+                for(int gg = 0; gg < DF_NG; gg++){
+                    const float sc = (gg < ng && chunk * DF_CW + gg * a.group < a.F) ? csc[gg] : 0.0f;
 #pragma unroll
-                    for(int gg = 0; gg < DF_NG; gg++)
-                        *(float2 *)&xs[gg][r][0] = make_float2(xv[0] * sc[gg], xv[1] * sc[gg]);
+                    for(int m = 0; m < DF_MB; m++) v[gg][m] = xv[m] * sc;
                 }
-                __syncthreads();
             } else {
                 const u64 *p1 = a.part1 + (((size_t)prob * 2) * a.S1 * DF_MB) * a.F + k0;
                 const size_t sstride = (size_t)DF_MB * a.F;
-                df_wait_first(2 * a.S1, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, [=](int i){ return p1 + (size_t)i * sstride; });
-                for(int r = tid; r < rows; r += DF_THREADS){
-                    float sc[DF_NG];
+                /* with a full grid, one polling thread per producer first (everybody re-reading its sums until they
+                 * are there slows the producers down: T=16 +0.6 us per layer); with few workgroups the poll and its
+                 * barrier only add to the chain (T=1, 4: -0.3 us without) */
+                if(lim1 * 2 > nslot) df_wait_first(2 * a.S1, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, [=](int i){ return p1 + (size_t)i * sstride; });
+                float hv[DF_MB];
 #pragma unroll
-                    for(int gg = 0; gg < DF_NG; gg++) sc[gg] = (gg < ng && chunk * DF_CW + gg * a.group < a.D) ? csc[gg] : 0.0f;
-                    float hv[DF_MB];
+                for(int m = 0; m < DF_MB; m++) hv[m] = 0.0f;
+                if(live){
+                    /* h = silu(gate) * up (k_swiglu, cudalm.cu:2430-2432), both summed over the K slices in order.
+                     * The sums of both input rows are read in one round trip (a second row that does not exist
+                     * re-reads the first: its words are never written). */
+                    const u64 *src[2 * DF_MB];
 #pragma unroll
                     for(int m = 0; m < DF_MB; m++){
-                        hv[m] = 0.0f;
-                        if(m < M){
-                            /* h = silu(gate) * up (k_swiglu, cudalm.cu:2430-2432), both summed over the K slices in order */
-                            const u64 *const src[2] = { p1 + (size_t)m * a.F + r, p1 + (size_t)a.S1 * sstride + (size_t)m * a.F + r };
-                            float gu[2];
-                            df_sum_wait<2, 6>(src, sstride, a.S1, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, gu);
-                            hv[m] = (gu[0] / (1.0f + expf(-gu[0]))) * gu[1];
-                        }
+                        const int mm = m < M ? m : 0;
+                        src[2 * m] = p1 + (size_t)mm * a.F + r; src[2 * m + 1] = p1 + (size_t)a.S1 * sstride + (size_t)mm * a.F + r;
                     }
+                    float gu[2 * DF_MB];
+                    if(a.S1 <= 3) df_sum_wait<2 * DF_MB, 3>(src, sstride, a.S1, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, gu);
+                    else          df_sum_wait<2 * DF_MB, 6>(src, sstride, a.S1, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, gu);
 #pragma unroll
-                    for(int gg = 0; gg < DF_NG; gg++)
-                        *(float2 *)&xs[gg][r][0] = make_float2(hv[0] * sc[gg], hv[1] * sc[gg]);
+                    for(int m = 0; m < DF_MB; m++)
+                        if(m < M) hv[m] = (gu[2 * m] / (1.0f + expf(-gu[2 * m]))) * gu[2 * m + 1];
                 }
-                __syncthreads();
+#pragma unroll
+                for(int gg = 0; gg < DF_NG; gg++){
+                    const float sc = (gg < ng && chunk * DF_CW + gg * a.group < a.D) ? csc[gg] : 0.0f;
+#pragma unroll
+                    for(int m = 0; m < DF_MB; m++) v[gg][m] = hv[m] * sc;
+                }
             }
+            if(H) return df_stage(v, live, (uint32_t (*)[DF_RMAX / 2][2 * DF_MB])xs_raw, wmax);
+            return df_stage_f32(v, live, (float (*)[DF_RMAX][DF_MB])xs_raw);
         };
         /* the inner loop is compiled for 1 and 2 input rows */
-        if(M == 1) df_task<1>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1 DF_TRACE_ARG);
-        else       df_task<2>(a, cur, w0, w1, hs, xs, red, dst, mstride, prep, next0, next1 DF_TRACE_ARG);
+        if(M == 1) df_task<H, 1>(a, cur, w0, w1, hs, xs_raw, red, dst, mstride, prep, next0, next1 DF_TRACE_ARG);
+        else       df_task<H, 2>(a, cur, w0, w1, hs, xs_raw, red, dst, mstride, prep, next0, next1 DF_TRACE_ARG);
         cur = nxt;
 #pragma unroll
         for(int gg = 0; gg < DF_NG; gg++) csc[gg] = nsc[gg];
@@ -795,28 +942,30 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
         for(int q3 = blockIdx.x; q3 < ntask; q3 += G){
             const int n = q3 / a.NC2, chunk = q3 - n * a.NC2;
             const int col = chunk * DF_CW + tid;
-            {
-                const int S2 = a.S2, T = a.T, Dd = a.D; const int *pp = mt.pair_prob, *pm = mt.pair_m; const u64 *p2 = a.part2;
-                df_wait_first(a.K * S2, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, [=](int i) -> const u64 * {
-                    const int j = (i / S2) * T + n, prob = pp[j];
-                    if(prob < 0) return nullptr;
-                    return p2 + (((size_t)prob * S2 + i % S2) * DF_MB + pm[j]) * Dd + chunk * DF_CW; });
-            }
             if(col < a.D){
                 float o = a.out[(size_t)n * a.D + col];
-                for(int k = 0; k < a.K; k++){
-                    const int j = k * a.T + n, prob = mt.pair_prob[j];
-                    if(prob < 0) continue;
-                    const u64 *const src[1] = { a.part2 + (((size_t)prob * a.S2) * DF_MB + mt.pair_m[j]) * a.D + col };
-                    float y[1];
-                    df_sum_wait<1, 12>(src, (size_t)DF_MB * a.D, a.S2, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, y);
-                    o = o + a.gate[j] * y[0];
+                /* two passes' sums per round trip; an invalid pair re-reads the other's words and adds nothing */
+                for(int k = 0; k < a.K; k += 2){
+                    const int j0 = k * a.T + n, j1 = min(k + 1, a.K - 1) * a.T + n;
+                    const int prob0 = mt.pair_prob[j0], prob1 = k + 1 < a.K ? mt.pair_prob[j1] : -1;
+                    if(prob0 < 0 && prob1 < 0) continue;
+                    const int ja = prob0 >= 0 ? j0 : j1, jb = prob1 >= 0 ? j1 : j0;
+                    const u64 *const src[2] = { a.part2 + (((size_t)mt.pair_prob[ja] * a.S2) * DF_MB + mt.pair_m[ja]) * a.D + col,
+                                                a.part2 + (((size_t)mt.pair_prob[jb] * a.S2) * DF_MB + mt.pair_m[jb]) * a.D + col };
+                    float y[2];
+                    df_sum_wait<2, 12>(src, (size_t)DF_MB * a.D, a.S2, a.epoch ^ a.wait_xor, a.spin_limit, &giveup, a.status, y);
+                    if(prob0 >= 0) o = o + a.gate[j0] * y[0];
+                    if(prob1 >= 0) o = o + a.gate[j1] * y[1];
                 }
                 a.out[(size_t)n * a.D + col] = o;
             }
         }
     }
     DF_STAMP(4);
+#ifdef QLMX_DF_TRACE
+    __syncthreads();
+    if(tid < DF_TRACE_EV && blockIdx.x < DF_TRACE_WG) df_trace_tab[blockIdx.x][tid] = df_ev[tid];
+#endif
     /* the last workgroup to get here closes the call: clears the count and publishes the tag */
     if(tid == 0){
         const unsigned done = __hip_atomic_fetch_add(a.ctl + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -826,7 +975,6 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
         }
     }
 }
-#undef DF_LOAD
 
 /* ------------------------------------------------------------------------------------------
  * Host side. Per device: the launch shape, a status word in pinned host memory, a grow-only
@@ -860,7 +1008,10 @@ int qlmx_decode_setup(int device){
     *dv.status = 0;
     int nb = 0; hipDeviceProp_t pr;
     QLMX_HIP(hipGetDeviceProperties(&pr, device), "decode device properties");
-    QLMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, k_decode_fused, DF_THREADS, 0), "decode occupancy");
+    int nb32 = 0;
+    QLMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, k_decode_fused<true>, DF_THREADS, 0), "decode occupancy");
+    QLMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb32, k_decode_fused<false>, DF_THREADS, 0), "decode occupancy");
+    if(nb32 < nb) nb = nb32;                  /* one grid size for both loops: every workgroup of a launch must be resident */
     if(nb > 4) nb = 4;
     dv.grid = (nb * pr.multiProcessorCount) & ~7;
     QLMX_REQUIRE(dv.grid >= 8, "decode setup: device too small (%d resident workgroups)", dv.grid);
@@ -901,7 +1052,7 @@ static int df_rows(int Kdim, double tasks_per_slice, int grid){
     while((Kdim + R - 1) / R > 32 && R < DF_RMAX) R <<= 1;
     return R;
 }
-/* Rows per task of list 2 (a multiple of 32): as many slices of the contraction as still leave one task per
+/* Rows per task of list 2 (a multiple of 64, two halves of whole 32-row steps): as many slices of the contraction as still leave one task per
  * resident workgroup -- a second round of tasks would double the list's time -- but at most 12, which is what
  * the combine reads in one round trip, and none shorter than 64 rows. */
 static int df_rows_down(int Kdim, double tasks_per_slice, int grid){
@@ -910,9 +1061,26 @@ static int df_rows_down(int Kdim, double tasks_per_slice, int grid){
     if(S > 12) S = 12;
     if(S > smax) S = smax;
     if(S < smin) S = smin;
-    int R = ((Kdim + S - 1) / S + 31) & ~31;
+    int R = ((Kdim + S - 1) / S + 63) & ~63;
     if(R > DF_RMAX) R = DF_RMAX;
     return R;
+}
+
+/* Which multiply loop the decode layer runs. fp32 (the default): inputs as they are, 2.6 / 3.6 vector
+ * instructions per digit for one / two input rows, 4e-7 relative L2 on a layer's output against the fp32 oracle.
+ * fp16 inputs: the staged inputs as fp16 pairs and v_dot2_f32_f16, 1.4 / 2.0 instructions per digit, inputs
+ * rounded to 11 bits (3.7e-4), 1-4 % faster per layer (the layer is bound by its chain of hand-overs and by HBM,
+ * not by this loop). QLMX_DECODE_MATH=fp16 in the environment (read at the first call) or qlmx_decode_math(1)
+ * selects the fp16 loop, qlmx_decode_math(0) the fp32 one. */
+static int g_df_math = -1;
+static bool df_math_fp16(){
+    if(g_df_math < 0){ const char *e = getenv("QLMX_DECODE_MATH"); g_df_math = (e && !strcmp(e, "fp16")) ? 1 : 0; }
+    return g_df_math != 0;
+}
+extern "C" int qlmx_decode_math(int fp16_inputs){
+    QLMX_REQUIRE(fp16_inputs == 0 || fp16_inputs == 1, "qlmx_decode_math: 0 (fp32 loop) or 1 (fp16 inputs), not %d", fp16_inputs);
+    g_df_math = fp16_inputs;
+    return QLMX_OK;
 }
 
 /* Both entry points: checks, launch shape, workspace (`fixed`: the static array, else the grow-only one), launch. */
@@ -960,10 +1128,14 @@ static int df_forward(bool fixed, const char *who, const float *x, const int *as
         rc = df_reserve(dv.grown, 1, words2, st); if(rc) return rc;
         a.ctl = dv.grown.ctl; a.part1 = dv.grown.part[0]; a.part2 = dv.grown.part[1];
     }
-    /* fewer than 8 groups: the smallest number of pieces (a divisor of the chunk count) that gives every XCD one */
+    /* n groups left over after the last full round of 8: the number of pieces (a divisor of the chunk count) that
+     * leaves the fullest XCD with the fewest chunks, the smallest such number */
     a.parts1 = 0; a.parts2 = 0;
     for(int n = 0; n < 8; n++){
-        auto pieces = [&](int NC){ int pcs = NC; for(int c = 1; c <= NC; c++) if(NC % c == 0 && n * c >= 8){ pcs = c; break; } return n == 0 ? 1 : pcs; };
+        auto pieces = [&](int NC){
+            int best = 1, load = NC;
+            for(int c = 1; c <= NC && n > 0; c++) if(NC % c == 0){ const int l = ((n * c + 7) / 8) * (NC / c); if(l < load){ load = l; best = c; } }
+            return best; };
         a.parts1 |= (u64)pieces(a.NC1) << (8 * n); a.parts2 |= (u64)pieces(a.NC2) << (8 * n);
     }
     a.status = dv.status; a.epoch = 0;
@@ -980,7 +1152,8 @@ static int df_forward(bool fixed, const char *who, const float *x, const int *as
             return QLMX_E_LIMIT;
         }
     }
-    hipLaunchKernelGGL(k_decode_fused, dim3(grid), dim3(DF_THREADS), 0, st, a);
+    if(df_math_fp16()) hipLaunchKernelGGL(k_decode_fused<true>, dim3(grid), dim3(DF_THREADS), 0, st, a);
+    else               hipLaunchKernelGGL(k_decode_fused<false>, dim3(grid), dim3(DF_THREADS), 0, st, a);
     QLMX_LAUNCH_CHECK("decode launch");
     return QLMX_OK;
 }

@@ -339,6 +339,14 @@ int qlmx_test_force_wait_timeout(int which);
  * column count is a multiple of 256, tile = 128 goes back; QLMX_NT_TILE=256 in the environment is the same switch
  * from outside the process. */
 int qlmx_nt_tile(int tile);
+/* Math mode of the decode layer (no counterpart in the reference, whose decode path multiplies in fp32; the same
+ * kind of choice as QLMX_MATH_MFMA_F16 for the training forward). fp16_inputs = 0, the default: the fp32 loop,
+ * 4e-7 relative L2 on a layer's output against the fp32 reference. fp16_inputs = 1: a task's inputs (x times the
+ * group scale, or silu(gate) * up times the group scale) are rounded to fp16 -- 11 significant bits, scaled per
+ * task so that nothing underflows -- and multiplied with the exact digits by v_dot2_f32_f16 into fp32 sums:
+ * 3.7e-4, and 1-4 % faster per layer. Applies to both decode entry points from the next call on;
+ * QLMX_DECODE_MATH=fp16 in the environment is the same switch from outside the process. */
+int qlmx_decode_math(int fp16_inputs);
 /* Test hook. qlmx_step takes the square roots of the second moment with a short form of the correctly rounded
  * sqrtf() that is valid for arguments in [2^-96, +infinity] (and switches to sqrtf() itself below that). This
  * compares the two forms on the device for the `count` consecutive bit patterns starting at first_bits and adds

@@ -1,8 +1,11 @@
 """GPU parity of the decode-shaped (few-token) expert path: the streaming GEMV behind
 qlmx_moe_gemm_nn and the fused qlmx_moe_decode_forward, against the CPU oracle's rendered-weights
-fp32 layer (moe_forward call order, cudalm.cu:4193-4228). fp32 math: tolerance 1e-3 relative L2 as
-stated for matmul outputs, observed ~1e-6; routing indices come from the oracle's router and are
-consumed as given."""
+fp32 layer (moe_forward call order, cudalm.cu:4193-4228). Tolerance 1e-3 relative L2 as stated for
+matmul outputs. The fused layer has two multiply loops and every layer test runs with both: the default
+fp32 one differs from the oracle in summation order and the libm exp only (observed 4e-7, held to 2e-5),
+the other (qlmx_decode_math(1)) takes its inputs as fp16 pairs (11 significant bits; observed 2.4e-4 ..
+4.9e-4 on a layer's output, held to 7e-4 here). Routing indices come from the oracle's router and are consumed as
+given."""
 import numpy as np
 import pytest
 
@@ -17,6 +20,14 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(scope="module")
 def q():
     return pkg.load()
+
+
+@pytest.fixture(params=[0, 1], ids=["fp32", "fp16-inputs"])
+def tol(request, q):
+    """Selects the decode layer's multiply loop for one test and returns the bound its output is held to."""
+    q.call("qlmx_decode_math", request.param)
+    yield 7e-4 if request.param else 2e-5
+    q.call("qlmx_decode_math", 0)
 
 
 def dev(a):
@@ -81,7 +92,7 @@ def test_gemv_small_rows_vs_oracle(q, orc, K, N):
 
 @pytest.mark.parametrize("T,E,D,F,K", [(1, 32, 768, 2048, 2), (4, 32, 768, 2048, 2), (16, 32, 768, 2048, 2), (4, 8, 768, 2048, 2), (16, 8, 768, 2048, 2),
                                        (16, 4, 256, 384, 4), (5, 3, 128, 256, 1), (7, 6, 1024, 640, 3), (3, 4, 2048, 256, 2)])
-def test_decode_forward_vs_oracle_layer(q, orc, T, E, D, F, K):
+def test_decode_forward_vs_oracle_layer(q, orc, tol, T, E, D, F, K):
     import torch
     d, s, P, n = encode_layer(orc, 11 + T, E, D, F)
     x = orc.normal(T * D, 11, 2)
@@ -99,7 +110,7 @@ def test_decode_forward_vs_oracle_layer(q, orc, T, E, D, F, K):
     torch.cuda.synchronize()
     err = orc.relerr(out.cpu().numpy() - res, want - res)
     assert err < 1e-3, err
-    assert err < 2e-5, err          # fp32 math: only summation order and the libm exp differ
+    assert err < tol, err
     # run-to-run determinism: slice order, not arrival order, fixes the sums
     out2 = dev(res)
     q.decode_forward(dev(x), dev(asn), dev(gate), out2, dd, ds, 128, 0, n, 2 * n, T, K, E, D, F)
@@ -107,7 +118,7 @@ def test_decode_forward_vs_oracle_layer(q, orc, T, E, D, F, K):
     assert torch.equal(out, out2)
 
 
-def test_decode_all_tokens_one_expert(q, orc):
+def test_decode_all_tokens_one_expert(q, orc, tol):
     """Collision case: 16 tokens on the same two experts -> problems are cut into row pairs."""
     import torch
     T, E, D, F, K = 16, 4, 256, 512, 2
@@ -121,10 +132,10 @@ def test_decode_all_tokens_one_expert(q, orc):
     out = torch.zeros(T * D, device="cuda")
     q.decode_forward(dev(x), dev(asn), dev(gate), out, dev(d), dev(s), 128, 0, n, 2 * n, T, K, E, D, F)
     torch.cuda.synchronize()
-    assert orc.relerr(out.cpu().numpy(), want) < 2e-5
+    assert orc.relerr(out.cpu().numpy(), want) < tol
 
 
-def test_decode_group_256_and_rejected_groups(q, orc):
+def test_decode_group_256_and_rejected_groups(q, orc, tol):
     """Scale groups of 256 (one per task row) go through the same kernel; 64 and 96 are refused."""
     import torch
     T, E, D, F, K = 4, 4, 512, 768, 2
@@ -139,13 +150,13 @@ def test_decode_group_256_and_rejected_groups(q, orc):
     out = torch.zeros(T * D, device="cuda")
     q.decode_forward(dev(x), dev(asn), dev(gate), out, dev(d), dev(s), 256, 0, n, 2 * n, T, K, E, D, F)
     torch.cuda.synchronize()
-    assert orc.relerr(out.cpu().numpy(), want) < 2e-5
+    assert orc.relerr(out.cpu().numpy(), want) < tol
     for g in (64, 96):
         with pytest.raises(pkg.QlmxError, match="group"):
             q.decode_forward(dev(x), dev(asn), dev(gate), out, dev(d), dev(s), g, 0, n, 2 * n, T, K, E, D, F)
 
 
-def test_decode_invalid_expert_is_skipped(q, orc):
+def test_decode_invalid_expert_is_skipped(q, orc, tol):
     """A pair with an out-of-range expert adds nothing; the other pairs are unaffected."""
     import torch
     T, E, D, F, K = 3, 4, 256, 512, 2
@@ -161,7 +172,7 @@ def test_decode_invalid_expert_is_skipped(q, orc):
     out = torch.zeros(T * D, device="cuda")
     q.decode_forward(dev(x), dev(bad), dev(gate), out, dev(d), dev(s), 128, 0, n, 2 * n, T, K, E, D, F)
     torch.cuda.synchronize()
-    assert orc.relerr(out.cpu().numpy(), want) < 2e-5
+    assert orc.relerr(out.cpu().numpy(), want) < tol
     allbad = np.full(K * T, -1, np.int32)
     out.zero_()
     q.decode_forward(dev(x), dev(allbad), dev(gate), out, dev(d), dev(s), 128, 0, n, 2 * n, T, K, E, D, F)
@@ -169,7 +180,7 @@ def test_decode_invalid_expert_is_skipped(q, orc):
     assert float(out.abs().max()) == 0.0
 
 
-def test_decode_repeated_calls_alternating_shapes(q, orc):
+def test_decode_repeated_calls_alternating_shapes(q, orc, tol):
     """The hand-over words carry the call's epoch: stale partial sums of earlier calls, of other
     shapes and token counts, must never be taken for current ones."""
     import torch
@@ -192,10 +203,10 @@ def test_decode_repeated_calls_alternating_shapes(q, orc):
         outs.append((out, want))
     torch.cuda.synchronize()
     for out, want in outs:
-        assert orc.relerr(out.cpu().numpy(), want) < 2e-5
+        assert orc.relerr(out.cpu().numpy(), want) < tol
 
 
-def test_decode_wait_timeout_is_reported_once(q, orc):
+def test_decode_wait_timeout_is_reported_once(q, orc, tol):
     """The waits between the three task lists are bounded. Forced from the host (qlmx_test_force_wait_timeout: for
     one launch every wait looks, for one poll, for a tag nobody writes) all of them give up, the kernel still ends
     normally, the NEXT call returns QLMX_E_HIP once, and the call after that is correct again."""
@@ -220,7 +231,7 @@ def test_decode_wait_timeout_is_reported_once(q, orc):
     out.zero_()
     q.decode_forward(*args, out, dd, ds, 128, 0, n, 2 * n, T, K, E, D, F)
     torch.cuda.synchronize()
-    assert orc.relerr(out.cpu().numpy(), want) < 2e-5
+    assert orc.relerr(out.cpu().numpy(), want) < tol
 
 
 def test_decode_limits(q):

@@ -41,6 +41,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--fwd-math", default="f16", choices=["f16", "bf16x2"],
                     help="train, c5: forward GEMMs on the fp16 matrix core (one MFMA per product, 2e-4 relative L2) or as bf16 hi+lo (two, 3e-6)")
+    ap.add_argument("--bwd-streams", type=int, default=None, choices=[1, 2],
+                    help="2 = the weight gradient of every backward flush on the library's side stream beside its input gradient, 1 = one after the other; "
+                         "default: 2 for the config-3 step (+3.6 %%), 1 for config 5 (no gain at its size)")
     ap.add_argument("--step-only", action="store_true", help="train: skip the per-launch repetitions, so that a kernel trace holds nothing but steps")
     ap.add_argument("--adamw-weights", type=int, default=120 * 2 ** 20)
     ap.add_argument("--render-p", type=int, default=0, help="adamw: also write the fp32 view P (4 B/weight more)")
@@ -139,19 +142,31 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
     p_g13 = P(probs(Xp, D, dgp, F, G, 0, o1, True) + probs(Xp, D, dup, F, G, 0, o3, True))
     # the order of moe_forward / moe_backward (cudalm.cu:4211-4225, 4333-4335, 4362-4366): each backward flush
     # holds the weight gradient and the input gradient of the same operands
-    calls = [
-        ("fwd w1,w3 (nn)", lambda: q.gemm_nn(d, s, group, p_w13, 2 * E, D, F, ACT_BF16, FWD, stream), 2),
-        ("fwd w2 (nn)", lambda: q.gemm_nn(d, s, group, p_w2, E, F, D, ACT_BF16, FWD, stream), 1),
-        ("wgrad w2 (nt)", lambda: q.gemm_nt(p_g2, E, F, D, ACT_BF16, MATH_MFMA, stream), 1),
-        ("dgrad w2 (tn)", lambda: q.gemm_tn(d, s, group, p_d2, E, D, F, ACT_BF16, MATH_MFMA, stream), 1),
-        ("wgrad w1,w3 (nt)", lambda: q.gemm_nt(p_g13, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream), 2),
-        ("dgrad w1,w3 (tn pair)", lambda: q.gemm_tn_pair(d, s, group, p_d1, p_d3, E, F, D, ACT_BF16, MATH_MFMA, stream), 2),
-    ]
+    def mk(st):
+        return [
+            ("fwd w1,w3 (nn)", lambda: q.gemm_nn(d, s, group, p_w13, 2 * E, D, F, ACT_BF16, FWD, st), 2),
+            ("fwd w2 (nn)", lambda: q.gemm_nn(d, s, group, p_w2, E, F, D, ACT_BF16, FWD, st), 1),
+            ("wgrad w2 (nt)", lambda: q.gemm_nt(p_g2, E, F, D, ACT_BF16, MATH_MFMA, st), 1),
+            ("dgrad w2 (tn)", lambda: q.gemm_tn(d, s, group, p_d2, E, D, F, ACT_BF16, MATH_MFMA, st), 1),
+            ("wgrad w1,w3 (nt)", lambda: q.gemm_nt(p_g13, 2 * E, D, F, ACT_BF16, MATH_MFMA, st), 2),
+            ("dgrad w1,w3 (tn pair)", lambda: q.gemm_tn_pair(d, s, group, p_d1, p_d3, E, F, D, ACT_BF16, MATH_MFMA, st), 2),
+        ]
+    calls = mk(stream)
     unit = 2.0 * rows * D * F            # flops of one expert GEMM over all rows
 
     def step():
         for _, fn, _n in calls:
             fn()
+
+    if (args.bwd_streams or 2) == 2:
+        # each backward flush (cudalm.cu:4333-4335, 4362-4366) with its weight gradient on the library's side
+        # stream beside its input gradient: they read the same operands and write different outputs
+        side = mk(q.side_fork(stream)); q.side_join(stream)      # the handle is the same at every fork
+
+        def step():
+            calls[0][1](); calls[1][1]()
+            q.side_fork(stream); side[2][1](); calls[3][1](); q.side_join(stream)
+            q.side_fork(stream); side[4][1](); calls[5][1](); q.side_join(stream)
 
     tm = timed(torch, step, args.steps, args.warmup)
     per = {}
@@ -172,7 +187,9 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
     dom = max(per, key=lambda k: per[k]["ms"]) if per else "not timed"
     return {
         "workload": "%s: E=%d top-%d D=%d F=%d, %d bf16 tokens -> %d expert rows, Zipf(1.1) load (max %d, min %d rows); "
-                    "fwd+dgrad+wgrad = 9 grouped GEMMs in 6 launches" % (label, E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min())),
+                    "fwd+dgrad+wgrad = 9 grouped GEMMs in 6 launches%s" % (label, E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min()),
+                       ", the weight gradient of each backward flush on a second stream beside its input gradient" if (args.bwd_streams or 2) == 2 else ""),
+        "bwd_streams": args.bwd_streams or 2,
         "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tm["wall_ms"], "dtype": "bf16",
         "kernel_ms": tm, "per_launch": per, "beside_the_step": extra, "gflop_per_step": flops / 1e9,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
@@ -391,18 +408,30 @@ def bench_c5(torch, q, args, L=8, E=64, D=2048, F=1408, tokens=32768, topk=4):
         p_d2 = P(items(dyp, D, None, 0, dap, F, o2))
         p_g13 = P(items(Xp, D, dgp, F, G, 0, o1, True) + items(Xp, D, dup, F, G, 0, o3, True))
         p_d1 = P(items(dgp, F, None, 0, dXp, D, o1)); p_d3 = P(items(dup, F, None, 0, dXp, D, o3, beta=1.0))
-        calls += [
-            (lambda p=p_w13: q.gemm_nn(d, s, group, p, 2 * E, D, F, ACT_BF16, FWD, stream)),
-            (lambda p=p_w2: q.gemm_nn(d, s, group, p, E, F, D, ACT_BF16, FWD, stream)),
-            (lambda p=p_g2: q.gemm_nt(p, E, F, D, ACT_BF16, MATH_MFMA, stream)),
-            (lambda p=p_d2: q.gemm_tn(d, s, group, p, E, D, F, ACT_BF16, MATH_MFMA, stream)),
-            (lambda p=p_g13: q.gemm_nt(p, 2 * E, D, F, ACT_BF16, MATH_MFMA, stream)),
-            (lambda p=p_d1, pp=p_d3: q.gemm_tn_pair(d, s, group, p, pp, E, F, D, ACT_BF16, MATH_MFMA, stream)),
-        ]
+        calls.append(lambda st, p_w13=p_w13, p_w2=p_w2, p_g2=p_g2, p_d2=p_d2, p_g13=p_g13, p_d1=p_d1, p_d3=p_d3: [
+            (lambda: q.gemm_nn(d, s, group, p_w13, 2 * E, D, F, ACT_BF16, FWD, st)),
+            (lambda: q.gemm_nn(d, s, group, p_w2, E, F, D, ACT_BF16, FWD, st)),
+            (lambda: q.gemm_nt(p_g2, E, F, D, ACT_BF16, MATH_MFMA, st)),
+            (lambda: q.gemm_tn(d, s, group, p_d2, E, D, F, ACT_BF16, MATH_MFMA, st)),
+            (lambda: q.gemm_nt(p_g13, 2 * E, D, F, ACT_BF16, MATH_MFMA, st)),
+            (lambda: q.gemm_tn_pair(d, s, group, p_d1, p_d3, E, F, D, ACT_BF16, MATH_MFMA, st)),
+        ])
+    main_calls = [mk(stream) for mk in calls]
+    if (args.bwd_streams or 1) == 2:
+        side_st = q.side_fork(stream); q.side_join(stream)       # the handle is the same at every fork
+        side_calls = [mk(side_st) for mk in calls]
 
-    def gemms():
-        for fn in calls:
-            fn()
+        def gemms():
+            # each backward flush with its weight gradient on the library's side stream beside its input gradient
+            for m, sd in zip(main_calls, side_calls):
+                m[0](); m[1]()
+                q.side_fork(stream); sd[2](); m[3](); q.side_join(stream)
+                q.side_fork(stream); sd[4](); m[5](); q.side_join(stream)
+    else:
+        def gemms():
+            for m in main_calls:
+                for fn in m:
+                    fn()
 
     tg = timed(torch, gemms, steps, warmup)
     flops = L * 9 * 2.0 * rows * D * F

@@ -58,6 +58,8 @@ SIGNATURES = {
     "qlmx_memcpy_d2d": (c_i, [c_vp, c_vp, c_sz, c_vp]),
     "qlmx_memset": (c_i, [c_vp, c_i, c_sz, c_vp]),
     "qlmx_sync": (c_i, [c_vp]),
+    "qlmx_side_fork": (c_i, [c_vp, C.POINTER(c_vp)]),
+    "qlmx_side_join": (c_i, [c_vp]),
     "qlmx_qhashu": (C.c_uint, [c_u64]),
     "qlmx_qsri": (c_i, [c_f, c_u64, c_u64]),
     "qlmx_qclmp": (c_i, [c_i, c_i, c_i]),
@@ -266,6 +268,15 @@ class Qlmx:
 
     def sync(self, stream=None):
         self.call("qlmx_sync", stream)
+
+    def side_fork(self, stream=None):
+        """The library's side stream, ordered after what `stream` holds so far (a handle to pass as `stream`)."""
+        side = C.c_void_p()
+        self.call("qlmx_side_fork", stream, C.byref(side))
+        return side.value
+
+    def side_join(self, stream=None):
+        self.call("qlmx_side_join", stream)
 
 
 _cached = None

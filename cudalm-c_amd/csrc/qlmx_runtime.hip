@@ -71,6 +71,42 @@ extern "C" int qlmx_sync(void *stream){
     return QLMX_OK;
 }
 
+/* ---- a second stream beside the caller's, for launches that do not depend on each other ----
+ * One side stream and two events per device, made at the first fork (default priority, like every stream here).
+ * fork: the side stream waits for what `stream` holds so far; join: `stream` waits for what the side stream
+ * holds. Both are waits between queues on the device; the host does not block. */
+#define SIDE_MAX_DEVICES 16
+struct SideState { hipStream_t st = nullptr; hipEvent_t fork = nullptr, join = nullptr; };
+static SideState g_side[SIDE_MAX_DEVICES];
+static int side_of(SideState **out){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    int device = -1;
+    QLMX_HIP(hipGetDevice(&device), "side stream device");
+    QLMX_REQUIRE(device >= 0 && device < SIDE_MAX_DEVICES, "side stream: device %d is beyond the %d this library keeps state for", device, SIDE_MAX_DEVICES);
+    SideState &sd = g_side[device];
+    if(!sd.st){
+        QLMX_HIP(hipStreamCreateWithFlags(&sd.st, hipStreamNonBlocking), "side stream");
+        QLMX_HIP(hipEventCreateWithFlags(&sd.fork, hipEventDisableTiming), "side stream event");
+        QLMX_HIP(hipEventCreateWithFlags(&sd.join, hipEventDisableTiming), "side stream event");
+    }
+    *out = &sd;
+    return QLMX_OK;
+}
+extern "C" int qlmx_side_fork(void *stream, void **side){
+    QLMX_REQUIRE(side, "qlmx_side_fork: NULL out pointer");
+    SideState *sd; int rc = side_of(&sd); if(rc) return rc;
+    QLMX_HIP(hipEventRecord(sd->fork, (hipStream_t)stream), "side fork record");
+    QLMX_HIP(hipStreamWaitEvent(sd->st, sd->fork, 0), "side fork wait");
+    *side = (void *)sd->st;
+    return QLMX_OK;
+}
+extern "C" int qlmx_side_join(void *stream){
+    SideState *sd; int rc = side_of(&sd); if(rc) return rc;
+    QLMX_HIP(hipEventRecord(sd->join, sd->st), "side join record");
+    QLMX_HIP(hipStreamWaitEvent((hipStream_t)stream, sd->join, 0), "side join wait");
+    return QLMX_OK;
+}
+
 /* ---- host integer helpers (qlm.cuh:78-111) ---- */
 extern "C" unsigned int qlmx_qhashu(unsigned long long x){ return qx_hash(x); }
 extern "C" int qlmx_qsri(float v, unsigned long long i, unsigned long long t){

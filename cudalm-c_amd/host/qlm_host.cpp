@@ -445,7 +445,7 @@ static void mg_run_dual(void){
     g_qdual.clear();
 }
 
-static void mg_run(std::vector<MgItem> &v){
+static void mg_run(std::vector<MgItem> &v, void *stream = NULL){
     std::vector<char> done(v.size(), 0);
     for(size_t i = 0; i < v.size(); i++){
         if(done[i]) continue;
@@ -453,9 +453,9 @@ static void mg_run(std::vector<MgItem> &v){
         for(size_t j = i; j < v.size(); j++)
             if(!done[j] && v[j].mode == v[i].mode && v[j].K == v[i].K && v[j].N == v[i].N){ batch.push_back(v[j].p); done[j] = 1; }
         int rc;
-        if(v[i].mode == 0)      rc = qlmx_moe_gemm_nn(g_mg_q->d, g_mg_q->s, g_mg_q->group, batch.data(), (int)batch.size(), v[i].K, v[i].N, g_mg_act, g_mg_math, NULL);
-        else if(v[i].mode == 1) rc = qlmx_moe_gemm_tn(g_mg_q->d, g_mg_q->s, g_mg_q->group, batch.data(), (int)batch.size(), v[i].K, v[i].N, g_mg_act, g_mg_math, NULL);
-        else                    rc = qlmx_moe_gemm_nt(batch.data(), (int)batch.size(), v[i].K, v[i].N, g_mg_act, g_mg_math, NULL);
+        if(v[i].mode == 0)      rc = qlmx_moe_gemm_nn(g_mg_q->d, g_mg_q->s, g_mg_q->group, batch.data(), (int)batch.size(), v[i].K, v[i].N, g_mg_act, g_mg_math, stream);
+        else if(v[i].mode == 1) rc = qlmx_moe_gemm_tn(g_mg_q->d, g_mg_q->s, g_mg_q->group, batch.data(), (int)batch.size(), v[i].K, v[i].N, g_mg_act, g_mg_math, stream);
+        else                    rc = qlmx_moe_gemm_nt(batch.data(), (int)batch.size(), v[i].K, v[i].N, g_mg_act, g_mg_math, stream);
         if(rc != QLMX_OK){ fprintf(stderr, "grouped GEMM error %d at mg grouped: %s\n", rc, qlmx_last_error()); exit(1); }
     }
     v.clear();
@@ -492,4 +492,15 @@ static void mg_run_pairs(void){
     for(size_t j = 0; j < v1.size(); j++) if(!done[j]) r1.push_back(v1[j]);
     v0.swap(r0); v1.swap(r1);
 }
-void mg_flush(void){ mg_run_dual(); mg_run_pairs(); mg_run(g_q[0]); mg_run(g_q[1]); mg_run(g_q[2]); }
+/* The problems of a flush do not depend on each other except queue 1 on queue 0 (it accumulates into what queue 0
+ * writes). The weight gradients (queue 2) of a flush that also holds input gradients run on the library's side
+ * stream beside them: neither fills the device to the end of its last round of tiles. */
+void mg_flush(void){
+    mg_run_dual();
+    void *side = NULL;
+    const bool beside = !g_q[2].empty() && (!g_q[0].empty() || !g_q[1].empty()) && qlmx_side_fork(NULL, &side) == QLMX_OK;
+    if(beside) mg_run(g_q[2], side);
+    mg_run_pairs(); mg_run(g_q[0]); mg_run(g_q[1]);
+    if(beside){ if(qlmx_side_join(NULL) != QLMX_OK){ fprintf(stderr, "mg_flush: %s\n", qlmx_last_error()); exit(1); } }
+    else mg_run(g_q[2]);
+}

@@ -51,6 +51,16 @@ int         qlmx_memcpy_d2h(void *dst, const void *src, size_t bytes);
 int         qlmx_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
 int         qlmx_memset(void *dst, int value, size_t bytes, void *stream);
 int         qlmx_sync(void *stream);
+/* A second stream beside the caller's (no counterpart in the reference, which issues the grouped GEMMs of a
+ * flush one after the other on one stream, cudalm.cu:3243-3256). The weight gradient and the input gradient of a
+ * backward flush read the same operands and write different outputs; at config 3 neither fills the device to
+ * the end of its last round of tiles, and side by side they take 4 % less than one after the other.
+ * qlmx_side_fork(stream, &side): `side` (owned by the library, one per device) continues after everything queued
+ * on `stream` so far; pass it as the `stream` argument of the independent calls. qlmx_side_join(stream): `stream`
+ * continues after everything queued on the side stream. Neither blocks the host. Not for use under stream
+ * capture. */
+int         qlmx_side_fork(void *stream, void **side);
+int         qlmx_side_join(void *stream);
 
 /* ---- host integer helpers: the __host__ __device__ inlines of qlm.cuh:78-111, used by the
  *      reference's checkpoint code and selftest reference (cudalm.cu:10574-10580) ---- */

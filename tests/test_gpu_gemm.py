@@ -493,3 +493,45 @@ def test_mfma_nt_wide_tile(q, orc):
     assert np.array_equal(wide.view(np.uint32), narrow.view(np.uint32))
     with pytest.raises(pkg.QlmxError, match="128 or 256"):
         q.call("qlmx_nt_tile", 64)
+
+
+def test_side_stream_fork_join(q, orc):
+    """qlmx_side_fork / qlmx_side_join: work queued on the side stream starts after what the caller's stream held
+    at the fork, the caller's stream continues after it at the join; a backward flush with its weight gradient on
+    the side stream beside its input gradient gives the bits of the two launches one after the other."""
+    import torch
+    cur = torch.cuda.current_stream().cuda_stream
+    # ordering: a long fill on the caller's stream, a copy of its last bytes on the side stream, a read after the join
+    n = 1 << 28
+    src = torch.zeros(n, dtype=torch.uint8, device="cuda"); dst = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    for rep in range(3):
+        src.fill_(rep + 1)
+        side = q.side_fork(cur)
+        assert side and side != cur
+        q.call("qlmx_memcpy_d2d", dst, src[n - 4096:], 4096, side)
+        q.side_join(cur)
+        got = dst.clone()                                  # on the caller's stream, after the join
+        torch.cuda.synchronize()
+        assert int(got.min()) == rep + 1 and int(got.max()) == rep + 1
+    # a flush both ways
+    E, rows, K, N = 6, [700, 33, 0, 1290, 256, 64], 256, 512
+    tot = sum(rows); off = np.concatenate([[0], np.cumsum(rows)]).astype(int)
+    d, s, P = make_weights(orc, 17, E, K, N, 128)          # forward weights [K, N] per expert; dX[rows, K] = dY[rows, N] . W^T
+    dY = orc.bf16_round(orc.normal(tot * N, 17, 10)); X = orc.bf16_round(orc.normal(tot * K, 17, 11))
+    dYb, Xb = to_bf16_bits(dev(dY)), to_bf16_bits(dev(X))
+    dd, ds = dev(d), dev(s)
+    outs = []
+    for beside in (False, True):
+        G = dev(orc.normal(E * K * N, 17, 12, 0.1)); dX = torch.zeros(tot * K, device="cuda")
+        nt = q.problems([(Xb.data_ptr() + off[e] * K * 2, dYb.data_ptr() + off[e] * N * 2, G.data_ptr() + e * K * N * 4, 0, 0, rows[e], 1.0) for e in range(E)])
+        tn = q.problems([(dYb.data_ptr() + off[e] * N * 2, None, dX.data_ptr() + off[e] * K * 4, e * N * K, e * N * K // 128, rows[e], 0.0) for e in range(E)])
+        st = q.side_fork(cur) if beside else cur
+        q.gemm_nt(nt, E, K, N, pkg.ACT_BF16, pkg.MATH_MFMA, st)
+        q.gemm_tn(dd, ds, 128, tn, E, N, K, pkg.ACT_BF16, pkg.MATH_MFMA, cur)
+        if beside:
+            q.side_join(cur)
+        outs.append((G.clone(), dX.clone()))
+        torch.cuda.synchronize()
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    assert float(outs[0][1].abs().max()) > 0.0

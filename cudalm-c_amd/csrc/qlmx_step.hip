@@ -120,9 +120,11 @@ __device__ __forceinline__ ElemRes step_elem(const GroupCtx &c, float graw, int 
     return o;
 }
 
-/* STAT: the four counters are kept; HASP: the fp32 view is written. Both are fixed per launch, so they are
- * template parameters and the usual launch (neither) carries no trace of them. */
-template<bool ADAM, bool STAT, bool HASP>
+/* STAT: the four counters are kept; HASP: the fp32 view is written; V4: the second moment is stored as its
+ * fourth root (a.v4). All are fixed per launch, so they are template parameters and the usual launch (none of
+ * them) carries no trace of them: as a run-time flag, v4 made the compiler compute the second square root of
+ * every element and select (18 of 186 vector instructions per weight). */
+template<bool ADAM, bool STAT, bool HASP, bool V4>
 __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
     const int lane16 = threadIdx.x & 15;
     const int team = (int)((blockIdx.x * (unsigned)blockDim.x + threadIdx.x) >> 4);
@@ -142,10 +144,10 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
     c.dec = a.lr * a.wd * 128.0f;
     c.ms_old = a.m8s[gi];
     c.vs_old = (ADAM && a.v8s) ? a.v8s[gi] : 0.0f;
-    { float q1 = 1.0f * c.vs_old; if(a.v4) q1 = q1 * q1; c.veps = fmaxf(q1, 1e-8f); }
+    { float q1 = 1.0f * c.vs_old; if(V4) q1 = q1 * q1; c.veps = fmaxf(q1, 1e-8f); }
     c.b1 = a.b1; c.b2 = a.b2; c.omb1 = 1.0f - a.b1; c.omb2 = 1.0f - a.b2;
     c.inv_bc1 = a.inv_bc1; c.inv_sqrt_bc2 = a.inv_sqrt_bc2;
-    c.dmax = a.dmax; c.v4 = a.v4;
+    c.dmax = a.dmax; c.v4 = V4;
 
     const uint64_t kt  = a.t * QLMX_KT;
     const uint64_t ktm = kt + 0x5EEDULL * QLMX_KT;
@@ -176,7 +178,7 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
                 const int sh = 8 * (k & 3);
                 const float gr = gv[k] * c.gs;
                 const float mv = (float)(int)(signed char)(mword >> sh) * c.ms_old;
-                float sv = (float)((vword >> sh) & 0xFFu) * c.vs_old; if(c.v4) sv = sv * sv;
+                float sv = (float)((vword >> sh) & 0xFFu) * c.vs_old; if(V4) sv = sv * sv;
                 mn[k] = c.b1 * mv + c.omb1 * gr;
                 vv[k] = c.b2 * (sv * sv) + c.omb2 * gr * gr;
                 vmin = fminf(vmin, vv[k]);
@@ -193,7 +195,7 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
             for(int k = 0; k < 8; k++){
                 const float u = (mn[k] * c.inv_bc1) / (rv[k] * c.inv_sqrt_bc2 + c.veps);
                 uu[k] = fmaxf(-8.0f, fminf(8.0f, u));
-                if(c.v4) rv[k] = sqrtf(rv[k]);
+                if(V4) rv[k] = sqrtf(rv[k]);
             }
         } else {
 #pragma unroll
@@ -353,15 +355,17 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
     }
 }
 
-template<bool ADAM> static void step_launch_opt(const StepParams &a, unsigned blocks, hipStream_t st){
+template<bool ADAM, bool V4> static void step_launch_opt(const StepParams &a, unsigned blocks, hipStream_t st){
     const bool stat = a.stat != nullptr, hasp = a.P != nullptr;
-    if(stat && hasp)  hipLaunchKernelGGL((k_qlmx_step<ADAM, true, true>),   dim3(blocks), dim3(256), 0, st, a);
-    else if(stat)     hipLaunchKernelGGL((k_qlmx_step<ADAM, true, false>),  dim3(blocks), dim3(256), 0, st, a);
-    else if(hasp)     hipLaunchKernelGGL((k_qlmx_step<ADAM, false, true>),  dim3(blocks), dim3(256), 0, st, a);
-    else              hipLaunchKernelGGL((k_qlmx_step<ADAM, false, false>), dim3(blocks), dim3(256), 0, st, a);
+    if(stat && hasp)  hipLaunchKernelGGL((k_qlmx_step<ADAM, true, true, V4>),   dim3(blocks), dim3(256), 0, st, a);
+    else if(stat)     hipLaunchKernelGGL((k_qlmx_step<ADAM, true, false, V4>),  dim3(blocks), dim3(256), 0, st, a);
+    else if(hasp)     hipLaunchKernelGGL((k_qlmx_step<ADAM, false, true, V4>),  dim3(blocks), dim3(256), 0, st, a);
+    else              hipLaunchKernelGGL((k_qlmx_step<ADAM, false, false, V4>), dim3(blocks), dim3(256), 0, st, a);
 }
 static void step_launch(const StepParams &a, bool adam, unsigned blocks, hipStream_t st){
-    if(adam) step_launch_opt<true>(a, blocks, st); else step_launch_opt<false>(a, blocks, st);
+    /* v4 only exists for Adam's second moment (Lion keeps none) */
+    if(adam){ if(a.v4) step_launch_opt<true, true>(a, blocks, st); else step_launch_opt<true, false>(a, blocks, st); }
+    else step_launch_opt<false, false>(a, blocks, st);
 }
 
 /* qlm_step_launch (qlm.cuh:377-397) */

@@ -299,12 +299,15 @@ int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const
  * the same problem table from `assign` in LDS (stable counting sort by expert, the order of the
  * reference's host permutation, cudalm.cu:3586-3599).
  *
- * Task kernel: 256 threads cover 16 rows x 256 columns per step (a lane owns 16 columns = 8 bytes of
- * digits of one row; 16 lanes cover the 128 contiguous bytes of a row's chunk), two batches of
- * DF_BATCH steps in flight (the next batch is requested before the current one is consumed). The
- * input rows are staged in LDS already multiplied by the row's group scales, so the inner loop
- * loads digits only. Tasks of one (problem, matrix) are given to workgroups of one XCD so that the
- * 64-byte scale sectors shared by neighbouring chunks are fetched into one L2 only.
+ * Task kernel (a template over two multiply loops). fp32 loop, the default: 256 threads cover 16 rows x 256
+ * columns per step (a lane owns 16 columns = 8 bytes of digits of one row; 16 lanes cover the 128 contiguous
+ * bytes of a row's chunk). fp16-input loop (qlmx_decode_math(1)): 32 rows per step, a lane owns the same columns
+ * of two consecutive rows and multiplies both at once (see df_task). Either way a task is two halves of
+ * DF_BATCH 8-byte loads per lane, both in flight (the next task's halves are requested as soon as this task has
+ * consumed them). The input rows are staged in LDS already multiplied by the row's group scales, so the loop
+ * loads digits only. Tasks of one (problem, matrix) are given to workgroups of one XCD so that the 64-byte scale
+ * sectors shared by neighbouring chunks are fetched into one L2 only (the groups left over after a full round of
+ * 8 XCDs are cut into pieces, see the kernel).
  * ---------------------------------------------------------------------------------------- */
 #define DEC_MAXPAIR 64
 #define DF_THREADS 256
@@ -314,7 +317,8 @@ int qlmx_gemv_nn_dispatch(const signed char *d, const float *s, int group, const
 #define DF_CW 256             /* columns per task */
 #define DF_NG 2               /* scale groups per task row: group 128, or one when the group is a multiple of 256 */
 #define DF_RMAX 256           /* rows per task at most */
-#define DF_BATCH 8            /* 8-byte digit loads per lane and half task (4 steps of 32 rows, a lane's two rows each): a task is two halves of at most 128 rows */
+#define DF_BATCH 8            /* 8-byte digit loads per lane and half task (fp32 loop: 8 steps of 16 rows; fp16-input loop: 4 steps of
+                                 32 rows, a lane's two rows each): a task is two halves of at most 128 rows */
 #define DF_SPIN_LIMIT (1 << 17)
 #define DF_MAXTASKS 128        /* tasks of one workgroup at most (both lists); the host refuses shapes that would need more */
 typedef unsigned long long u64;

@@ -211,17 +211,27 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
         float pv[8];
         uint32_t dnew = 0, rn0 = 0, rn1 = 0;
         float am = 0.0f, vm = 0.0f;
-        uint64_t key = q * QLMX_KI;
+        /* The hash keys of the lane's eight elements are kept as running sums: the element stride as a value the
+         * compiler cannot see through (left as the literal, every key is rebuilt as q * KI + k * KI with the
+         * second product moved into a register pair first: five instructions per key instead of one), and the
+         * three step offsets added once. The clamp bounds likewise live in registers of their own: v_med3_i32
+         * takes one scalar operand at most, and without this both were copied into registers per element. */
+        uint64_t ki = QLMX_KI;
+        asm volatile("" : "+s"(ki));
+        int dlo = -c.dmax, dhi = c.dmax, mlo = -127, mhi = 127;
+        asm volatile("" : "+v"(dlo), "+v"(dhi), "+v"(mlo), "+v"(mhi));
+        const uint64_t key0 = q * QLMX_KI;
+        uint64_t key = key0 + kt;
 #pragma unroll
         for(int k = 0; k < 8; k++){
             const uint32_t rword = k < 4 ? rw.x : rw.y;
             const int rold = (int)(signed char)(rword >> (8 * (k & 3)));
             const int dd = qx_nib(dw, k);
-            const int idl = qx_sround(-(c.L * uu[k] + c.dec * (float)dd), key + kt);
+            const int idl = qx_sround(-(c.L * uu[k] + c.dec * (float)dd), key);
             const int rr0 = rold + idl;
             const int cy = qx_carry(rr0);
             const int rr = rr0 - cy * 128;
-            const int dn = qx_med3i(dd + cy, -c.dmax, c.dmax);
+            const int dn = qx_med3i(dd + cy, dlo, dhi);
             if(HASP) pv[k] = c.sg * (float)dn;
             dnew = __builtin_amdgcn_alignbit((uint32_t)dn, dnew, 4);
             if(k < 4) rn0 = __builtin_amdgcn_alignbit((uint32_t)rr, rn0, 8); else rn1 = __builtin_amdgcn_alignbit((uint32_t)rr, rn1, 8);
@@ -233,7 +243,7 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
                 st_rail += (dn == c.dmax) | (dn == -c.dmax);
                 st_zero += (dn == 0);
             }
-            key += QLMX_KI;
+            key += ki;
         }
         *(uint32_t *)(a.d + (q >> 1)) = dnew;
         *(uint2 *)(a.r + q) = make_uint2(rn0, rn1);
@@ -253,7 +263,7 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
         /* one choice for the wavefront: the reciprocal form when all four groups allow it (the usual case) */
         const bool recip = __builtin_amdgcn_ballot_w64(!(dms.fast && (!ADAM || dvs.fast))) == 0;
         uint32_t mo0 = 0, mo1 = 0, vo0 = 0, vo1 = 0;
-        key = q * QLMX_KI;
+        uint64_t keym = key0 + ktm, keyv = key0 + ktv;
 #pragma unroll
         for(int k = 0; k < 8; k++){
             float qm, qv = 0.0f;
@@ -264,20 +274,20 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
                 qm = mn[k] / ms;
                 if(ADAM) qv = rv[k] / vs;
             }
-            const int mq = qx_med3i(qx_sround(qm, key + ktm), -127, 127);
+            const int mq = qx_med3i(qx_sround(qm, keym), mlo, mhi);
             if(k < 4) mo0 = __builtin_amdgcn_alignbit((uint32_t)mq, mo0, 8); else mo1 = __builtin_amdgcn_alignbit((uint32_t)mq, mo1, 8);
             if(ADAM){
                 /* floor + stochastic increment stay in floating point (whole numbers, exact); the conversion that
                  * packs the byte saturates to [0, 255], which is the clamp of qlm.cuh:274; a positive moment
                  * never rounds to the code 0 (qlm.cuh:275) */
                 const float fl = floorf(qv);
-                const uint32_t h = qx_hash(key + ktv);
+                const uint32_t h = qx_hash(keyv);
                 const float ur = (float)(h >> 8) * (1.0f / 16777216.0f);
                 float vq = fl + (ur < (qv - fl) ? 1.0f : 0.0f);
                 vq = fmaxf(vq, rv[k] > 0.0f ? 1.0f : 0.0f);
                 if(k < 4) vo0 = __builtin_amdgcn_cvt_pk_u8_f32(vq, k & 3, vo0); else vo1 = __builtin_amdgcn_cvt_pk_u8_f32(vq, k & 3, vo1);
             }
-            key += QLMX_KI;
+            keym += ki; keyv += ki;
         }
         *(uint2 *)(a.m8 + q) = make_uint2(mo0, mo1);
         if(ADAM) *(uint2 *)(a.v8 + q) = make_uint2(vo0, vo1);

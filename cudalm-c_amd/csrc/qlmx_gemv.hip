@@ -1047,12 +1047,14 @@ static int df_reserve(DfSpace &ws, int which, size_t words, hipStream_t st){
 }
 
 /* Rows per task of list 1: 256 keeps the per-task fixed cost (staging, reduction, hand-over) small against
- * the streaming part; only when even that leaves most of the grid without a gate|up task (a single
- * token) are the slices halved. The number of problems is only known on the device; the host uses
- * the expected number of distinct experts hit by `npair` uniform picks out of E. */
+ * the streaming part; the slices are halved only while they leave fewer than 0.15 x the grid with a gate|up task
+ * (a single token: 128 rows, 192 tasks). More, shorter slices cost the down tasks a second round trip for their
+ * sums: measured at E=32 D=768 F=2048 top-2, rows 256 / 128 / 64 give 16.3 / 15.6 / 18.2 us per layer for one
+ * token, 18.8 / 21.4 / 26.4 for four, 29.7 / 32.7 / 42.0 for sixteen. The number of problems is only known on the
+ * device; the host uses the expected number of distinct experts hit by `npair` uniform picks out of E. */
 static int df_rows(int Kdim, double tasks_per_slice, int grid){
     int R = DF_RMAX;
-    while(R > 64 && tasks_per_slice * ((Kdim + R - 1) / R) < 0.25 * grid) R >>= 1;
+    while(R > 64 && tasks_per_slice * ((Kdim + R - 1) / R) < 0.15 * grid) R >>= 1;
     while((Kdim + R - 1) / R > 32 && R < DF_RMAX) R <<= 1;
     return R;
 }

@@ -850,7 +850,7 @@ def cpu_decode(args, E=32, D=768, F=2048, topk=2, T=16, layers=2):
 # (64.1 MiB read + 5.1 MiB written). The figures are constants of the code state they were measured at; that
 # state is named in the JSON line so that a reader can tell a stale one.
 PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.373e9, "decode": 7.39e7}
-PROFILED_AT = "git e24a32b (adamw, train), ef06021 (decode)"
+PROFILED_AT = "git e24a32b (train), ef06021 (decode), 771b539 (adamw)"
 
 
 def main():

@@ -118,6 +118,27 @@ def test_decode_forward_vs_oracle_layer(q, orc, tol, T, E, D, F, K):
     assert torch.equal(out, out2)
 
 
+@pytest.mark.parametrize("T", [2, 3, 5, 6, 7, 9, 11, 13, 24, 32])
+def test_decode_token_counts_cover_leftover_groups(q, orc, tol, T):
+    """Token counts whose numbers of problems leave every remainder modulo the 8 XCDs (the groups left over after
+    a full round are cut into pieces over the XCDs), up to the 64 (pass, token) pairs a call may carry."""
+    import torch
+    E, D, F, K = 16, 256, 512, 2
+    d, s, P, n = encode_layer(orc, 70 + T, E, D, F)
+    x = orc.normal(T * D, 70 + T, 2)
+    rt = orc.normal(T * E, 70 + T, 3)
+    pr = np.zeros(T * E, f32); asn = np.zeros(K * T, np.int32); gate = np.zeros(K * T, f32)
+    orc.router_topk(rt, pr, asn, gate, T, E, K)
+    want = np.zeros(T * D, f32)
+    rc, ws = orc.moe_forward(x, P[:n], P[n:2 * n], P[2 * n:], asn, gate, want, T, D, F, E, K)
+    orc.moe_ws_free(ws)
+    assert rc == 0
+    out = torch.zeros(T * D, device="cuda")
+    q.decode_forward(dev(x), dev(asn), dev(gate), out, dev(d), dev(s), 128, 0, n, 2 * n, T, K, E, D, F)
+    torch.cuda.synchronize()
+    assert orc.relerr(out.cpu().numpy(), want) < tol
+
+
 def test_decode_all_tokens_one_expert(q, orc, tol):
     """Collision case: 16 tokens on the same two experts -> problems are cut into row pairs."""
     import torch

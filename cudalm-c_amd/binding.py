@@ -82,6 +82,7 @@ SIGNATURES = {
     "qlmx_moe_gemm_nt": (c_i, [c_vp, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_decode_forward": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "qlmx_moe_decode_forward_noalloc": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_u64, c_u64, c_u64, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "qlmx_decode_status": (c_i, []),
     "qlmx_test_force_wait_timeout": (c_i, [c_i]),
     "qlmx_nt_tile": (c_i, [c_i]),
     "qlmx_decode_math": (c_i, [c_i]),

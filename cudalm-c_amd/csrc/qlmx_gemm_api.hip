@@ -199,8 +199,9 @@ extern "C" int qlmx_moe_gemm_tn_pair_scatter(const signed char *d, const float *
 /* mg_abt (the down projection's input gradient) + e_swigb (cudalm.cu:4340-4346) in one launch: problem i computes
  * d(act) = A . W^T [M, N] and, instead of storing it, applies k_swiglu_bwd to it: with o the element offset of
  * probs[i].C inside gp (probs[i].C points at the problem's rows of the forward's gate pre-activations),
- * dgp[o ..] and dup[o ..] (bf16) receive the gradients computed from gp[o ..], up[o ..] (fp32). Element for
- * element the operations of qlmx_swiglu_bwd on the stored product: bit-identical to the two separate calls. */
+ * dgp[o ..] and dup[o ..] (bf16) receive the gradients computed from gp[o ..], up[o ..] (fp32): the operations of
+ * qlmx_swiglu_bwd on the product, with the sigmoid from the transcendental unit instead of the polynomial
+ * (3e-7 relative apart), so a bf16 result can differ from the two separate calls by one unit in its last place. */
 extern "C" int qlmx_moe_gemm_tn_swiglu_bwd(const signed char *d, const float *s, int group,
                                            const qlmx_gemm_prob *probs, int nprob, int K, int N,
                                            const float *gp, const float *up, void *dgp, void *dup, void *stream){

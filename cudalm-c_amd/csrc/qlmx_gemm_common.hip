@@ -3,16 +3,21 @@
  * The tables of a launch (problems, and for scheduled launches the unit table) are put together in
  * ordinary host memory and then written, with one streaming copy by the CPU, into a slot of a ring that
  * lies in DEVICE memory the host can write directly (fine-grained device memory, mapped through the PCIe
- * BAR). The posted writes reach the device before the launch's doorbell does, no copy kernel or DMA
- * stands in front of the launch (a 4 us copy kernel and its dependency cost 20 us of a 1 ms training
+ * BAR; only where the device reports a large BAR, i.e. all of its memory host-visible). The writes are
+ * write-combined, so a store fence follows them: the launch's doorbell is a later store of the same
+ * thread and must not overtake them. No copy kernel or DMA stands in front of the launch (a 4 us copy kernel and its dependency cost 20 us of a 1 ms training
  * step), and the kernels' dependent table reads at the start of every tile cost a trip to local memory
  * or L2 (170-420 cycles measured) instead of one across PCIe to pinned host memory (1300). Where such
  * memory cannot be had the ring falls back to pinned host memory. A slot is handed out again only after
  * the host has waited for an event recorded behind the kernel that last read it. Because the slots are
  * rewritten, launches that use them must not be captured into a HIP graph. */
 #include "qlmx_gemm.h"
+#include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 #include <algorithm>
+#include <atomic>
+#include <immintrin.h>
 
 /* Reuse guard of a ring: an event behind every launch costs about 6 us of idle GPU between that kernel
  * and the next (the record makes the end of the kernel visible to the host), so the slots are guarded
@@ -72,10 +77,25 @@ static int guard_launched(RingGuard &g, int slot, hipStream_t stream){
 /* Table memory the host writes and the kernels read: device memory mapped into the host's address space,
  * else pinned host memory. Never read back by the host (reads across the BAR are slow) and never freed. */
 static int table_alloc(void **p, size_t bytes, const char *what){
-    if(hipExtMallocWithFlags(p, bytes, hipDeviceMallocFinegrained) == hipSuccess && *p) return QLMX_OK;
+    int dev = 0, large_bar = 0;
+    if(hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&large_bar, hipDeviceAttributeIsLargeBar, dev) != hipSuccess) large_bar = 0;
+    (void)hipGetLastError();
+    const bool say = getenv("QLMX_VERBOSE") != nullptr;
+    if(large_bar && hipExtMallocWithFlags(p, bytes, hipDeviceMallocFinegrained) == hipSuccess && *p){
+        if(say) fprintf(stderr, "[qlmx] %s: %zu bytes of host-writable device memory\n", what, bytes);
+        return QLMX_OK;
+    }
     (void)hipGetLastError();
     QLMX_HIP(hipHostMalloc(p, bytes, hipHostMallocDefault), what);
+    if(say) fprintf(stderr, "[qlmx] %s: %zu bytes of pinned host memory (large BAR: %d)\n", what, bytes, large_bar);
     return QLMX_OK;
+}
+/* Everything written into a table so far is on its way to the device before anything the thread stores next
+ * (the queue's doorbell): sfence drains the write-combining buffers, the thread fence keeps the compiler
+ * from moving the copies past it. */
+static inline void table_publish(void){
+    std::atomic_thread_fence(std::memory_order_seq_cst);
+    _mm_sfence();
 }
 
 #define RING_SLOTS 64
@@ -148,6 +168,7 @@ static int upload_problems(const qlmx_gemm_prob *probs, const qlmx_gemm_prob *se
     (void)stream;
     DevProb *dst = g_ring_h + (size_t)slot * QLMX_MAX_PROBLEMS;
     memcpy(dst, stage, (size_t)n * sizeof(DevProb));
+    table_publish();
     out->dev = dst; out->ntiles = (int)tiles; out->nprob = n;
     *slot_out = slot;
     return QLMX_OK;
@@ -218,6 +239,7 @@ void qlmx_unit_commit(const UnitUpload *u, int nprob, int nunits){
     const size_t uoff = unit_offset(nprob);
     memcpy((void *)u->dprob, u->hprob, (size_t)nprob * sizeof(DevProb));
     memcpy((void *)u->dunit, u->hunit, (size_t)nunits * sizeof(DevUnit));
+    table_publish();
     (void)uoff;
 }
 int qlmx_unit_done(int slot, hipStream_t stream){ return guard_launched(g_unit_guard, slot, stream); }

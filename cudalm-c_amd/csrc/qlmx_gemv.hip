@@ -849,7 +849,7 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
     auto scales_ahead = [&](const DfT &t, float (&sc)[DF_NG]){
         const float *sp = scales_of(t) + (size_t)min(tid, t.rows - 1) * (t.list == 1 ? gprF : gprD);
 #pragma unroll
-        for(int gg = 0; gg < DF_NG; gg++) sc[gg] = sp[gg < ng ? gg : 0];
+        for(int gg = 0; gg < DF_NG; gg++) sc[gg] = sp[(gg < ng && t.chunk * DF_CW + gg * a.group < t.N) ? gg : 0];   /* a group past the row's end re-reads the first */
     };
     float csc[DF_NG];
     DF_STAMP(20);
@@ -1161,6 +1161,22 @@ static int df_forward(bool fixed, const char *who, const float *x, const int *as
     if(df_math_fp16()) hipLaunchKernelGGL(k_decode_fused<true>, dim3(grid), dim3(DF_THREADS), 0, st, a);
     else               hipLaunchKernelGGL(k_decode_fused<false>, dim3(grid), dim3(DF_THREADS), 0, st, a);
     QLMX_LAUNCH_CHECK("decode launch");
+    return QLMX_OK;
+}
+
+/* Host-only query for callers whose decode launches do not pass through df_forward (HIP-graph replays): reads
+ * and clears the pinned word a launch sets when one of its bounded waits gave up. No GPU call. */
+extern "C" int qlmx_decode_status(void){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    int device = -1;
+    QLMX_HIP(hipGetDevice(&device), "decode device");
+    QLMX_REQUIRE(device >= 0 && device < DF_MAX_DEVICES && g_dfdev[device].ready, "qlmx_decode_status: qlmx_init has not run for device %d", device);
+    DfDevice &dv = g_dfdev[device];
+    if(*(volatile unsigned *)dv.status){
+        *dv.status = 0;
+        qlmx_set_error("qlmx_decode_status: a decode launch gave up waiting for a task of its own grid; its output is invalid");
+        return QLMX_E_HIP;
+    }
     return QLMX_OK;
 }
 

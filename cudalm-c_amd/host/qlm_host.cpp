@@ -495,10 +495,28 @@ static void mg_run_pairs(void){
 /* The problems of a flush do not depend on each other except queue 1 on queue 0 (it accumulates into what queue 0
  * writes). The weight gradients (queue 2) of a flush that also holds input gradients run on the library's side
  * stream beside them: neither fills the device to the end of its last round of tiles. */
+static bool q2_reads_what_the_flush_writes(void){
+    /* the reference issues queue 0, 1, 2 in order on one stream (cudalm.cu:3243), so there a weight-gradient
+     * problem may read an output of the same flush; side by side that would race, so such a flush runs in order */
+    const size_t asz = g_mg_act == QLMX_ACT_BF16 ? 2 : 4;
+    auto overlaps = [](const void *p, size_t n, const void *q, size_t m){
+        const uintptr_t a = (uintptr_t)p, b = (uintptr_t)q;
+        return p && q && a < b + m && b < a + n;
+    };
+    for(const MgItem &w : g_q[2])
+        for(int qn = 0; qn < 2; qn++)
+            for(const MgItem &o : g_q[qn]){
+                const size_t out = (size_t)o.p.M * (size_t)o.N * 4;
+                if(overlaps(w.p.A, (size_t)w.p.M * (size_t)w.K * asz, o.p.C, out) || overlaps(w.p.B, (size_t)w.p.M * (size_t)w.N * asz, o.p.C, out))
+                    return true;
+            }
+    return false;
+}
 void mg_flush(void){
     mg_run_dual();
     void *side = NULL;
-    const bool beside = !g_q[2].empty() && (!g_q[0].empty() || !g_q[1].empty()) && qlmx_side_fork(NULL, &side) == QLMX_OK;
+    const bool beside = !g_q[2].empty() && (!g_q[0].empty() || !g_q[1].empty()) && !q2_reads_what_the_flush_writes()
+                     && qlmx_side_fork(NULL, &side) == QLMX_OK;
     if(beside) mg_run(g_q[2], side);
     mg_run_pairs(); mg_run(g_q[0]); mg_run(g_q[1]);
     if(beside){ if(qlmx_side_join(NULL) != QLMX_OK){ fprintf(stderr, "mg_flush: %s\n", qlmx_last_error()); exit(1); } }

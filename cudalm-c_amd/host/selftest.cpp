@@ -34,9 +34,15 @@ static std::vector<unsigned char> slurp(const char *path){
 /* qlm_selftest optq IN OUT PREFIX GAP N0 [N1 ...]: a Qlm of that layout without weights, qlm_load(IN) into its
  * device state, qlm_save(OUT) from it. The caller compares the two files.
  * qlm_selftest sref PFILE OUT PREFIX GAP N0 [N1 ...]: qlm_gpu_init from the fp32 parameters in PFILE; OUT gets
- * the frozen reference scale of every span followed by all group scales (raw fp32). */
+ * the frozen reference scale of every span followed by all group scales (raw fp32).
+ * qlm_selftest update PFILE OUT PREFIX GAP N0 [N1 ...]: qlm_gpu_init from PFILE, then QLM_TEST_STEPS calls of
+ * qlm_gpu_update (t = 1, 2, ...; lr 3e-4, betas 0.9 / 0.95, weight decay 0.1, bias corrections 1 - beta^t as
+ * cudalm.cu:6454 forms them; the gradient of step t is the t-th block of np floats in QLM_TEST_GRADS; when
+ * QLM_TEST_CLIP is set the step takes its clip multiplier from a device scalar holding that value). The servo
+ * period, the optimizer and the LR mode come from the environment as in the reference. OUT gets, raw and in this
+ * order: d, r, m8, v8 (Adam only), s, m8s, v8s (Adam only), sref per span, the fp32 view P. */
 static int tool(int argc, char **argv){
-    if(argc < 7){ fprintf(stderr, "usage: %s optq|sref IN OUT PREFIX GAP N0 [N1 ...]\n", argv[0]); return 2; }
+    if(argc < 7){ fprintf(stderr, "usage: %s optq|sref|update IN OUT PREFIX GAP N0 [N1 ...]\n", argv[0]); return 2; }
     size_t np = 0;
     std::vector<QlmSpanDesc> sp = layout(atoi(argv[4]), atoi(argv[5]), argc - 6, argv + 6, &np);
     Qlm q;
@@ -65,6 +71,47 @@ static int tool(int argc, char **argv){
         if(!f || fwrite(out.data(), 4, out.size(), f) != out.size()){ fprintf(stderr, "sref: cannot write %s\n", argv[3]); return 1; }
         fclose(f);
         printf("sref: %d spans %llu groups, %d float gaps holding %llu parameters\n", q.nspan, q.ngrp, q.nfs, q.nfloat);
+        return 0;
+    }
+    if(!strcmp(argv[1], "update")){
+        std::vector<unsigned char> raw = slurp(argv[2]);
+        if(raw.size() != np * 4){ fprintf(stderr, "update: %s holds %zu bytes, the layout needs %zu\n", argv[2], raw.size(), np * 4); return 1; }
+        const int steps = atoi(getenv("QLM_TEST_STEPS") ? getenv("QLM_TEST_STEPS") : "4");
+        std::vector<unsigned char> graw = slurp(getenv("QLM_TEST_GRADS") ? getenv("QLM_TEST_GRADS") : "");
+        if(graw.size() != np * 4 * (size_t)steps){ fprintf(stderr, "update: QLM_TEST_GRADS must hold %d x %zu floats\n", steps, np); return 1; }
+        float *Pd = (float *)dmalloc(np * 4), *Gd = (float *)dmalloc(np * 4), *gsd = NULL;
+        qlmx_memcpy_h2d(Pd, raw.data(), np * 4);
+        if(getenv("QLM_TEST_CLIP")){
+            const float clip = (float)atof(getenv("QLM_TEST_CLIP"));
+            gsd = (float *)dmalloc(8); qlmx_memcpy_h2d(gsd, &clip, 4);
+        }
+        qlm_gpu_init(&q, sp.data(), (int)sp.size(), Pd, np);
+        const float lr = 3e-4f, b1 = 0.9f, b2 = 0.95f, wd = 0.1f;
+        int servo_passes = 0;
+        for(int t = 1; t <= steps; t++){
+            qlmx_memcpy_h2d(Gd, graw.data() + (size_t)(t - 1) * np * 4, np * 4);
+            qlm_gpu_update(&q, Pd, Gd, lr, b1, b2, wd, 1.0f - powf(b1, (float)t), 1.0f - powf(b2, (float)t), t, gsd);
+            servo_passes += q.servo_every > 0 && t % q.servo_every == 0;
+        }
+        /* the reference renders P after a servo pass only through the next step; the last step's P is what it left */
+        qlmx_sync(NULL);
+        FILE *f = fopen(argv[3], "wb");
+        if(!f){ fprintf(stderr, "update: cannot write %s\n", argv[3]); return 1; }
+        auto dump = [&](const void *dev, size_t bytes){
+            std::vector<unsigned char> h(bytes);
+            qlmx_memcpy_d2h(h.data(), dev, bytes);
+            return fwrite(h.data(), 1, bytes, f) == bytes;
+        };
+        bool okw = dump(q.d, (size_t)qlmx_qd_bytes(q.nq, q.packed)) && dump(q.r, q.nq) && dump(q.m8, q.nq);
+        if(q.adam) okw = okw && dump(q.v8, q.nq);
+        okw = okw && dump(q.s, q.ngrp * 4) && dump(q.m8s, q.ngrp * 4);
+        if(q.adam) okw = okw && dump(q.v8s, q.ngrp * 4);
+        for(int i = 0; i < q.nspan; i++) okw = okw && fwrite(&q.spanH[i].sref, 4, 1, f) == 1;
+        okw = okw && dump(Pd, np * 4);
+        fclose(f);
+        if(!okw){ fprintf(stderr, "update: short write to %s\n", argv[3]); return 1; }
+        printf("update: %d steps, %d servo passes, adam %d lrmode %d group %d dmax %d, %llu weights %llu groups\n",
+               steps, servo_passes, q.adam, q.lrmode, q.group, q.dmax, q.nq, q.ngrp);
         return 0;
     }
     fprintf(stderr, "unknown mode %s\n", argv[1]); return 2;
@@ -189,6 +236,25 @@ int main(int argc, char **argv){
         Yref[(size_t)m * F + f] = (float)acc; }
     double num = 0, den = 0; for(size_t i = 0; i < Y.size(); i++){ double dlt = (double)Y[i] - Yref[i]; num += dlt * dlt; den += (double)Yref[i] * Yref[i]; }
     check("moe expert fwd (mg_ab) rel-err", sqrt(num / den), 1e-3);
+
+    /* (d2) a weight-gradient problem that reads an output of the SAME flush (the reference runs its queues in
+     * order on one stream, cudalm.cu:3243, so this is legal there): Gw[D,F] += X^T . Y with Y written by the queue-0
+     * problem above it. The flush must notice the dependency and not run the two side by side. */
+    {
+        const int e = 2, ne = off[e + 1] - off[e];
+        std::vector<float> Gw((size_t)D * F, 0.f), Gref((size_t)D * F, 0.f);
+        float *Gwd = (float *)dmalloc(Gw.size() * 4);
+        qlmx_memset(Gwd, 0, Gw.size() * 4, NULL); qlmx_memset(Yd, 0, Y.size() * 4, NULL);
+        mg_ab(Xd + (size_t)off[e] * D, Pd + 16 + (size_t)e * D * F, Yd + (size_t)off[e] * F, ne, D, F);
+        mg_atb(Xd + (size_t)off[e] * D, Yd + (size_t)off[e] * F, Gwd, ne, D, F);
+        mg_flush(); qlmx_sync(NULL);
+        qlmx_memcpy_d2h(Gw.data(), Gwd, Gw.size() * 4);
+        double n2 = 0, d2 = 0;
+        for(int k = 0; k < D; k++) for(int f = 0; f < F; f++){
+            double acc = 0; for(int m = off[e]; m < off[e + 1]; m++) acc += (double)X[(size_t)m * D + k] * Yref[(size_t)m * F + f];
+            const double dlt = (double)Gw[(size_t)k * F + f] - acc; n2 += dlt * dlt; d2 += acc * acc; }
+        check("wgrad reading the flush's own output", sqrt(n2 / d2), 1e-3);
+    }
 
     /* (e) input gradient of w1 and w3 through the queue as the reference issues it (beta 0, then beta 1
      * on the same output), bf16 activations on the matrix cores: the flush runs each pair as one launch */

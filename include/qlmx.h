@@ -5,7 +5,13 @@
  * CPU build by cpu_rt.h / cpu_kern.h. Every entry point below replaces one of those call sites and
  * cites it (paths relative to the reference tree). All device buffers are caller-owned; `stream`
  * is a hipStream_t passed as void* (NULL = the default stream, which is what the reference uses).
- * Launches are asynchronous and ordered by the stream. Every function returns 0 on success and a
+ * Launches are asynchronous and ordered by the stream.
+ * ONE HOST THREAD, ONE STREAM AT A TIME (as the reference: one thread, the default stream, cudalm.cu:6628): the
+ * library keeps process-wide state -- the table rings of the grouped GEMMs and their staging copies, the chain flags
+ * of split contractions, the partial sums of qlmx_sqsum, the decode workspace -- so calls must come from one host
+ * thread, and calls whose kernels could overlap on different streams are not supported, except the documented
+ * pairing of qlmx_side_fork / qlmx_side_join.
+ * Every function returns 0 on success and a
  * negative QLMX_E_* code on failure; qlmx_last_error() holds the message of the calling thread's
  * last failure. The reference's print-and-exit(1) behaviour (ck/ckb, cudalm.cu:147-152) is kept by
  * the C++ mirror in cudalm-c_amd/host/, not here.
@@ -193,7 +199,8 @@ int qlmx_moe_gemm_tn_pair(const signed char *d, const float *s, int group,
  * ap to up[i].B (bf16 [M, N], the down GEMM's input). up[i] must repeat M; its A and beta are ignored.
  * On bf16 activations with QLMX_MATH_MFMA (N % 64 == 0, K % 32 == 0, group a power of two >= 64, at most
  * QLMX_MAX_PROBLEMS / 2 problems) an output tile holds 64 columns of both matrices and the SwiGLU is applied
- * to the accumulators; every other combination runs the two GEMM launches and a SwiGLU launch per problem. */
+ * to the accumulators (gp and up bit-identical to the two GEMM calls; ap computed with the polynomial sigmoid of
+ * qlmx_swiglu on QLMX_MATH_MFMA); every other combination runs the two GEMM launches and a SwiGLU launch per problem. */
 int qlmx_moe_gemm_nn_swiglu(const signed char *d, const float *s, int group,
                             const qlmx_gemm_prob *gate_host, const qlmx_gemm_prob *up_host, int nprob,
                             int K, int N, int act_dtype, int math, void *stream);
@@ -216,8 +223,12 @@ int qlmx_moe_gemm_nn_scatter(const signed char *d, const float *s, int group,
 int qlmx_moe_gemm_tn_pair_scatter(const signed char *d, const float *s, int group,
                                   const qlmx_gemm_prob *first_host, const qlmx_gemm_prob *second_host, int nprob, int K, int N,
                                   float *dst, void *stream);
-/* The SwiGLU and its gradient folded into the GEMMs next to them (fp16 forward kernel, bf16 input-gradient kernel;
- * element for element the operations of qlmx_swiglu / qlmx_swiglu_bwd, so results equal the separate calls bit for bit):
+/* The SwiGLU and its gradient folded into the GEMMs next to them (fp16 forward kernel, bf16 input-gradient kernel).
+ * The fp32 gate and up outputs equal the separate GEMM calls bit for bit. The epilogues take the sigmoid from the
+ * transcendental unit (v_exp_f32, v_rcp_f32) where qlmx_swiglu / qlmx_swiglu_bwd use the CPU build's polynomial
+ * (cpu_kern.h:376-394): the two agree to 3e-7 relative, so the bf16 outputs (activation, dgp, dup) equal the
+ * separate calls except where that difference crosses a bf16 rounding boundary -- one bf16 unit in the last place on
+ * fewer than 1 element in 10,000 (the bound the tests hold):
  *   qlmx_moe_gemm_nn_swiglu with QLMX_MATH_MFMA_F16: as documented above on the fp16 matrix core; gate[i].C and
  *     up[i].C may then both be NULL, and only the bf16 SwiGLU output up[i].B is written (a forward pass that does
  *     not keep gp / up for the backward: cudalm.cu:4211-4215 with the stash off).
@@ -261,12 +272,19 @@ int qlmx_moe_gemm_nt(const qlmx_gemm_prob *probs_host, int nprob, int K, int N,
  * orders the hand-over between workgroups lives in device memory and moves on by itself, so a call
  * may be recorded into a HIP graph and replayed (once the workspace has its size: a call that would
  * have to grow it during a capture fails with QLMX_E_ARG); a replay does not pass through the host,
- * so a wait that gave up is reported by the next direct call.
+ * so a wait that gave up is reported by the next direct call or by qlmx_decode_status(), which a loop of
+ * replays should ask after each synchronised replay. The launch is a grid of co-resident workgroups that wait for
+ * each other: it assumes that no other kernel occupies the device while it runs (with the CUs partly taken, late
+ * workgroups make the others wait, and past the bound -- of the order of 0.1 s -- the launch gives up).
  * ===================================================================================== */
 int qlmx_moe_decode_forward(const float *x, const int *assign, const float *gate, float *out,
                             const signed char *d, const float *s, int group,
                             unsigned long long w1q, unsigned long long w3q, unsigned long long w2q,
                             int T, int K, int E, int D, int F, void *stream);
+
+/* Host-only, no GPU call: QLMX_OK, or QLMX_E_HIP (once) when a decode launch on the current device has given up a
+ * bounded wait since the last report -- its `out` is invalid. No counterpart in the reference. */
+int qlmx_decode_status(void);
 
 /* qlmx_moe_decode_forward for callers that cannot allocate (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same arguments,

@@ -207,3 +207,70 @@ def test_train_size_mfma_vs_fp32_kernels_and_properties(q, orc, E, D, F, rows):
         want = np.zeros(D * F, f32)
         orc.gemm_nt(A, B, want, m, D, F)
         assert orc.relerr(G1[e * D * F:(e + 1) * D * F].cpu().numpy(), want) < 1e-3, (e, m)
+
+
+@pytest.mark.parametrize("opt,lrmode,clip", [("adam", "rel", None), ("qlion", "rel", None), ("adam", "abs", 0.37)])
+def test_host_mirror_update_driver_equals_the_oracle(orc, tmp_path, opt, lrmode, clip):
+    """qlm_gpu_init -> five qlm_gpu_update calls through libqlmx_host (cudalm.cu:6082-6103) with QLM_SERVO=2, so the
+    servo runs after steps 2 and 4 and the steps behind it work on rescaled groups; d, r, s, m8, v8, m8s, v8s, the
+    frozen reference scales and the fp32 view P byte for byte against the oracle's encode / step / servo called in
+    the reference's order. QLM_FSTAR=0.02 puts groups with one railed digit under the lower threshold (they shrink)
+    and groups with four or more over the upper one (they grow; some groups are built with six weights at the
+    group maximum), so every branch of the servo is taken. The last span ends in a short group."""
+    group, dmax, steps, fstar = 128, 7, 5, 0.02
+    sizes = [128 * 40, 128 * 24, 128 * 9 + 56]
+    prefix, gap = 16, 8
+    tab, nq, ng = make_spans(sizes, group, pofs=[prefix, prefix + sizes[0] + gap, prefix + sizes[0] + sizes[1] + 2 * gap])
+    np_ = prefix + sum(sizes) + 2 * gap + 2
+    P = orc.normal(np_, 5, 1, 0.02)
+    for si in range(3):                       # every third group: six weights at +- the group's largest magnitude
+        pof = int(tab["pof"][si])
+        for g in range(0, int(tab["ngrp"][si]) - 1, 3):
+            seg = P[pof + g * group: pof + (g + 1) * group]
+            seg[5:11] = np.abs(seg).max() * np.array([1, -1, 1, 1, -1, 1], f32)
+    G = np.concatenate([orc.normal(np_, 5, 10 + t, 2e-2) for t in range(steps)])
+    src, gsrc, dst = str(tmp_path / "P.f32"), str(tmp_path / "G.f32"), str(tmp_path / "state.bin")
+    P.tofile(src); G.tofile(gsrc)
+    env = dict(os.environ, QLM_SERVO="2", QLM_FSTAR=str(fstar), QLM_LRMODE=lrmode, QLM_TEST_STEPS=str(steps), QLM_TEST_GRADS=gsrc)
+    if opt == "qlion":
+        env["QLM_OPT"] = "qlion"
+    if clip is not None:
+        env["QLM_TEST_CLIP"] = repr(clip)
+    p = subprocess.run([os.path.join(PKG_DIR, "qlm_selftest"), "update", src, dst, str(prefix), str(gap)] + [str(n) for n in sizes],
+                       env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert p.returncode == 0, p.stdout
+    adam = opt != "qlion"
+    assert "update: %d steps, 2 servo passes, adam %d lrmode %d" % (steps, adam, lrmode == "abs") in p.stdout, p.stdout
+
+    hP = P.copy()
+    hd = np.zeros((nq + 1) // 2, np.int8); hr = np.zeros(nq, np.int8); hs = np.zeros(ng, f32)
+    hm8 = np.zeros(nq, np.int8); hv8 = np.zeros(nq, np.uint8); hm8s = np.zeros(ng, f32); hv8s = np.zeros(ng, f32)
+    orc.encode(hP, hd, hr, hs, tab, group, dmax, 1, ng)
+    orc.span_sref(tab, hs)
+    orc.render(hP, hd, hs, tab, group, 1, 0, ng)
+    b1, b2 = f32(0.9), f32(0.95)
+    import ctypes
+    powf = ctypes.CDLL("libm.so.6").powf
+    powf.restype = ctypes.c_float; powf.argtypes = [ctypes.c_float, ctypes.c_float]
+    f_hi, f_lo = float(f32(fstar) * f32(1.5)), float(f32(fstar) * f32(0.5))
+    gsp = None if clip is None else np.array([clip, 0], f32)
+    rescaled = 0
+    for t in range(1, steps + 1):
+        bc1 = f32(1) - f32(powf(b1, f32(t))); bc2 = f32(1) - f32(powf(b2, f32(t)))      # the C library's powf, as the driver's caller
+        orc.step(hP, G[(t - 1) * np_: t * np_], hd, hr, hs, hm8, hm8s, hv8, hv8s, tab, group, dmax, 3e-4, 0.9, 0.95, 0.1, 1.0, gsp,
+                 float(f32(1) / bc1), float(f32(1) / np.sqrt(bc2)), int(lrmode == "abs"), t, int(adam), None, 1, 0, ng)
+        if t % 2 == 0:
+            before = hs.copy()
+            orc.servo(hd, hr, hs, tab, group, dmax, f_hi, f_lo, 1, ng)
+            grew, shrank = int((hs > before).sum()), int((hs < before).sum())
+            assert grew > 0 and shrank > 0 and grew + shrank < ng, (t, grew, shrank, ng)
+            rescaled += grew + shrank
+    got = np.fromfile(dst, dtype=np.uint8)
+    want = [hd, hr, hm8] + ([hv8] if adam else []) + [hs, hm8s] + ([hv8s] if adam else []) + [tab["sref"].astype(f32), hP]
+    names = ["d", "r", "m8"] + (["v8"] if adam else []) + ["s", "m8s"] + (["v8s"] if adam else []) + ["sref", "P"]
+    at = 0
+    for name, w in zip(names, want):
+        wb = np.ascontiguousarray(w).view(np.uint8).ravel()
+        assert np.array_equal(got[at: at + wb.size], wb), "%s differs after %d steps (%d groups rescaled on the way)" % (name, steps, rescaled)
+        at += wb.size
+    assert at == got.size

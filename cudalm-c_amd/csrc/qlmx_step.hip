@@ -29,6 +29,7 @@ struct StepParams {
     unsigned long long t; unsigned long long *stat;
     int packed, gi_base, ng, v4;
     int vec_ok;      /* base pointers are aligned for the 128/64/32-bit accesses of the fast path */
+    int mid_ok;      /* 0 <= inv_sqrt_bc2 <= 2^10: the mid-range forms of the fast path may be tried */
     /* touched-group form (k_ng_q4_step, cudalm.cu:4472): team w steps group touched[w] of one span
      * that starts at element 0, and its gradient is the compact row Gc[w*group ..] */
     const int *touched; qlmx_span one;
@@ -70,6 +71,52 @@ __device__ __forceinline__ float qx_sqrt_above_2m96(float x){
     float r = rdn <= 0.0f ? dn : s;
     r = rup > 0.0f ? up : r;
     return r;
+}
+/* ---- the usual case of the 8-weights-per-lane path ----
+ * The kernel is bound by the number of vector instructions it issues (single-instruction loops on the device: every
+ * vector instruction takes a SIMD's issue slot for four cycles, rcp and sqrt for eight; the two-cycle rate of plain
+ * fp32 / integer adds, multiplies and logic only appears when all wavefronts of a SIMD run nothing else, never in a
+ * mix). The forms below therefore drop instructions that do nothing for operands in the middle of the range: the
+ * correctly rounded division without its scaling and special-case steps, the row maxima as one DPP instruction per
+ * step. They are checked against `/` on the device over billions of operand pairs; values outside the guarded
+ * ranges take the general code. */
+/* correctly rounded n / d for d in [2^-40, 2^40] and n = 0 or |n| in [2^-40, 2^40]: the compiler's division
+ * sequence without v_div_scale (which leaves such operands alone), with a plain FMA for v_div_fmas and without
+ * v_div_fixup */
+__device__ __forceinline__ float qx_div_mid(float n, float d){
+    const float y0 = __builtin_amdgcn_rcpf(d);
+    const float e = __builtin_fmaf(-d, y0, 1.0f);
+    const float y1 = __builtin_fmaf(e, y0, y0);
+    const float q0 = n * y1;
+    const float r0 = __builtin_fmaf(-d, q0, n);
+    const float q1 = __builtin_fmaf(r0, y1, q0);
+    const float r1 = __builtin_fmaf(-d, q1, n);
+    return __builtin_fmaf(r1, y1, q1);
+}
+/* qx_hash of a key that already carries the hash's additive constant; returns u = top 24 bits * 2^-24 */
+__device__ __forceinline__ float qx_hash_unit(uint64_t x){
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ULL;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBULL;
+    const uint32_t h = (uint32_t)(x ^ (x >> 31));
+    return (float)(h >> 8) * (1.0f / 16777216.0f);
+}
+/* row maximum of non-negative floats, as unsigned integers (same order, no NaN quieting in between): one
+ * instruction per step; a DPP operand needs two idle cycles after the instruction that wrote its register */
+__device__ __forceinline__ float qx_row16_max_nonneg(float f){
+    uint32_t v = __float_as_uint(f);
+    asm("s_nop 1\n\tv_max_u32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf" : "+v"(v));
+    return __uint_as_float(v);
+}
+/* byte `B` of `word` = low byte of a - b, the other bytes kept (a sub-dword destination instead of a subtract and
+ * a funnel shift) */
+template<int B> __device__ __forceinline__ void qx_sub_to_byte(uint32_t &word, int a, int b){
+    if(B == 0) asm("v_sub_u32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(word) : "v"(a), "v"(b));
+    if(B == 1) asm("v_sub_u32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(word) : "v"(a), "v"(b));
+    if(B == 2) asm("v_sub_u32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(word) : "v"(a), "v"(b));
+    if(B == 3) asm("v_sub_u32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(word) : "v"(a), "v"(b));
 }
 __device__ __forceinline__ int qx_med3i(int v, int lo, int hi){            /* clamp in one instruction; lo <= hi */
     int r; asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi)); return r;
@@ -120,6 +167,119 @@ __device__ __forceinline__ ElemRes step_elem(const GroupCtx &c, float graw, int 
     return o;
 }
 
+/* One full, aligned group of 128 for a row of 16 lanes, Adam, no statistics, operands in the middle of the range.
+ * Nothing is stored before the guards have passed for the whole wavefront; when they fail the function returns
+ * false and the caller runs the general code on the same registers. Guards (each makes a short form exact, none
+ * changes a result): second moments >= 2^-96 with roots <= 2^25, |m * inv_bc1| in [2^-40, 2^40] (zero excluded, so
+ * that the quotient's residuals cannot underflow), the lane's largest |m| in [2^-32, 2^40], eps <= 2^20; the launch
+ * checks 0 <= inv_sqrt_bc2 <= 2^10 on the host (a.mid_ok). */
+template<bool HASP, bool V4>
+__device__ __forceinline__ bool step_row8_mid(const StepParams &a, const GroupCtx &c, int gi, int lane16, uint64_t q, uint64_t pofe,
+                                              const float (&gv)[8], uint32_t dw, uint2 rw, uint2 mw, uint2 vw,
+                                              uint64_t kt, uint64_t ktm, uint64_t ktv){
+    float mn[8], vv[8], rv[8], uu[8];
+    float vmin = 3.0e38f, amin = 3.0e38f, am = 0.0f, vm = 0.0f;
+#pragma unroll
+    for(int k = 0; k < 8; k++){
+        const uint32_t mword = k < 4 ? mw.x : mw.y, vword = k < 4 ? vw.x : vw.y;
+        const int sh = 8 * (k & 3);
+        const float gr = gv[k] * c.gs;
+        const float mv = (float)(int)(signed char)(mword >> sh) * c.ms_old;
+        float sv = (float)((vword >> sh) & 0xFFu) * c.vs_old; if(V4) sv = sv * sv;
+        mn[k] = c.b1 * mv + c.omb1 * gr;
+        vv[k] = c.b2 * (sv * sv) + c.omb2 * gr * gr;
+        vmin = fminf(vmin, vv[k]);
+        amin = fminf(amin, fabsf(mn[k])); am = fmaxf(am, fabsf(mn[k]));
+    }
+    if(__builtin_amdgcn_ballot_w64(!(vmin >= 0x1p-96f)) != 0) return false;        /* NaN compares false */
+#pragma unroll
+    for(int k = 0; k < 8; k++){
+        rv[k] = qx_sqrt_above_2m96(vv[k]);
+        const float u = qx_div_mid(mn[k] * c.inv_bc1, rv[k] * c.inv_sqrt_bc2 + c.veps);
+        uu[k] = __builtin_amdgcn_fmed3f(u, -8.0f, 8.0f);
+        vm = fmaxf(vm, rv[k]);                           /* the guard wants the plain root also when V4 */
+    }
+    {   /* operands outside these ranges made the loop above compute garbage, which is dropped */
+        const float nlo = amin * c.inv_bc1, nhi = am * c.inv_bc1;
+        const bool lane_ok = vm <= 0x1p25f && nlo >= 0x1p-40f && nhi <= 0x1p40f && am >= 0x1p-32f && am <= 0x1p40f && c.veps <= 0x1p20f;
+        if(__builtin_amdgcn_ballot_w64(!lane_ok) != 0) return false;
+    }
+    if(V4){
+        vm = 0.0f;
+#pragma unroll
+        for(int k = 0; k < 8; k++){ rv[k] = qx_sqrt_above_2m96(rv[k]); vm = fmaxf(vm, rv[k]); }   /* stored as the fourth root, in [2^-24, 2^13] */
+    }
+    /* ---- digits and residuals (qlm.cuh:230-242) ---- */
+    uint64_t ki = QLMX_KI;
+    asm volatile("" : "+s"(ki));
+    int dlo = -c.dmax, dhi = c.dmax;
+    asm volatile("" : "+v"(dlo), "+v"(dhi));
+    const uint64_t key0 = q * QLMX_KI + 0x9E3779B97F4A7C15ULL;       /* the hash's own additive constant rides along */
+    float pv[8];
+    uint32_t dnew = 0, rn0 = 0, rn1 = 0;
+    uint64_t key = key0 + kt;
+#pragma unroll
+    for(int k = 0; k < 8; k++){
+        const uint32_t rword = k < 4 ? rw.x : rw.y;
+        const int rold = (int)(signed char)(rword >> (8 * (k & 3)));
+        const int dd = qx_nib(dw, k);
+        const float v = -(c.L * uu[k] + c.dec * (float)dd);
+        const float fl = floorf(v);
+        const int rr0 = rold + (int)fl + (qx_hash_unit(key) < (v - fl) ? 1 : 0);
+        const int cyv = rr0 + 63 - (rr0 >> 31);
+        const int cy = cyv >> 7;                                       /* qx_carry(rr0) */
+        /* the new residual rr0 - 128 cy, of which only the low byte is kept: 128 cy and cyv agree from bit 7 up */
+        if(k == 0) qx_sub_to_byte<0>(rn0, rr0, cyv & 0x80); if(k == 1) qx_sub_to_byte<1>(rn0, rr0, cyv & 0x80);
+        if(k == 2) qx_sub_to_byte<2>(rn0, rr0, cyv & 0x80); if(k == 3) qx_sub_to_byte<3>(rn0, rr0, cyv & 0x80);
+        if(k == 4) qx_sub_to_byte<0>(rn1, rr0, cyv & 0x80); if(k == 5) qx_sub_to_byte<1>(rn1, rr0, cyv & 0x80);
+        if(k == 6) qx_sub_to_byte<2>(rn1, rr0, cyv & 0x80); if(k == 7) qx_sub_to_byte<3>(rn1, rr0, cyv & 0x80);
+        const int dn = qx_med3i(dd + cy, dlo, dhi);
+        if(HASP) pv[k] = c.sg * (float)dn;
+        dnew = __builtin_amdgcn_alignbit((uint32_t)dn, dnew, 4);
+        key += ki;
+    }
+    *(uint32_t *)(a.d + (q >> 1)) = dnew;
+    *(uint2 *)(a.r + q) = make_uint2(rn0, rn1);
+    if(HASP){
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        f4 p0 = {pv[0], pv[1], pv[2], pv[3]}, p1 = {pv[4], pv[5], pv[6], pv[7]};
+        __builtin_nontemporal_store(p0, (f4 *)(a.P + pofe));
+        __builtin_nontemporal_store(p1, (f4 *)(a.P + pofe + 4));
+    }
+    /* ---- fresh scales and the re-quantised moments (qlm.cuh:244-278); both maxima are positive here ---- */
+    am = qx_row16_max_nonneg(am); vm = qx_row16_max_nonneg(vm);
+    const float ms = qx_div_mid(am, 127.0f), vs = qx_div_mid(vm, 255.0f);
+    const float ym = qx_div_mid(1.0f, ms), yv = qx_div_mid(1.0f, vs);      /* ms, vs in [2^-40, 2^34]: qx_gdiv's reciprocal form holds */
+    if(lane16 == 0){ a.m8s[gi] = ms; a.v8s[gi] = vs; }
+    uint32_t mo0 = 0, mo1 = 0, vo0 = 0, vo1 = 0;
+    uint64_t keym = key0 + ktm, keyv = key0 + ktv;
+#pragma unroll
+    for(int k = 0; k < 8; k++){
+        const float t = mn[k] * ym;
+        /* clamped before the rounding instead of after it: above 127 both give 127, below -127 both give -127
+         * (floor -128 or lower, plus at most one), in between nothing is clamped */
+        const float qm = __builtin_amdgcn_fmed3f(fmaf(fmaf(-t, ms, mn[k]), ym, t), -127.0f, 127.0f);
+        const float w = rv[k] * yv, qv = fmaf(fmaf(-w, vs, rv[k]), yv, w);
+        {
+            const float fl = floorf(qm);
+            const int mq = (int)fl + (qx_hash_unit(keym) < (qm - fl) ? 1 : 0);
+            if(k < 4) mo0 = __builtin_amdgcn_alignbit((uint32_t)mq, mo0, 8); else mo1 = __builtin_amdgcn_alignbit((uint32_t)mq, mo1, 8);
+        }
+        {
+            /* floor + increment stay whole numbers in floating point; the packing conversion saturates to [0, 255]
+             * (the clamp of qlm.cuh:274); a positive moment never rounds to the code 0 (qlm.cuh:275), and every
+             * root is positive on this path */
+            const float fl = floorf(qv);
+            const float vq = fmaxf(fl + (qx_hash_unit(keyv) < (qv - fl) ? 1.0f : 0.0f), 1.0f);
+            if(k < 4) vo0 = __builtin_amdgcn_cvt_pk_u8_f32(vq, k & 3, vo0); else vo1 = __builtin_amdgcn_cvt_pk_u8_f32(vq, k & 3, vo1);
+        }
+        keym += ki; keyv += ki;
+    }
+    *(uint2 *)(a.m8 + q) = make_uint2(mo0, mo1);
+    *(uint2 *)(a.v8 + q) = make_uint2(vo0, vo1);
+    return true;
+}
+
 /* STAT: the four counters are kept; HASP: the fp32 view is written; V4: the second moment is stored as its
  * fourth root (a.v4). All are fixed per launch, so they are template parameters and the usual launch (none of
  * them) carries no trace of them: as a run-time flag, v4 made the compiler compute the second square root of
@@ -160,6 +320,16 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
     if(fast){
         const uint64_t e0 = (uint64_t)lane16 * 8;
         const uint64_t q = qi0 + e0;
+        if(ADAM && !STAT && a.mid_ok){
+            const float4 h0 = *(const float4 *)(a.G + gof + e0);
+            const float4 h1 = *(const float4 *)(a.G + gof + e0 + 4);
+            const float hv[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
+            if(step_row8_mid<HASP, V4>(a, c, gi, lane16, q, pof + e0, hv, *(const uint32_t *)(a.d + (q >> 1)), *(const uint2 *)(a.r + q),
+                                       *(const uint2 *)(a.m8 + q), *(const uint2 *)(a.v8 + q), kt, ktm, ktv)) return;
+            /* nothing was stored; the general code loads its operands again rather than keep them in registers
+             * across the attempt (the barrier keeps the compiler from merging the two sets of loads) */
+            asm volatile("" ::: "memory");
+        }
         const float4 g0 = *(const float4 *)(a.G + gof + e0);
         const float4 g1 = *(const float4 *)(a.G + gof + e0 + 4);
         const uint32_t dw = *(const uint32_t *)(a.d + (q >> 1));
@@ -401,6 +571,7 @@ extern "C" int qlmx_step(float *P, const float *G, signed char *d, signed char *
     a.inv_bc1 = inv_bc1; a.inv_sqrt_bc2 = inv_sqrt_bc2; a.lrmode = lrmode;
     a.t = t; a.stat = (unsigned long long *)stat; a.packed = packed; a.gi_base = gi_base; a.ng = ng; a.v4 = v4;
     a.touched = nullptr;
+    a.mid_ok = inv_sqrt_bc2 >= 0.0f && inv_sqrt_bc2 <= 1024.0f;
     a.vec_ok = (((uintptr_t)P | (uintptr_t)G) & 15) == 0 && (((uintptr_t)r | (uintptr_t)m8 | (uintptr_t)v8) & 7) == 0
                && ((uintptr_t)d & 3) == 0;
     const unsigned blocks = (unsigned)((ng + 15) / 16);
@@ -436,6 +607,7 @@ extern "C" int qlmx_step_touched(float *P, const float *Gc, signed char *d, sign
     a.vec_ok = (((uintptr_t)P | (uintptr_t)Gc) & 15) == 0 && (((uintptr_t)r | (uintptr_t)m8 | (uintptr_t)v8) & 7) == 0
                && ((uintptr_t)d & 3) == 0;
     a.touched = touched_gi;
+    a.mid_ok = inv_sqrt_bc2 >= 0.0f && inv_sqrt_bc2 <= 1024.0f;
     a.one.pof = 0; a.one.gof = 0; a.one.qi0 = 0; a.one.n = nt; a.one.gi0 = 0;
     a.one.ngrp = (int)((nt + (unsigned long long)group - 1) / (unsigned long long)group); a.one.sref = sref;
     const unsigned blocks = (unsigned)((ntouched + 15) / 16);
@@ -522,6 +694,29 @@ extern "C" int qlmx_gnorm(const float *part, int nside, int clip_side, float *gs
     QLMX_REQUIRE(part && gs && nside >= 0, "qlmx_gnorm: bad arguments");
     hipLaunchKernelGGL(k_qlmx_gnorm, dim3(1), dim3(1), 0, (hipStream_t)stream, part, nside, clip_side, gs);
     QLMX_LAUNCH_CHECK("qlmx_gnorm launch");
+    return QLMX_OK;
+}
+
+/* ---- test hook: the short division form against `/` on pseudo-random operand pairs inside its range ---- */
+__global__ void __launch_bounds__(256) k_qlmx_test_div(unsigned long long seed, unsigned long long count, unsigned long long *mismatches){
+    unsigned long long bad = 0;
+    for(unsigned long long i = (unsigned long long)blockIdx.x * 256 + threadIdx.x; i < count; i += (unsigned long long)gridDim.x * 256){
+        uint64_t r = seed + i * 0x9E3779B97F4A7C15ULL;
+        r = (r ^ (r >> 30)) * 0xBF58476D1CE4E5B9ULL; r = (r ^ (r >> 27)) * 0x94D049BB133111EBULL; r ^= r >> 31;
+        /* |n| and d with exponents 2^-40 .. 2^40 and random significands, n of either sign */
+        const uint32_t en = 87u + (uint32_t)((r >> 23) % 81u), ed = 87u + (uint32_t)((r >> 55) % 81u);
+        const float n = __uint_as_float(((uint32_t)r & 0x807FFFFFu) | (en << 23));
+        const float d = __uint_as_float(((uint32_t)(r >> 32) & 0x007FFFFFu) | (ed << 23));
+        bad += __float_as_uint(qx_div_mid(n, d)) != __float_as_uint(n / d);
+        bad += __float_as_uint(qx_div_mid(0.0f, d)) != 0u;
+    }
+    if(bad) atomicAdd(mismatches, bad);
+}
+extern "C" int qlmx_test_div_form(unsigned long long seed, unsigned long long count, unsigned long long *mismatches_dev, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(mismatches_dev, "qlmx_test_div_form: NULL counter");
+    hipLaunchKernelGGL(k_qlmx_test_div, dim3(4096), dim3(256), 0, (hipStream_t)stream, seed, count, mismatches_dev);
+    QLMX_LAUNCH_CHECK("division test launch");
     return QLMX_OK;
 }
 

@@ -380,6 +380,11 @@ int qlmx_decode_math(int fp16_inputs);
  * compares the two forms on the device for the `count` consecutive bit patterns starting at first_bits and adds
  * the number of differing results to *mismatches_dev (device memory, unsigned long long). */
 int qlmx_test_sqrt_form(unsigned first_bits, unsigned long long count, unsigned long long *mismatches_dev, void *stream);
+/* Test hook. For operands in the middle of the range (divisor in [2^-40, 2^40], dividend 0 or of a magnitude in that
+ * interval) qlmx_step divides with the compiler's correctly rounded sequence minus its scaling and special-case
+ * instructions, which do nothing there. This compares that form with `/` on the device for `count` pseudo-random
+ * operand pairs of that range (derived from `seed`) and adds the number of differing results to *mismatches_dev. */
+int qlmx_test_div_form(unsigned long long seed, unsigned long long count, unsigned long long *mismatches_dev, void *stream);
 
 /* =====================================================================================
  * q4n wire format (host only, no device needed): quantize_params / dequantize_params with qtype 3

@@ -285,6 +285,59 @@ def test_step_zero_and_tiny_second_moments_take_the_general_square_root(q, orc):
         assert beq(got, want), nm
 
 
+def test_step_short_division_equals_the_full_one(q):
+    """The step's mid-range division (no scaling, no special-case fix-up) gives the bits of `/` on 2^33 pseudo-random
+    operand pairs with magnitudes in [2^-40, 2^40], and an exact zero for a zero dividend."""
+    import torch
+    bad = torch.zeros(1, dtype=torch.int64, device="cuda")
+    q.call("qlmx_test_div_form", 12345, 1 << 33, bad, None)
+    torch.cuda.synchronize()
+    assert int(bad.item()) == 0
+
+
+@pytest.mark.parametrize("v4,render,inv_sqrt_bc2", [(0, False, 4.4721), (1, True, 4.4721), (0, True, 2000.0)])
+def test_step_operands_at_the_edges_of_the_mid_range_forms(q, orc, v4, render, inv_sqrt_bc2):
+    """Groups built to sit on either side of every guard of the step's mid-range forms (whole wavefronts of four groups
+    each, and single elements inside ordinary groups): first moments that are exactly zero, tiny (below 2^-40 after
+    the bias correction) and huge, gradients that put the second moment's root above 2^25, a stored second-moment
+    scale above 2^20, a group whose largest first moment is below 2^-32, and -- third case -- an inverse bias
+    correction outside the range the host admits. Two steps; every byte equals the oracle, with and without the
+    fp32 view and in the fourth-root form."""
+    import torch
+    group, dmax = 128, 7
+    tab, nq, ng = make_spans([128 * 96], group)
+    tab["sref"] = [0.0086]
+    hd = orc.digits(nq, 11, 20); hr = orc.int8(nq, 11, 21, -64, 64); hm8 = orc.int8(nq, 11, 22, -127, 127)
+    hv8 = orc.u8(nq, 11, 23, 1, 255)
+    hs = orc.uniform(ng, 11, 24, 0.5, 1.5) * f32(0.02 * 3 / 7)
+    hm8s = orc.uniform(ng, 11, 25, 0.5, 1.5) * f32(3e-3 / 127); hv8s = orc.uniform(ng, 11, 26, 0.5, 1.5) * f32(3e-3 / 255)
+    hG = orc.normal(nq, 11, 27, 1e-3)
+    g = lambda a, b: slice(128 * a, 128 * b)
+    hG[g(0, 4)] = 0.0; hm8[g(0, 4)] = 0                             # first moment exactly zero, second moment live
+    hG[g(8, 12)] *= f32(1e-12); hm8[g(8, 12)] = 0                   # |m| ~ 1e-16: below 2^-40
+    hG[g(16, 20)] *= f32(1e9)                                        # sqrt(v) ~ 2e5, m ~ 1e5: inside
+    hG[g(24, 28)] *= f32(1e13)                                       # sqrt(v) ~ 2e9 > 2^25, m ~ 1e9
+    hG[g(32, 36)] *= f32(1e17)                                       # m * inv_bc1 > 2^40
+    hv8s[40:44] = f32(3e6)                                           # eps = stored scale > 2^20
+    hG[g(48, 52)] *= f32(1e-8); hm8[g(48, 52)] = 0; hv8[g(48, 52)] = 200    # largest |m| of a lane below 2^-32
+    hG[128 * 60 + 7] = 0.0; hm8[128 * 60 + 7] = 0                    # single zero first moment in an ordinary group
+    hG[128 * 64 + 9] = f32(1e-15); hm8[128 * 64 + 9] = 0             # single tiny one
+    hG[128 * 68 + 3] = f32(5e7)                                      # single huge one
+    hm8[g(72, 76)] = 127; hG[g(72, 76)] = f32(2e-3)                  # every quotient of the requantisation at the rail
+    P = torch.zeros(nq, device="cuda") if render else None
+    hP = np.zeros(nq, f32) if render else None
+    d, r, m8, v8, s, m8s, v8s, G = (dev(x) for x in (hd, hr, hm8, hv8, hs, hm8s, hv8s, hG))
+    for t in (1, 2):
+        hp = (3e-4, 0.9, 0.95, 0.1, 1.0, None, 10.0, inv_sqrt_bc2, 0, t, 1, None, 1, 0, ng)
+        q.step(P, G, d, r, s, m8, m8s, v8, v8s, dev(tab), 1, group, dmax, *hp, v4)
+        orc.step(hP, hG, hd, hr, hs, hm8, hm8s, hv8, hv8s, tab, group, dmax, *hp, v4)
+    pairs = [(d, hd, "d"), (r, hr, "r"), (m8, hm8, "m8"), (v8, hv8, "v8"), (m8s, hm8s, "m8s"), (v8s, hv8s, "v8s")]
+    if render:
+        pairs.append((P, hP, "P"))
+    for got, want, nm in pairs:
+        assert beq(got, want), nm
+
+
 def test_argument_errors(q):
     import torch
     x = torch.zeros(256, device="cuda")

@@ -21,7 +21,7 @@ struct DevProb {
  * the given tile shape over an output of rows_of(p) x ncols, and returns the pointer the kernel reads
  * the table through and the total tile count. Slots are guarded by events, so a slot is never
  * rewritten while a kernel launched with it may still read it. */
-struct ProbUpload { const DevProb *dev; int ntiles; int nprob; };
+struct ProbUpload { const DevProb *dev; int ntiles; int nprob; int nfull; };
 int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K, int N,
                          int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot);
 /* Problems with a second half (same M, K, N). tn: the contraction continues over second[i].A and the
@@ -30,6 +30,14 @@ int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K
  * is followed by an entry holding the second half's fields that owns no tile. */
 int qlmx_upload_problem_pairs(const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int mode, int K, int N,
                               int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot);
+/* The same with every problem entered as two: its whole row tiles first (all problems, in the caller's order), then
+ * the ragged last row tiles of all problems, tallest first, so that a launch hands out its longest tiles first
+ * (nn and tn only: rows are independent there). `rb` says how many bytes a row of each pointer field takes (4 where
+ * the field is a list of row indices); out->nfull = tiles of the first part. The kernel maps workgroups to tiles
+ * with qx_lpt_tile and the grid is qx_lpt_grid(nfull, ntiles). `second` may be NULL. */
+struct RowBytes { size_t a, c, a2, b2, c2; };
+int qlmx_upload_problems_split(const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int mode, int K, int N,
+                               int tile_rows, int tile_cols, const RowBytes *rb, hipStream_t stream, ProbUpload *out, int *slot);
 int qlmx_upload_done(int slot, hipStream_t stream);
 
 /* Locate the problem owning flattened tile t: the last one whose tile0 <= t (tile0 ascending, empty
@@ -55,6 +63,18 @@ __device__ __forceinline__ int qx_xcd_tile(int b, int grid){
     const int per = grid >> 3;
     return (b & 7) * per + (b >> 3);
 }
+
+/* Tile of workgroup b for a table whose first nfull tiles are whole-height ones and whose remaining tiles are the
+ * problems' last row tiles, tallest first: XCD x takes the x-th contiguous eighth of the first part (tiles that share
+ * an expert's rows and weights meet in one L2), then every eighth tile of the second part, so that all XCDs run out
+ * of whole tiles and then of tall last tiles at about the same time. 0x7FFFFFFF = no tile. */
+__device__ __forceinline__ int qx_lpt_tile(int b, int nfull, int ntiles){
+    const int x = b & 7, k = b >> 3, per = (nfull + 7) >> 3;
+    if(k < per){ const int t = x * per + k; return t < nfull ? t : 0x7FFFFFFF; }
+    const int t = nfull + (k - per) * 8 + x;
+    return t < ntiles ? t : 0x7FFFFFFF;
+}
+static inline int qx_lpt_grid(int nfull, int ntiles){ return 8 * ((nfull + 7) / 8 + (ntiles - nfull + 7) / 8); }
 
 /* Weight gradients (tile cost = the expert's row count): every problem owns rp rows of g tiles; a
  * row shares the A-side slab (activations), a column the B-side slab (output gradients).

@@ -114,10 +114,11 @@ static int ring_init(void){
  * Such a problem is followed in the table by an entry that carries the second half's fields and owns
  * no tile (its tile0 is the next problem's), and has `chunk` set to 1. */
 static int upload_problems(const qlmx_gemm_prob *probs, const qlmx_gemm_prob *second, int nprob, int mode, int K, int N,
-                           int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot_out){
+                           int tile_rows, int tile_cols, const RowBytes *rb, hipStream_t stream, ProbUpload *out, int *slot_out){
     QLMX_REQUIRE(probs && nprob >= 0, "grouped gemm: NULL problem list");
-    if(nprob * (second ? 2 : 1) > QLMX_MAX_PROBLEMS){
-        qlmx_set_error("grouped gemm: %d problems exceed the limit of %d", nprob, QLMX_MAX_PROBLEMS / (second ? 2 : 1));
+    const int per = (second ? 2 : 1) * (rb ? 2 : 1);                 /* table entries a problem may take */
+    if(nprob * per > QLMX_MAX_PROBLEMS){
+        qlmx_set_error("grouped gemm: %d problems exceed the limit of %d", nprob, QLMX_MAX_PROBLEMS / per);
         return QLMX_E_LIMIT;
     }
     int rc = ring_init(); if(rc) return rc;
@@ -146,42 +147,75 @@ static int upload_problems(const qlmx_gemm_prob *probs, const qlmx_gemm_prob *se
         const int i = order[oi];
         const qlmx_gemm_prob &p = probs[i];
         QLMX_REQUIRE(p.M >= 0, "grouped gemm: problem %d has M=%d", i, p.M);
-        if(p.M == 0) continue;
         QLMX_REQUIRE(p.A && (p.C || (second && mode == GEMM_NN)), "grouped gemm: problem %d has a NULL operand", i);
         QLMX_REQUIRE(mode != GEMM_NT || p.B, "grouped gemm nt: problem %d has no B operand", i);
         QLMX_REQUIRE(p.beta == 0.0f || p.beta == 1.0f, "grouped gemm: beta must be 0 or 1");
-        const int rows = mode == GEMM_NT ? K : p.M;
-        DevProb &q = h[n++];
-        q.A = p.A; q.B = p.B; q.C = p.C; q.wq = p.wq; q.wg = p.wg; q.M = p.M;
-        q.beta = mode == GEMM_NN ? 0.0f : p.beta;
-        q.tile0 = (int)tiles; q.tiles_n = tiles_n; q.chunk = second ? 1 : 0; q.flag0 = 0;
-        tiles += (long long)((rows + tile_rows - 1) / tile_rows) * tiles_n;
-        QLMX_REQUIRE(tiles < (1LL << 30), "grouped gemm: too many tiles");
         if(second){
             const qlmx_gemm_prob &p2 = second[i];
             QLMX_REQUIRE(p2.M == p.M, "grouped gemm: problem %d and its second half differ in rows (%d, %d)", i, p.M, p2.M);
             QLMX_REQUIRE(mode == GEMM_TN ? p2.A != nullptr : (p2.B != nullptr && (p2.C != nullptr) == (p.C != nullptr)), "grouped gemm: the second half of problem %d lacks a pointer", i);
-            DevProb &c = h[n++];
-            c = q; c.A = p2.A; c.B = p2.B; c.C = p2.C; c.wq = p2.wq; c.wg = p2.wg; c.tile0 = (int)tiles; c.chunk = 0;
         }
     }
+    /* One table entry (two for a problem with a second half) covering rows [r0, r0 + m) of problem i. */
+    auto emit = [&](int i, int r0, int m){
+        const qlmx_gemm_prob &p = probs[i];
+        const int rows = mode == GEMM_NT ? K : m;
+        auto adv = [&](const void *ptr, size_t row_bytes) -> const void * { return (ptr && r0) ? (const void *)((const char *)ptr + (size_t)r0 * row_bytes) : ptr; };
+        DevProb &q = h[n++];
+        q.A = adv(p.A, rb ? rb->a : 0); q.B = p.B; q.C = (float *)adv(p.C, rb ? rb->c : 0); q.wq = p.wq; q.wg = p.wg; q.M = m;
+        q.beta = mode == GEMM_NN ? 0.0f : p.beta;
+        q.tile0 = (int)tiles; q.tiles_n = tiles_n; q.chunk = second ? 1 : 0; q.flag0 = 0;
+        tiles += (long long)((rows + tile_rows - 1) / tile_rows) * tiles_n;
+        if(second){
+            const qlmx_gemm_prob &p2 = second[i];
+            DevProb &c = h[n++];
+            c = q; c.A = adv(p2.A, rb ? rb->a2 : 0); c.B = adv(p2.B, rb ? rb->b2 : 0); c.C = (float *)adv(p2.C, rb ? rb->c2 : 0);
+            c.wq = p2.wq; c.wg = p2.wg; c.tile0 = (int)tiles; c.chunk = 0;
+        }
+    };
+    int nfull = 0;
+    if(rb){
+        /* Longest tiles first: a launch ends when its last workgroup does, workgroups start in table order, and
+         * under a skewed load a full-height tile handed out at the very end leaves most of the device waiting for
+         * it. Every problem is therefore entered twice: its whole row tiles in the first part of the table (in the
+         * caller's order, so that an expert's tiles stay together), its ragged last row tile in the second part,
+         * tallest first. Rows are independent in these products, so a part is a problem of its own whose row
+         * pointers start further down. */
+        for(int oi = 0; oi < live; oi++){ const int i = order[oi], full = probs[i].M / tile_rows * tile_rows; if(full) emit(i, 0, full); }
+        QLMX_REQUIRE(tiles < (1LL << 30), "grouped gemm: too many tiles");
+        nfull = (int)tiles;
+        static int tails[QLMX_MAX_PROBLEMS];
+        int nt = 0;
+        for(int oi = 0; oi < live; oi++) if(probs[order[oi]].M % tile_rows) tails[nt++] = order[oi];
+        std::stable_sort(tails, tails + nt, [&](int x, int y){ return probs[x].M % tile_rows > probs[y].M % tile_rows; });
+        for(int k = 0; k < nt; k++){ const int i = tails[k], full = probs[i].M / tile_rows * tile_rows; emit(i, full, probs[i].M - full); }
+    } else {
+        for(int oi = 0; oi < live; oi++) emit(order[oi], 0, probs[order[oi]].M);
+        nfull = (int)tiles;
+    }
+    QLMX_REQUIRE(tiles < (1LL << 30), "grouped gemm: too many tiles");
     (void)stream;
     DevProb *dst = g_ring_h + (size_t)slot * QLMX_MAX_PROBLEMS;
     memcpy(dst, stage, (size_t)n * sizeof(DevProb));
     table_publish();
-    out->dev = dst; out->ntiles = (int)tiles; out->nprob = n;
+    out->dev = dst; out->ntiles = (int)tiles; out->nprob = n; out->nfull = nfull;
     *slot_out = slot;
     return QLMX_OK;
 }
 
 int qlmx_upload_problems(const qlmx_gemm_prob *probs, int nprob, int mode, int K, int N,
                          int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot_out){
-    return upload_problems(probs, nullptr, nprob, mode, K, N, tile_rows, tile_cols, stream, out, slot_out);
+    return upload_problems(probs, nullptr, nprob, mode, K, N, tile_rows, tile_cols, nullptr, stream, out, slot_out);
 }
 int qlmx_upload_problem_pairs(const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int mode, int K, int N,
                               int tile_rows, int tile_cols, hipStream_t stream, ProbUpload *out, int *slot_out){
     QLMX_REQUIRE(second && (mode == GEMM_TN || mode == GEMM_NN), "grouped gemm: NULL list of second halves");
-    return upload_problems(first, second, nprob, mode, K, N, tile_rows, tile_cols, stream, out, slot_out);
+    return upload_problems(first, second, nprob, mode, K, N, tile_rows, tile_cols, nullptr, stream, out, slot_out);
+}
+int qlmx_upload_problems_split(const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int mode, int K, int N,
+                               int tile_rows, int tile_cols, const RowBytes *rb, hipStream_t stream, ProbUpload *out, int *slot_out){
+    QLMX_REQUIRE(rb && (mode == GEMM_TN || mode == GEMM_NN), "grouped gemm: row sizes are needed to split problems");
+    return upload_problems(first, second, nprob, mode, K, N, tile_rows, tile_cols, rb, stream, out, slot_out);
 }
 
 int qlmx_upload_done(int slot, hipStream_t stream){ return guard_launched(g_ring_guard, slot, stream); }

@@ -75,6 +75,20 @@ def timed(torch, fn, steps, warmup):
     return {"wall_ms": wall, "event_ms_avg": a.elapsed_time(b) / steps}
 
 
+def step_spread(torch, fn, steps):
+    """Duration of every single step of `steps` more (an event behind each: some 6 us of idle GPU per step ride along,
+    which is why the mean comes from timed() and only the spread from here): a stall that a mean would hide shows as max."""
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    ev[0].record()
+    for i in range(steps):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    ms = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(steps))
+    return {"min": ms[0], "p50": ms[len(ms) // 2], "p99": ms[min(len(ms) - 1, (len(ms) * 99) // 100)], "max": ms[-1],
+            "note": "per-step events: each adds a few us of idle GPU to its step"}
+
+
 
 # --------------------------------------------------------------------------------------------- train
 def zipf_counts(E, tokens, topk, seed=0):
@@ -169,6 +183,7 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
             q.side_fork(stream); side[4][1](); calls[5][1](); q.side_join(stream)
 
     tm = timed(torch, step, args.steps, args.warmup)
+    spread = step_spread(torch, step, args.steps)
     per = {}
     for name, fn, ng in ([] if args.step_only else calls):
         t1 = timed(torch, fn, max(5, args.steps // 2), 2)
@@ -179,7 +194,7 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
     g_up = P([(None, act.data_ptr() + off[e] * F * 2, up.data_ptr() + off[e] * F * 4, o3 + e * D * F, (o3 + e * D * F) // group, int(cnt[e]), 0.0)
               for e in range(E)])
     extra = {}
-    for name, fn in [] if args.step_only else [("fwd w1,w3 + SwiGLU, one launch", lambda: q.gemm_nn_swiglu(d, s, group, g_gate, g_up, E, D, F, ACT_BF16, MATH_MFMA, stream)),
+    for name, fn in [] if args.step_only else [("fwd w1,w3 + SwiGLU, one launch", lambda: q.gemm_nn_swiglu(d, s, group, g_gate, g_up, E, D, F, ACT_BF16, FWD, stream)),
                      ("SwiGLU kernel alone", lambda: q.swiglu(gp, up, act, rows * F, ACT_BF16, stream))]:
         extra[name] = {"ms": timed(torch, fn, max(5, args.steps // 2), 2)["event_ms_avg"]}
     flops = 9 * unit
@@ -190,10 +205,11 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
                     "fwd+dgrad+wgrad = 9 grouped GEMMs in 6 launches%s" % (label, E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min()),
                        ", the weight gradient of each backward flush on a second stream beside its input gradient" if (args.bwd_streams or 2) == 2 else ""),
         "bwd_streams": args.bwd_streams or 2,
-        "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tm["wall_ms"], "dtype": "bf16",
-        "kernel_ms": tm, "per_launch": per, "beside_the_step": extra, "gflop_per_step": flops / 1e9,
+        "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tm["wall_ms"],
+        "dtype": "bf16" if args.fwd_math == "bf16x2" else "bf16 (fwd: fp16 MFMA)",
+        "kernel_ms": tm, "step_ms_spread": spread, "per_launch": per, "beside_the_step": extra, "gflop_per_step": flops / 1e9,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "kernel": "k_gemm_nn_lds, k_gemm_tn_lds, k_gemm_nt_lds (all 6 launches; slowest: %s)" % dom,
+                     "traffic": None, "kernel": "k_gemm_nn_h, k_gemm_tn_lds, k_gemm_nt_lds (all 6 launches; slowest: %s)" % dom,
                      "note": "algorithmic flops only; forward math: " + ("bf16 hi+lo weight split, two MFMAs per product" if args.fwd_math == "bf16x2" else
                              "fp16 matrix core, bf16 activations converted exactly, weights rounded once to fp16 (2e-4 relative L2), one MFMA per product")},
     }
@@ -332,15 +348,30 @@ def bench_layer(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2):
     t_sep = timed(torch, lambda: layer(per_pass, False, False), steps, warmup)
     t_fus = timed(torch, lambda: layer(per_pass, True, False), steps, warmup)
     t_mrg = timed(torch, lambda: layer(one_list, True, True), steps, warmup)
+    spread = step_spread(torch, lambda: layer(one_list, True, True), steps)
+
+    def glue_only():
+        """the kernels of the merged layer that are not GEMMs: token matrix to bf16, the gather for the weight gradient,
+        the gate gradient, the two combines"""
+        L = one_list
+        q.moe_gather(x, ident, xb, N, D, ACT_BF16, stream)
+        q.moe_combine(yp, L.inv, gate, out, N, K, D, stream)
+        q.moe_gather(x, L.tok, Xp, L.R, D, ACT_BF16, stream)
+        q.moe_dgate_merged(dout, yp, L.perm, gate, dgate, dyp, N, K, D, ACT_BF16, stream)
+        q.moe_combine(dXp, L.inv, None, dx, N, K, D, stream)
+    t_glue = timed(torch, glue_only, steps, warmup)
     flops = K * 12 * 2.0 * N * D * F                       # per pass: 3 forward GEMMs, 3 recomputed in the backward, 3 dgrad, 3 wgrad
     tf = flops / (t_mrg["event_ms_avg"] * 1e-3) / 1e12
     return {"workload": "C3 whole expert layer, forward + backward with the recomputed forward (%d tokens top-%d, E=%d D=%d F=%d): GEMMs and glue" % (N, K, E, D, F),
             "metric": "layer TFLOP/s (12 GEMMs per token and pass incl. the recomputed forward; all passes as one grouped list, glue folded in)",
-            "value": tf, "unit": "TFLOP/s", "ms_per_step": t_mrg["wall_ms"], "dtype": "bf16", "steps": steps, "warmup": warmup,
+            "value": tf, "unit": "TFLOP/s", "ms_per_step": t_mrg["wall_ms"], "dtype": "bf16 (fwd: fp16 MFMA)", "steps": steps, "warmup": warmup,
+            "gflop_per_step": flops / 1e9, "step_ms_spread": spread,
+            "glue_ms": {"the five kernels of the merged layer that are not GEMMs, timed on their own": t_glue["event_ms_avg"]},
             "layer_ms": {"pass by pass, glue as separate kernels": t_sep["event_ms_avg"], "pass by pass, glue folded into the GEMMs": t_fus["event_ms_avg"],
                          "all passes as one list, glue folded in": t_mrg["event_ms_avg"]},
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
-                         "kernel": "whole layer: grouped GEMMs + router-independent glue"}}
+                         "kernel": "whole layer: 8 grouped GEMM launches (k_gemm_nn_h, k_gemm_nn_h_swiglu, k_gemm_tn_lds, k_gemm_nt_lds) + 5 glue kernels",
+                         "note": "algorithmic flops only (12 GEMMs per token and pass, the recomputed forward included); glue time is inside the step"}}
 
 
 # --------------------------------------------------------------------------------------------- c5
@@ -864,7 +895,7 @@ def main():
     pkg = load_package()
     q = pkg.load()           # raises if libqlmx.so is missing or no gfx950 device
     torch.cuda.set_device(0)
-    want = ["train", "decode", "adamw", "c5"] if args.workload == "all" else [args.workload]
+    want = ["train", "layer", "decode", "adamw", "c5"] if args.workload == "all" else [args.workload]
     runners = {"adamw": bench_adamw, "train": bench_train, "decode": bench_decode, "copy": bench_copy, "codec": bench_codec, "glue": bench_glue, "c5": bench_c5, "layer": bench_layer,
                "train5": lambda t, qq, a: bench_train(t, qq, a, E=64, D=2048, F=1408, tokens=32768, topk=4, label="C5 train layer (one of 8)")}
     results = {}

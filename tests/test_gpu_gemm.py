@@ -121,6 +121,62 @@ def test_f32_c1_single_expert(q, orc):
             assert orc.relerr(got, want) < TOL_F32, (mode, K, N)
 
 
+def test_f32_c1_whole_chain_into_the_integer_step(q, orc):
+    """BASELINE config 1 as one chain on its own two matrices: X fp32 [1024,512] ~ N(0,1), W_up [512,1536] and W_down
+    [1536,512] from 0.02 N(0,1) through encode; H = X.W_up, Y = H.W_down; dH = dY.W_down^T, dX = dH.W_up^T;
+    dW_down = H^T.dY, dW_up = X^T.dH with dY ~ N(0,1) (SURVEY's statement of the config: no activation between the two);
+    then one Integer AdamW step, t = 1, from fresh state (m8 = v8 = 0, moment scales 0) on both matrices with the weight
+    gradients scaled to the config's 1e-3 (the device clip scalar: gsp). Every GEMM against the oracle's at 1e-5; the
+    step byte for byte against the oracle's step fed the same gradient bits (the step's parity is defined on equal
+    gradients: it rounds stochastically on every bit of them)."""
+    import torch
+    M, D, F, group, dmax = 1024, 512, 1536, 128, 7
+    n_up, n_dn = D * F, F * D
+    tab, nq, ng = make_spans([n_up, n_dn], group)
+    P = orc.normal(nq, 0, 1, 0.02)
+    hd = np.zeros(nq // 2, np.int8); hr = np.zeros(nq, np.int8); hs = np.zeros(ng, f32)
+    orc.encode(P, hd, hr, hs, tab, group, dmax, 1, ng)
+    orc.span_sref(tab, hs)
+    orc.render(P, hd, hs, tab, group, 1, 0, ng)
+    X = orc.normal(M * D, 0, 2); dY = orc.normal(M * D, 0, 3)
+    dd, ds, dX_, ddY = dev(hd), dev(hs), dev(X), dev(dY)
+    z = lambda k: torch.zeros(k, device="cuda")
+    H, Y, dH, dXo, G = z(M * F), z(M * D), z(M * F), z(M * D), z(nq)
+    one = lambda A, B, C, wq, beta=0.0: q.problems([(A, B, C, wq, wq // group, M, beta)])
+    f = (pkg.ACT_F32, pkg.MATH_F32)
+    q.gemm_nn(dd, ds, group, one(dX_, None, H, 0), 1, D, F, *f)
+    q.gemm_nn(dd, ds, group, one(H, None, Y, n_up), 1, F, D, *f)
+    q.gemm_tn(dd, ds, group, one(ddY, None, dH, n_up), 1, D, F, *f)
+    q.gemm_tn(dd, ds, group, one(dH, None, dXo, 0), 1, F, D, *f)
+    q.gemm_nt(q.problems([(H.data_ptr(), ddY.data_ptr(), G.data_ptr() + n_up * 4, 0, 0, M, 1.0)]), 1, F, D, *f)
+    q.gemm_nt(q.problems([(dX_.data_ptr(), dH.data_ptr(), G.data_ptr(), 0, 0, M, 1.0)]), 1, D, F, *f)
+    torch.cuda.synchronize()
+    w_up, w_dn = P[:n_up], P[n_up:]
+    hH = np.zeros(M * F, f32); orc.gemm_nn(X, w_up, hH, M, D, F)
+    hY = np.zeros(M * D, f32); orc.gemm_nn(hH, w_dn, hY, M, F, D)
+    hdH = np.zeros(M * F, f32); orc.gemm_tn(dY, w_dn, hdH, M, D, F, 0.0)
+    hdX = np.zeros(M * D, f32); orc.gemm_tn(hdH, w_up, hdX, M, F, D, 0.0)
+    hG = np.zeros(nq, f32); orc.gemm_nt(hH, dY, hG[n_up:], M, F, D); orc.gemm_nt(X, hdH, hG[:n_up], M, D, F)
+    for name, got, want in [("H", H, hH), ("Y", Y, hY), ("dH", dH, hdH), ("dX", dXo, hdX), ("dW", G, hG)]:
+        assert orc.relerr(got.cpu().numpy(), want) < TOL_F32, name
+    # the step on the device's own gradient bits, scaled to ~1e-3 by the clip scalar
+    gG = G.cpu().numpy()
+    scale = np.array([1e-3 / float(np.sqrt(np.mean(gG.astype(np.float64) ** 2))), 0.0], f32)
+    r, m8, v8 = dev(hr), torch.zeros(nq, dtype=torch.int8, device="cuda"), torch.zeros(nq, dtype=torch.uint8, device="cuda")
+    m8s, v8s = z(ng), z(ng)
+    hm8, hv8, hm8s, hv8s = np.zeros(nq, np.int8), np.zeros(nq, np.uint8), np.zeros(ng, f32), np.zeros(ng, f32)
+    bc1, bc2 = f32(1) - f32(0.9), f32(1) - f32(0.95)
+    span_bytes = tab.view(np.uint8)
+    hp = (3e-4, 0.9, 0.95, 0.1, 1.0)
+    tail = (float(f32(1) / bc1), float(f32(1) / np.sqrt(bc2)), 0, 1, 1, None, 1, 0, ng)
+    q.step(None, G, dd, r, ds, m8, m8s, v8, v8s, dev(span_bytes), 2, group, dmax, *hp, dev(scale), *tail)
+    orc.step(None, gG, hd, hr, hs, hm8, hm8s, hv8, hv8s, tab, group, dmax, *hp, scale, *tail)
+    torch.cuda.synchronize()
+    assert int((hm8 != 0).sum()) > nq // 2 and int((hv8 != 0).sum()) > nq // 2        # the step did something
+    for name, got, want in [("d", dd, hd), ("r", r, hr), ("m8", m8, hm8), ("v8", v8, hv8), ("m8s", m8s, hm8s), ("v8s", v8s, hv8s)]:
+        assert np.array_equal(got.cpu().numpy().view(np.uint8), want.view(np.uint8)), name
+
+
 def test_f32_bf16_acts_and_group64(q, orc):
     got, want = run_case(q, orc, "nn", 3, [40, 1, 77], 192, 128, pkg.ACT_BF16, pkg.MATH_F32, seed=5, group=64)
     assert orc.relerr(got, want) < TOL_F32

@@ -519,7 +519,8 @@ def test_layer_forward_backward_vs_oracle(q, orc, math, N, E, D, F, K):
     # that is off by eps lands on the other side of a rounding boundary with probability eps / 2^-8 and is then off by
     # a whole bf16 step, sqrt(2e-4 * 2^-8) = 9e-4 in relative L2 -- against an oracle that rounds the exact values the
     # whole layer therefore shows 0.9e-3 to 1.1e-3 (observed), of which the GEMMs' own share is the 2e-4.
-    if fused: tol = 1.5e-3
+    # (1.11e-3 is the largest figure of the five fused cases below; every GEMM's own share is asserted further down.)
+    if fused: tol = 1.2e-3
     d, s, P, n = encode_layer(orc, 40 + N, E, D, F)
     x = orc.normal(N * D, 41, 1)
     dout = orc.normal(N * D, 41, 2)
@@ -569,24 +570,44 @@ def test_layer_forward_backward_vs_oracle(q, orc, math, N, E, D, F, K):
         assert torch.equal(out, out2) and torch.equal(dx, dx2) and torch.equal(dgate, dgate2)
         for a, b in zip(G, G2):
             assert orc.relerr(a.cpu().numpy(), b.cpu().numpy()) < 1e-5
-        # every matmul of the layer against the oracle ON THE LAYER'S OWN INPUTS (the grouped buffers hold all K*N rows
-        # after the backward pass), for the expert with the most rows: the 1e-3 bar of a matmul output
-        e = int(np.argmax(np.diff(L.offh[0]))); o, ne = int(L.offh[0][e]), int(L.offh[0][e + 1] - L.offh[0][e]); DF = D * F
-        rows = lambda t, cols, bf: (bf16_to_f32(t[o * cols:(o + ne) * cols]) if bf else t[o * cols:(o + ne) * cols].cpu().numpy())
-        Xp_e, ap_e, dyp_e, dgp_e, dup_e = rows(L.Xp, D, 1), rows(L.ap, F, 1), rows(L.dyp, D, 1), rows(L.dgp, F, 1), rows(L.dup, F, 1)
-        w1, w3, w2 = P[e * DF:(e + 1) * DF], P[n + e * DF:n + (e + 1) * DF], P[2 * n + e * DF:2 * n + (e + 1) * DF]
-        stage = {}
-        c = np.zeros(ne * F, f32); orc.gemm_nn(Xp_e, w1, c, ne, D, F); stage["gp"] = orc.relerr(rows(L.gp, F, 0), c)
-        c = np.zeros(ne * F, f32); orc.gemm_nn(Xp_e, w3, c, ne, D, F); stage["up"] = orc.relerr(rows(L.up, F, 0), c)
-        c = np.zeros(ne * D, f32); orc.gemm_nn(ap_e, w2, c, ne, F, D); stage["yp"] = orc.relerr(rows(L.yp, D, 0), c)
-        c = np.zeros(ne * D, f32); orc.gemm_tn(dgp_e, w1, c, ne, F, D, 0.0); orc.gemm_tn(dup_e, w3, c, ne, F, D, 1.0)
-        stage["dXp"] = orc.relerr(rows(L.dXp, D, 0), c)
-        c = np.zeros(DF, f32); orc.gemm_nt(ap_e, dyp_e, c, ne, F, D); stage["G_w2"] = orc.relerr(G[2][e * DF:(e + 1) * DF].cpu().numpy(), c)
-        c = np.zeros(DF, f32); orc.gemm_nt(Xp_e, dgp_e, c, ne, D, F); stage["G_w1"] = orc.relerr(G[0][e * DF:(e + 1) * DF].cpu().numpy(), c)
-        c = np.zeros(DF, f32); orc.gemm_nt(Xp_e, dup_e, c, ne, D, F); stage["G_w3"] = orc.relerr(G[1][e * DF:(e + 1) * DF].cpu().numpy(), c)
-        print("    expert %d (%d rows), each matmul on the layer's own inputs:" % (e, ne), {k: "%.2e" % v for k, v in stage.items()})
-        assert max(stage.values()) < 1e-3, stage
     if math == "mfma":
+        # Every matmul of the layer against the oracle ON THE LAYER'S OWN INPUTS, for the expert with the most rows and
+        # the one with the fewest: the 1e-3 bar of a matmul output, one GEMM at a time. After the backward pass the
+        # grouped buffers hold the rows of the last list that ran (all K*N rows when merged, the last pass otherwise); a
+        # pass-by-pass layer sums its weight gradients over the passes, so there the three weight-gradient GEMMs are
+        # run once more on the last pass's buffers into gradients of their own.
+        k = L.offh.shape[0] - 1
+        Gs = G
+        if variant != "merged":
+            Gs = [zeros(n) for _ in range(3)]
+            if fused:
+                pr = lambda A, a_cols, Gm, B, b_cols: L.probs(k, A, a_cols, Gm, 0, 0, B=B, b_cols=b_cols, beta=1.0, out_expert=True)
+            else:
+                pr = lambda A, a_cols, Gm, B, b_cols: L.probs(k, A, a_cols, 2, Gm, 0, 0, B=B, b_cols=b_cols, b_esz=2, beta=1.0, out_expert=True)
+            q.gemm_nt(pr(L.ap, F, Gs[2], L.dyp, D), E, F, D, pkg.ACT_BF16, pkg.MATH_MFMA)
+            q.gemm_nt(pr(L.Xp, D, Gs[0], L.dgp, F), E, D, F, pkg.ACT_BF16, pkg.MATH_MFMA)
+            q.gemm_nt(pr(L.Xp, D, Gs[1], L.dup, F), E, D, F, pkg.ACT_BF16, pkg.MATH_MFMA)
+            torch.cuda.synchronize()
+        cnt = np.diff(L.offh[k]); DF = D * F
+        for e in sorted({int(np.argmax(cnt)), int(np.argmin(np.where(cnt > 0, cnt, cnt.max() + 1)))}):
+            o, ne = int(L.offh[k][e]), int(cnt[e])
+            rows = lambda t, cols, bf: (bf16_to_f32(t[o * cols:(o + ne) * cols]) if bf else t[o * cols:(o + ne) * cols].cpu().numpy())
+            Xp_e, ap_e, dyp_e, dgp_e, dup_e = rows(L.Xp, D, 1), rows(L.ap, F, 1), rows(L.dyp, D, 1), rows(L.dgp, F, 1), rows(L.dup, F, 1)
+            w1, w3, w2 = P[e * DF:(e + 1) * DF], P[n + e * DF:n + (e + 1) * DF], P[2 * n + e * DF:2 * n + (e + 1) * DF]
+            stage = {}
+            c = np.zeros(ne * F, f32); orc.gemm_nn(Xp_e, w1, c, ne, D, F); stage["gp"] = orc.relerr(rows(L.gp, F, 0), c)
+            c = np.zeros(ne * F, f32); orc.gemm_nn(Xp_e, w3, c, ne, D, F); stage["up"] = orc.relerr(rows(L.up, F, 0), c)
+            c = np.zeros(ne * D, f32); orc.gemm_nn(ap_e, w2, c, ne, F, D); stage["yp"] = orc.relerr(rows(L.yp, D, 0), c)
+            if not fused:                                              # the fused layer never stores d(act)
+                c = np.zeros(ne * F, f32); orc.gemm_tn(dyp_e, w2, c, ne, D, F, 0.0); stage["dap"] = orc.relerr(rows(L.dap, F, 0), c)
+            if variant != "fused":                                     # ... and its pass-by-pass form scatters dXp from the accumulators
+                c = np.zeros(ne * D, f32); orc.gemm_tn(dgp_e, w1, c, ne, F, D, 0.0); orc.gemm_tn(dup_e, w3, c, ne, F, D, 1.0)
+                stage["dXp"] = orc.relerr(rows(L.dXp, D, 0), c)
+            c = np.zeros(DF, f32); orc.gemm_nt(ap_e, dyp_e, c, ne, F, D); stage["G_w2"] = orc.relerr(Gs[2][e * DF:(e + 1) * DF].cpu().numpy(), c)
+            c = np.zeros(DF, f32); orc.gemm_nt(Xp_e, dgp_e, c, ne, D, F); stage["G_w1"] = orc.relerr(Gs[0][e * DF:(e + 1) * DF].cpu().numpy(), c)
+            c = np.zeros(DF, f32); orc.gemm_nt(Xp_e, dup_e, c, ne, D, F); stage["G_w3"] = orc.relerr(Gs[1][e * DF:(e + 1) * DF].cpu().numpy(), c)
+            print("    expert %d (%d rows), each matmul on the layer's own inputs:" % (e, ne), {k_: "%.2e" % v for k_, v in stage.items()})
+            assert max(stage.values()) < 1e-3, (e, stage)
         f_out, f_dx, f_dgate, f_G = oracle_layer(False)             # the CPU build's all-fp32 layer, end to end
         want = {"out": f_out, "dx": f_dx, "dgate": f_dgate, "G_w1": f_G[0], "G_w3": f_G[1], "G_w2": f_G[2]}
         e2e = {k: orc.relerr(got[k].cpu().numpy(), want[k]) for k in got}

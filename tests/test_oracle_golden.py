@@ -510,3 +510,28 @@ def test_sqsum_closed_forms(orc):
     assert part[13] == 9.0 and part[50] == 16.0 and part.sum() == 25.0
     gs = orc.gnorm(part, 0, 0)
     assert gs[1] == 5.0 and gs[0] == f32(1.0) / f32(5.0)
+
+
+def test_span_sref_is_the_mean_of_the_span_scales(orc):
+    """orc_span_sref (qlm.cuh:527-536: the double sum of a span's group scales in group order, divided by the group
+    count, rounded to float) against math.fsum -- the exactly rounded sum, which a running double sum of at most a few
+    thousand floats of one magnitude can only miss by units in the last place of a double, far below half a float
+    ulp except on an exact tie -- for spans of 1 to 3000 groups, scales spread over six decades, plus the closed forms:
+    equal scales give that scale back, and one span's mean does not depend on its neighbours."""
+    import math
+    sizes = [128 * k for k in (1, 2, 3, 7, 64, 999, 3000)]
+    tab, nq, ng = make_spans(sizes, 128)
+    s = (orc.uniform(ng, 3, 1, 0.5, 1.5) * np.float32(10.0) ** (orc.uniform(ng, 3, 2, -6.0, 0.0))).astype(np.float32)
+    orc.span_sref(tab, s)
+    for i in range(len(sizes)):
+        g0, n = int(tab["gi0"][i]), int(tab["ngrp"][i])
+        want = np.float32(math.fsum(float(v) for v in s[g0:g0 + n]) / n)
+        assert np.float32(tab["sref"][i]).view(np.uint32) == want.view(np.uint32), (i, tab["sref"][i], want)
+    flat = np.full(ng, np.float32(0.0123), np.float32)
+    orc.span_sref(tab, flat)
+    assert all(np.float32(v) == np.float32(0.0123) for v in tab["sref"])
+    tab2, _, ng2 = make_spans(sizes[3:5], 128)
+    g0 = int(tab["gi0"][3])
+    orc.span_sref(tab, s)
+    orc.span_sref(tab2, s[g0:g0 + ng2].copy())
+    assert np.array_equal(np.asarray(tab2["sref"], np.float32), np.asarray(tab["sref"][3:5], np.float32))

@@ -28,22 +28,26 @@ typedef short  s16x4  __attribute__((ext_vector_type(4)));
 typedef short  s16x8  __attribute__((ext_vector_type(8)));
 typedef float  f32x16 __attribute__((ext_vector_type(16)));
 
-/* Two tile shapes, one kernel body (template parameter BN = columns of dY per tile):
+/* Two tile shapes, one kernel body (template parameters BN = columns of dY per tile, NW = wavefronts):
  *   256 x 128: four wavefronts of 128 x 64, two workgroups per CU (256 registers each);
- *   256 x 256: four wavefronts of 128 x 128, one workgroup per CU, the 256 accumulator registers of a
- *              wavefront in the accumulation half of its 512: a third fewer LDS bytes read and a third fewer
- *              bytes brought into LDS per multiplication, but nothing else resident on the CU to cover a
- *              workgroup's waits, prologue and epilogue. Not faster as measured (see nt3_pick_bn); opt-in. */
+ *   256 x 256: eight wavefronts of 128 x 64, one workgroup per CU: a third fewer bytes brought into LDS per
+ *              multiplication, but all eight wavefronts meet at one barrier per step, so the two on a SIMD read
+ *              their operands at the same time instead of one multiplying while the other reads, and nothing
+ *              else is resident to cover the prologue and the epilogue. Not faster as measured (see
+ *              nt3_pick_bn); opt-in. */
 #define NT3_BM 256
 #define NT3_BK 32
 #define NT3_STAGES 3
 #define NT3_A_BYTES (NT3_BK * NT3_BM * 2)      /* 16384 */
-template<int BN> struct Nt3Shape {
-    static constexpr int NJ = BN / 64;                       /* 32-column accumulator tiles per wavefront */
-    static constexpr int NB = BN / 64;                       /* 16-byte pieces of dY a thread fetches per tile */
+template<int BN, int NW> struct Nt3Shape {
+    static constexpr int NT = NW * 64;                       /* threads */
+    static constexpr int WN = NW / 2;                        /* wavefronts side by side along dY's columns (two along X's) */
+    static constexpr int NJ = BN / (32 * WN);                /* 32-column accumulator tiles per wavefront */
+    static constexpr int NA = NT3_A_BYTES / 16 / NT;         /* 16-byte pieces of X a thread fetches per tile */
+    static constexpr int NB = NT3_BK * BN * 2 / 16 / NT;     /* and of dY */
     static constexpr int B_BYTES = NT3_BK * BN * 2;
     static constexpr int STAGE_BYTES = NT3_A_BYTES + B_BYTES;
-    static constexpr int NREQ = 4 + NB;                      /* requests per thread and tile */
+    static constexpr int NREQ = NA + NB;                     /* requests per thread and tile */
     static constexpr int LDS_BYTES = NT3_STAGES * STAGE_BYTES;
     static constexpr int WG_PER_CU = BN == 128 ? 2 : 1;
 };
@@ -86,12 +90,6 @@ __device__ __forceinline__ void nt3_wait_reads(Nt3Ops<2> &o){
         : "+v"(o.a[0][0]), "+v"(o.a[0][1]), "+v"(o.a[1][0]), "+v"(o.a[1][1]), "+v"(o.a[2][0]), "+v"(o.a[2][1]),
           "+v"(o.a[3][0]), "+v"(o.a[3][1]), "+v"(o.b[0][0]), "+v"(o.b[0][1]), "+v"(o.b[1][0]), "+v"(o.b[1][1]));
 }
-__device__ __forceinline__ void nt3_wait_reads(Nt3Ops<4> &o){
-    asm volatile("s_waitcnt lgkmcnt(0)"
-        : "+v"(o.a[0][0]), "+v"(o.a[0][1]), "+v"(o.a[1][0]), "+v"(o.a[1][1]), "+v"(o.a[2][0]), "+v"(o.a[2][1]),
-          "+v"(o.a[3][0]), "+v"(o.a[3][1]), "+v"(o.b[0][0]), "+v"(o.b[0][1]), "+v"(o.b[1][0]), "+v"(o.b[1][1]),
-          "+v"(o.b[2][0]), "+v"(o.b[2][1]), "+v"(o.b[3][0]), "+v"(o.b[3][1]));
-}
 __device__ __forceinline__ bf16x8 nt3_pack(const i32x2 lo, const i32x2 hi){
     const i32x4 v = {lo[0], lo[1], hi[0], hi[1]};
     return __builtin_bit_cast(bf16x8, v);
@@ -101,10 +99,10 @@ __device__ __forceinline__ int t_of(int b, const Nt3Args &a){
     return (a.rows_p & 7) ? qx_xcd_tile_probs(b, a.tiles_n, a.rows_p) : qx_xcd_tile_rows(b, a.tiles_n);
 }
 
-template<int BN>
-__global__ void __launch_bounds__(256, Nt3Shape<BN>::WG_PER_CU) k_gemm_nt_lds(Nt3Args a){
-    typedef Nt3Shape<BN> SH;
-    constexpr int NJ = SH::NJ, NB = SH::NB;
+template<int BN, int NW>
+__global__ void __launch_bounds__(NW * 64, (Nt3Shape<BN, NW>::WG_PER_CU)) k_gemm_nt_lds(Nt3Args a){
+    typedef Nt3Shape<BN, NW> SH;
+    constexpr int NJ = SH::NJ, NA = SH::NA, NB = SH::NB, NT = SH::NT;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     /* scheduled launch: the unit table says what to do; otherwise the tile follows from the index */
     int pi, i0, j0, k0 = 0, depth = -1, seq = 0, nseq = 1, flag = 0;
@@ -133,21 +131,21 @@ __global__ void __launch_bounds__(256, Nt3Shape<BN>::WG_PER_CU) k_gemm_nt_lds(Nt
         i0 = ti * NT3_BM; j0 = tj * BN; depth = P.M;
     }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wi = (wave >> 1) * 128, wj = (wave & 1) * (BN / 2);
+    const int wi = (wave / SH::WN) * 128, wj = (wave % SH::WN) * (BN / SH::WN);
 
     /* ---- what this thread fetches per tile: four 16-byte pieces of X, two of dY. Piece p of a tile
      * (LDS position 16*p) is row p/32 (p/16 for dY), stored unit p%32 = logical unit ^ swizzle. ---- */
-    const char *srcA[4]; const char *srcB[NB]; int rowA[4], rowB[NB];
+    const char *srcA[NA]; const char *srcB[NB]; int rowA[NA], rowB[NB];
 #pragma unroll
-    for(int h = 0; h < 4; h++){
-        const int p = h * 256 + tid, row = p >> 5, lu = (p & 31) ^ ((row & 3) << 2);
+    for(int h = 0; h < NA; h++){
+        const int p = h * NT + tid, row = p >> 5, lu = (p & 31) ^ ((row & 3) << 2);
         const int col = i0 + lu * 8;
         rowA[h] = row;
         srcA[h] = (const char *)P.A + ((size_t)(k0 + row) * a.K + (col < a.K ? col : 0)) * 2;   /* columns past K feed rows that are never stored */
     }
 #pragma unroll
     for(int h = 0; h < NB; h++){
-        const int p = h * 256 + tid, row = p / (BN / 8), lu = (p & (BN / 8 - 1)) ^ ((row & 3) << 2);
+        const int p = h * NT + tid, row = p / (BN / 8), lu = (p & (BN / 8 - 1)) ^ ((row & 3) << 2);
         rowB[h] = row;
         srcB[h] = (const char *)P.B + ((size_t)(k0 + row) * a.N + j0 + lu * 8) * 2;
     }
@@ -158,12 +156,12 @@ __global__ void __launch_bounds__(256, Nt3Shape<BN>::WG_PER_CU) k_gemm_nt_lds(Nt
     auto issue_one = [&](int tile, int stage, int h){
         const int kt = tile * NT3_BK;
         unsigned char *base = lds + stage * SH::STAGE_BYTES + wave_off;
-        if(h < 4){
+        if(h < NA){
             const char *g = (kt + rowA[h] < depth) ? srcA[h] + (size_t)tile * stepA : (const char *)a.zeros;
-            __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(base + h * 4096), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(base + h * (NT * 16)), 16, 0, 0);
         } else {
-            const char *g = (kt + rowB[h - 4] < depth) ? srcB[h - 4] + (size_t)tile * stepB : (const char *)a.zeros;
-            __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(base + NT3_A_BYTES + (h - 4) * 4096), 16, 0, 0);
+            const char *g = (kt + rowB[h - NA] < depth) ? srcB[h - NA] + (size_t)tile * stepB : (const char *)a.zeros;
+            __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(base + NT3_A_BYTES + (h - NA) * (NT * 16)), 16, 0, 0);
         }
     };
     auto issue = [&](int tile, int stage){
@@ -310,20 +308,24 @@ static int nt3_schedule(DevProb *pr, int n, int K, int N, int BN, int slots_per_
     return nent * g;
 }
 
-template<int BN> static int nt3_launch(const Nt3Args &a, int grid, hipStream_t st){
+template<int BN, int NW> static int nt3_launch(const Nt3Args &a, int grid, hipStream_t st){
     static bool attr_set = false;
     if(!attr_set){
-        QLMX_HIP(hipFuncSetAttribute((const void *)k_gemm_nt_lds<BN>, hipFuncAttributeMaxDynamicSharedMemorySize, Nt3Shape<BN>::LDS_BYTES), "nt LDS size");
+        QLMX_HIP(hipFuncSetAttribute((const void *)(k_gemm_nt_lds<BN, NW>), hipFuncAttributeMaxDynamicSharedMemorySize, (Nt3Shape<BN, NW>::LDS_BYTES)), "nt LDS size");
         attr_set = true;
     }
-    hipLaunchKernelGGL(k_gemm_nt_lds<BN>, dim3(grid), dim3(256), Nt3Shape<BN>::LDS_BYTES, st, a);
+    hipLaunchKernelGGL((k_gemm_nt_lds<BN, NW>), dim3(grid), dim3(NW * 64), (Nt3Shape<BN, NW>::LDS_BYTES), st, a);
     return QLMX_OK;
 }
+static int nt3_launch_any(int BN, const Nt3Args &a, int grid, hipStream_t st){
+    return BN == 128 ? nt3_launch<128, 4>(a, grid, st) : nt3_launch<256, 8>(a, grid, st);
+}
 
-/* Which tile. The wide one is built and correct but not faster on this GPU (uniform 2048-row experts,
- * K=768 N=2048: 873 against 861 TFLOP/s; 8192 rows: 841 against 943; with the operand reads issued a slice
- * ahead and the barrier between the slices: 807), so it is only taken on request: QLMX_NT_TILE=256 in the
- * environment (read at the first call), or qlmx_nt_tile(256). */
+/* Which tile. The wide one is built and correct but not faster on this GPU. Uniform experts, K=768 N=2048,
+ * TFLOP/s at 512 / 2048 / 8192 rows per expert: 128 columns 733 / 931 / 932; 256 columns 690 / 972 / 872 (on
+ * four wavefronts of 128 x 128 it was 636 / 935 / 824); the config-5 step is the same with either (870 and
+ * 872 TFLOP/s). So the wide tile is only taken on request: QLMX_NT_TILE=256 in the environment (read at the
+ * first call) or qlmx_nt_tile(256). */
 static int g_nt3_forced = -1;
 static int nt3_pick_bn(int N){
     if(g_nt3_forced < 0){ const char *e = getenv("QLMX_NT_TILE"); g_nt3_forced = e ? atoi(e) : 0; }
@@ -371,7 +373,7 @@ int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N
                 if(nflags && qlmx_test_take_forced_timeout(2)){ a.wait_epoch = a.epoch ^ 0x00A5A5A5u; a.wait_limit = 1; }
                 for(int p = 0; p < n; p++) uu.hprob[p].flag0 += first;
                 qlmx_unit_commit(&uu, n, nent);
-                rc = BN == 128 ? nt3_launch<128>(a, grid, st) : nt3_launch<256>(a, grid, st); if(rc) return rc;
+                rc = nt3_launch_any(BN, a, grid, st); if(rc) return rc;
                 QLMX_LAUNCH_CHECK("grouped gemm nt (scheduled) launch");
                 return qlmx_unit_done(uslot, st);
             }
@@ -385,7 +387,7 @@ int qlmx_gemm_nt_lds_launch(const qlmx_gemm_prob *probs, int nprob, int K, int N
     int grid;
     if(a.rows_p & 7) grid = 8 * a.tiles_n * a.rows_p * ((up.nprob + 7) / 8);
     else             grid = 8 * a.tiles_n * ((up.ntiles / a.tiles_n + 7) / 8);
-    rc = BN == 128 ? nt3_launch<128>(a, grid, st) : nt3_launch<256>(a, grid, st); if(rc) return rc;
+    rc = nt3_launch_any(BN, a, grid, st); if(rc) return rc;
     QLMX_LAUNCH_CHECK("grouped gemm nt (direct-to-LDS) launch");
     return qlmx_upload_done(slot, st);
 }

@@ -362,7 +362,7 @@ int qlmx_swiglu_bwd(const float *Gg, const float *U, const float *dact, void *dg
  * entry point returns QLMX_E_HIP once, exactly as after a real time-out. One-shot; the call after that is normal. */
 int qlmx_test_force_wait_timeout(int which);
 /* Tuning and test hook (no counterpart in the reference). qlmx_moe_gemm_nt on bf16 operands computes 256 x 128 output
- * tiles; a 256 x 256 variant (one workgroup per CU, accumulators in the second half of the register file) exists and
+ * tiles; a 256 x 256 variant (one workgroup of eight wavefronts per CU) exists and
  * is correct but not faster on MI355X, so it is never chosen by itself. tile = 256 selects it for later calls whose
  * column count is a multiple of 256, tile = 128 goes back; QLMX_NT_TILE=256 in the environment is the same switch
  * from outside the process. */

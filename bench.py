@@ -41,9 +41,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--fwd-math", default="f16", choices=["f16", "bf16x2"],
                     help="train, c5: forward GEMMs on the fp16 matrix core (one MFMA per product, 2e-4 relative L2) or as bf16 hi+lo (two, 3e-6)")
-    ap.add_argument("--bwd-streams", type=int, default=None, choices=[1, 2],
-                    help="2 = the weight gradient of every backward flush on the library's side stream beside its input gradient, 1 = one after the other; "
-                         "default: 2 for the config-3 step (+3.6 %%), 1 for config 5 (no gain at its size)")
+    ap.add_argument("--bwd", default="pair", choices=["pair", "serial", "streams"],
+                    help="train, c5: the two grouped GEMMs of every backward flush as one launch (qlmx_pair_begin / qlmx_pair_end), "
+                         "one after the other, or the weight gradient on the library's side stream beside the input gradient")
     ap.add_argument("--step-only", action="store_true", help="train: skip the per-launch repetitions, so that a kernel trace holds nothing but steps")
     ap.add_argument("--adamw-weights", type=int, default=120 * 2 ** 20)
     ap.add_argument("--render-p", type=int, default=0, help="adamw: also write the fp32 view P (4 B/weight more)")
@@ -172,7 +172,7 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
         for _, fn, _n in calls:
             fn()
 
-    if (args.bwd_streams or 2) == 2:
+    if args.bwd == "streams":
         # each backward flush (cudalm.cu:4333-4335, 4362-4366) with its weight gradient on the library's side
         # stream beside its input gradient: they read the same operands and write different outputs
         side = mk(q.side_fork(stream)); q.side_join(stream)      # the handle is the same at every fork
@@ -181,6 +181,12 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
             calls[0][1](); calls[1][1]()
             q.side_fork(stream); side[2][1](); calls[3][1](); q.side_join(stream)
             q.side_fork(stream); side[4][1](); calls[5][1](); q.side_join(stream)
+    elif args.bwd == "pair":
+        # each backward flush as one launch: the tiles of its weight gradient and of its input gradient in one grid
+        def step():
+            calls[0][1](); calls[1][1]()
+            q.pair_begin(stream); calls[2][1](); calls[3][1](); q.pair_end(stream)
+            q.pair_begin(stream); calls[4][1](); calls[5][1](); q.pair_end(stream)
 
     tm = timed(torch, step, args.steps, args.warmup)
     spread = step_spread(torch, step, args.steps)
@@ -202,14 +208,16 @@ def bench_train(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2, label=
     dom = max(per, key=lambda k: per[k]["ms"]) if per else "not timed"
     return {
         "workload": "%s: E=%d top-%d D=%d F=%d, %d bf16 tokens -> %d expert rows, Zipf(1.1) load (max %d, min %d rows); "
-                    "fwd+dgrad+wgrad = 9 grouped GEMMs in 6 launches%s" % (label, E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min()),
-                       ", the weight gradient of each backward flush on a second stream beside its input gradient" if (args.bwd_streams or 2) == 2 else ""),
-        "bwd_streams": args.bwd_streams or 2,
+                    "fwd+dgrad+wgrad = 9 grouped GEMMs in %s" % (label, E, topk, D, F, tokens, rows, int(cnt.max()), int(cnt.min()),
+                       {"pair": "4 launches (each backward flush -- weight gradient and input gradient of the same operands -- is one grid)",
+                        "streams": "6 launches, the weight gradient of each backward flush on a second stream beside its input gradient",
+                        "serial": "6 launches"}[args.bwd]),
+        "bwd": args.bwd,
         "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tm["wall_ms"],
         "dtype": "bf16" if args.fwd_math == "bf16x2" else "bf16 (fwd: fp16 MFMA)",
         "kernel_ms": tm, "step_ms_spread": spread, "per_launch": per, "beside_the_step": extra, "gflop_per_step": flops / 1e9,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "kernel": "k_gemm_nn_h, k_gemm_tn_lds, k_gemm_nt_lds (all 6 launches; slowest: %s)" % dom,
+                     "traffic": None, "kernel": "k_gemm_nn_h, k_gemm_tn_lds, k_gemm_nt_lds (every launch of the step; slowest on its own: %s)" % dom,
                      "note": "algorithmic flops only; forward math: " + ("bf16 hi+lo weight split, two MFMAs per product" if args.fwd_math == "bf16x2" else
                              "fp16 matrix core, bf16 activations converted exactly, weights rounded once to fp16 (2e-4 relative L2), one MFMA per product")},
     }
@@ -329,19 +337,20 @@ def bench_layer(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2):
             q.gemm_nn(d, s, group, T["w2"], E, F, D, ACT_BF16, MATH_MFMA_F16, stream)
             if merged: q.moe_dgate_merged(dout, yp, L.perm, gate, dgate, dyp, N, K, D, ACT_BF16, stream)
             else:      q.moe_dgate(dout, yp, tok, gk, dgate[k * N:(k + 1) * N], dyp, N, D, ACT_BF16, stream)
+            # each backward flush (weight gradient + input gradient of the same operands) is one grid
+            q.pair_begin(stream)
             q.gemm_nt(T["g2"], E, F, D, ACT_BF16, MATH_MFMA, stream)
             if fused: q.gemm_tn_swiglu_bwd(d, s, group, T["d2s"], E, D, F, gp, up, dgp, dup, stream)
-            else:
-                q.gemm_tn(d, s, group, T["d2"], E, D, F, ACT_BF16, MATH_MFMA, stream)
-                q.swiglu_bwd(gp, up, dap, dgp, dup, R * F, ACT_BF16, stream)
+            else:     q.gemm_tn(d, s, group, T["d2"], E, D, F, ACT_BF16, MATH_MFMA, stream)
+            q.pair_end(stream)
+            if not fused: q.swiglu_bwd(gp, up, dap, dgp, dup, R * F, ACT_BF16, stream)
+            q.pair_begin(stream)
             q.gemm_nt(T["g13"], 2 * E, D, F, ACT_BF16, MATH_MFMA, stream)
-            if merged:
-                q.gemm_tn_pair(d, s, group, T["d1"], T["d3"], E, F, D, ACT_BF16, MATH_MFMA, stream)
-                q.moe_combine(dXp, L.inv, None, dx, N, K, D, stream)
-            elif fused: q.gemm_tn_pair_scatter(d, s, group, T["d1s"], T["d3s"], E, F, D, dx, stream)
-            else:
-                q.gemm_tn_pair(d, s, group, T["d1"], T["d3"], E, F, D, ACT_BF16, MATH_MFMA, stream)
-                q.moe_scatter_add(dXp, tok, dx, N, D, stream)
+            if fused and not merged: q.gemm_tn_pair_scatter(d, s, group, T["d1s"], T["d3s"], E, F, D, dx, stream)
+            else:                    q.gemm_tn_pair(d, s, group, T["d1"], T["d3"], E, F, D, ACT_BF16, MATH_MFMA, stream)
+            q.pair_end(stream)
+            if merged:      q.moe_combine(dXp, L.inv, None, dx, N, K, D, stream)
+            elif not fused: q.moe_scatter_add(dXp, tok, dx, N, D, stream)
 
     steps, warmup = max(5, args.steps // 4), max(2, args.warmup // 4)
     per_pass, one_list = Lists(False), Lists(True)
@@ -448,7 +457,7 @@ def bench_c5(torch, q, args, L=8, E=64, D=2048, F=1408, tokens=32768, topk=4):
             (lambda: q.gemm_tn_pair(d, s, group, p_d1, p_d3, E, F, D, ACT_BF16, MATH_MFMA, st)),
         ])
     main_calls = [mk(stream) for mk in calls]
-    if (args.bwd_streams or 1) == 2:
+    if args.bwd == "streams":
         side_st = q.side_fork(stream); q.side_join(stream)       # the handle is the same at every fork
         side_calls = [mk(side_st) for mk in calls]
 
@@ -458,6 +467,12 @@ def bench_c5(torch, q, args, L=8, E=64, D=2048, F=1408, tokens=32768, topk=4):
                 m[0](); m[1]()
                 q.side_fork(stream); sd[2](); m[3](); q.side_join(stream)
                 q.side_fork(stream); sd[4](); m[5](); q.side_join(stream)
+    elif args.bwd == "pair":
+        def gemms():
+            for m in main_calls:
+                m[0](); m[1]()
+                q.pair_begin(stream); m[2](); m[3](); q.pair_end(stream)
+                q.pair_begin(stream); m[4](); m[5](); q.pair_end(stream)
     else:
         def gemms():
             for m in main_calls:

@@ -60,6 +60,8 @@ SIGNATURES = {
     "qlmx_sync": (c_i, [c_vp]),
     "qlmx_side_fork": (c_i, [c_vp, C.POINTER(c_vp)]),
     "qlmx_side_join": (c_i, [c_vp]),
+    "qlmx_pair_begin": (c_i, [c_vp]),
+    "qlmx_pair_end": (c_i, [c_vp]),
     "qlmx_qhashu": (C.c_uint, [c_u64]),
     "qlmx_qsri": (c_i, [c_f, c_u64, c_u64]),
     "qlmx_qclmp": (c_i, [c_i, c_i, c_i]),
@@ -279,6 +281,14 @@ class Qlmx:
 
     def side_join(self, stream=None):
         self.call("qlmx_side_join", stream)
+
+    def pair_begin(self, stream=None):
+        """Hold back the next input-gradient and weight-gradient launches on `stream` (qlmx_pair_begin)."""
+        self.call("qlmx_pair_begin", stream)
+
+    def pair_end(self, stream=None):
+        """Issue what qlmx_pair_begin held back, as one launch when both kinds are there."""
+        self.call("qlmx_pair_end", stream)
 
 
 _cached = None

@@ -26,7 +26,7 @@ HOST_LIB = os.path.join(HERE, "libqlmx_host.so")
 ARCH = "gfx950"
 
 HIP_SOURCES = ["qlmx_runtime.hip", "qlmx_step.hip", "qlmx_codec.hip", "qlmx_gemm_common.hip",
-               "qlmx_gemm_f32.hip", "qlmx_gemm_mfma.hip", "qlmx_gemm_nt_lds.hip", "qlmx_gemm_tn_lds.hip", "qlmx_gemm_nn_lds.hip", "qlmx_gemm_nn_h.hip", "qlmx_gemv.hip", "qlmx_gemm_api.hip", "qlmx_glue.hip", "qlmx_q4n.hip"]
+               "qlmx_gemm_f32.hip", "qlmx_gemm_mfma.hip", "qlmx_gemm_nt_lds.hip", "qlmx_gemm_tn_lds.hip", "qlmx_gemm_bwd.hip", "qlmx_gemm_nn_lds.hip", "qlmx_gemm_nn_h.hip", "qlmx_gemv.hip", "qlmx_gemm_api.hip", "qlmx_glue.hip", "qlmx_q4n.hip"]
 HIP_FLAGS = ["-O3", "--offload-arch=" + ARCH, "-std=c++17", "-fPIC", "-ffp-contract=off",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]   # = PK_FLAGS, spelled out
 

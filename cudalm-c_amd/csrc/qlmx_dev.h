@@ -11,6 +11,8 @@
 void qlmx_set_error(const char *fmt, ...);
 int qlmx_cu_count(void);
 int  qlmx_check_ready(void);
+int  qlmx_check_ready_keep(void);        /* the same without issuing what an open pair holds */
+int  qlmx_pair_flush(void);              /* issues the launches held back for a pair, if any */
 int  qlmx_decode_setup(int device);   /* per-device state of the decode entry points; qlmx_init calls it */
 #define QLMX_HIP(call, what)                                                                  \
     do { hipError_t e_ = (call);                                                              \

@@ -13,7 +13,10 @@ int qlmx_gemm_mfma_dispatch(int mode, const signed char *d, const float *s, int 
 static int gemm_entry(const char *who, int mode, const signed char *d, const float *s, int group,
                       const qlmx_gemm_prob *probs, int nprob, int K, int N, int act_dtype, int math, void *stream,
                       const qlmx_gemm_prob *second = nullptr){
-    int rc = qlmx_check_ready(); if(rc) return rc;
+    /* an input or weight gradient on bf16 operands can wait for its partner in an open pair; every other call
+     * first issues what such a pair holds, so that the stream keeps the order of the calls */
+    const bool pairable = mode != GEMM_NN && act_dtype == QLMX_ACT_BF16 && math != QLMX_MATH_F32;
+    int rc = pairable ? qlmx_check_ready_keep() : qlmx_check_ready(); if(rc) return rc;
     QLMX_REQUIRE(K > 0 && N > 0, "%s: K=%d N=%d", who, K, N);
     QLMX_REQUIRE(act_dtype == QLMX_ACT_F32 || act_dtype == QLMX_ACT_BF16, "%s: act_dtype %d", who, act_dtype);
     QLMX_REQUIRE(math == QLMX_MATH_F32 || math == QLMX_MATH_MFMA || math == QLMX_MATH_MFMA_F16, "%s: math %d", who, math);
@@ -126,8 +129,8 @@ int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, con
                             const float *gp, const float *up_, void *dg, void *du, hipStream_t st);
 
 static int rows_entry_checks(const char *who, const signed char *d, const float *s, int group, const qlmx_gemm_prob *probs,
-                             const qlmx_gemm_prob *second, int nprob, int K, int N, int bk, bool idx_in_a){
-    int rc = qlmx_check_ready(); if(rc) return rc;
+                             const qlmx_gemm_prob *second, int nprob, int K, int N, int bk, bool idx_in_a, bool pairable = false){
+    int rc = pairable ? qlmx_check_ready_keep() : qlmx_check_ready(); if(rc) return rc;
     QLMX_REQUIRE(d && s && probs && nprob >= 0 && K > 0 && N > 0, "%s: NULL or empty argument", who);
     QLMX_REQUIRE(((uintptr_t)d & 15) == 0, "%s: digit array is not 16-byte aligned", who);
     QLMX_REQUIRE(N % 128 == 0 && K % bk == 0, "%s: N=%d must be a multiple of 128 and K=%d of %d", who, N, K, bk);
@@ -192,7 +195,7 @@ extern "C" int qlmx_moe_gemm_nn_scatter(const signed char *d, const float *s, in
 extern "C" int qlmx_moe_gemm_tn_pair_scatter(const signed char *d, const float *s, int group,
                                              const qlmx_gemm_prob *first, const qlmx_gemm_prob *second, int nprob, int K, int N,
                                              float *dst, void *stream){
-    int rc = rows_entry_checks("qlmx_moe_gemm_tn_pair_scatter", d, s, group, first, second, nprob, K, N, 64, false); if(rc) return rc;
+    int rc = rows_entry_checks("qlmx_moe_gemm_tn_pair_scatter", d, s, group, first, second, nprob, K, N, 64, false, true); if(rc) return rc;
     QLMX_REQUIRE(dst && second && nprob * 2 <= QLMX_MAX_PROBLEMS, "qlmx_moe_gemm_tn_pair_scatter: NULL output or too many problems");
     return qlmx_gemm_tn_lds_launch(d, s, group, first, second, nprob, K, N, dst, nullptr, nullptr, nullptr, nullptr, nullptr, (hipStream_t)stream);
 }
@@ -205,7 +208,7 @@ extern "C" int qlmx_moe_gemm_tn_pair_scatter(const signed char *d, const float *
 extern "C" int qlmx_moe_gemm_tn_swiglu_bwd(const signed char *d, const float *s, int group,
                                            const qlmx_gemm_prob *probs, int nprob, int K, int N,
                                            const float *gp, const float *up, void *dgp, void *dup, void *stream){
-    int rc = rows_entry_checks("qlmx_moe_gemm_tn_swiglu_bwd", d, s, group, probs, nullptr, nprob, K, N, 64, false); if(rc) return rc;
+    int rc = rows_entry_checks("qlmx_moe_gemm_tn_swiglu_bwd", d, s, group, probs, nullptr, nprob, K, N, 64, false, true); if(rc) return rc;
     QLMX_REQUIRE(gp && up && dgp && dup && (((uintptr_t)gp | (uintptr_t)up | (uintptr_t)dgp | (uintptr_t)dup) & 3) == 0, "qlmx_moe_gemm_tn_swiglu_bwd: NULL or misaligned buffer");
     for(int i = 0; i < nprob; i++)
         QLMX_REQUIRE(probs[i].M == 0 || (probs[i].C >= gp && (probs[i].C - gp) % 2 == 0), "qlmx_moe_gemm_tn_swiglu_bwd: problem %d: C must point into gp at an even element", i);

@@ -47,7 +47,10 @@ static int guard_take(RingGuard &g, int *slot_out){
     const int slot = g.next; g.next = (g.next + 1) % g.nslots;
     if(slot % g.per_seg == 0){
         const int nseg = g.nslots / g.per_seg, cur = slot / g.per_seg;
-        int rc = guard_close(g.seg[(cur + nseg - 1) % nseg]); if(rc) return rc;
+        /* a launch held back for a pair owns a slot of the segment that is closed here: issue it first, so
+         * that the segment's events come after it */
+        int rc = qlmx_pair_flush(); if(rc) return rc;
+        rc = guard_close(g.seg[(cur + nseg - 1) % nseg]); if(rc) return rc;
         RingSeg &sg = g.seg[cur];
         for(int i = 0; i < sg.nrec; i++) QLMX_HIP(hipEventSynchronize(sg.ev[i]), "table ring wait");
         sg.nrec = 0;

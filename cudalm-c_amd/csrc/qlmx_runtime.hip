@@ -16,10 +16,18 @@ void qlmx_set_error(const char *fmt, ...){
     vsnprintf(g_err, sizeof g_err, fmt, ap);
     va_end(ap);
 }
-int qlmx_check_ready(void){
+int qlmx_check_ready_keep(void){
     if(g_ready) return QLMX_OK;
     qlmx_set_error("libqlmx: qlmx_init() has not succeeded (no gfx950 device bound)");
     return QLMX_E_NODEV;
+}
+/* Every entry point that queues work starts here. Launches held back for a pair (qlmx_pair_begin) are issued
+ * first, so that whatever this call queues comes after them on the stream; the two kinds of call that can be
+ * held themselves use qlmx_check_ready_keep. */
+int qlmx_pair_flush(void);
+int qlmx_check_ready(void){
+    const int rc = qlmx_check_ready_keep(); if(rc) return rc;
+    return qlmx_pair_flush();
 }
 
 static int g_cus = 256;
@@ -57,15 +65,21 @@ extern "C" int qlmx_malloc(void **p, size_t bytes){
     return QLMX_OK;
 }
 extern "C" int qlmx_free(void *p){ QLMX_HIP(hipFree(p), "hipFree"); return QLMX_OK; }
+/* copies, fills and waits come after what an open pair holds, like every call that queues work */
 extern "C" int qlmx_memcpy_h2d(void *dst, const void *src, size_t bytes){
+    int rc = qlmx_pair_flush(); if(rc) return rc;
     QLMX_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice), "hipMemcpy h2d"); return QLMX_OK; }
 extern "C" int qlmx_memcpy_d2h(void *dst, const void *src, size_t bytes){
+    int rc = qlmx_pair_flush(); if(rc) return rc;
     QLMX_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost), "hipMemcpy d2h"); return QLMX_OK; }
 extern "C" int qlmx_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream){
+    int rc = qlmx_pair_flush(); if(rc) return rc;
     QLMX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream), "hipMemcpy d2d"); return QLMX_OK; }
 extern "C" int qlmx_memset(void *dst, int value, size_t bytes, void *stream){
+    int rc = qlmx_pair_flush(); if(rc) return rc;
     QLMX_HIP(hipMemsetAsync(dst, value, bytes, (hipStream_t)stream), "hipMemset"); return QLMX_OK; }
 extern "C" int qlmx_sync(void *stream){
+    int rc = qlmx_pair_flush(); if(rc) return rc;
     if(stream) QLMX_HIP(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
     else       QLMX_HIP(hipDeviceSynchronize(), "hipDeviceSynchronize");
     return QLMX_OK;

@@ -493,11 +493,12 @@ static void mg_run_pairs(void){
     v0.swap(r0); v1.swap(r1);
 }
 /* The problems of a flush do not depend on each other except queue 1 on queue 0 (it accumulates into what queue 0
- * writes). The weight gradients (queue 2) of a flush that also holds input gradients run on the library's side
- * stream beside them: neither fills the device to the end of its last round of tiles. */
+ * writes). The weight gradients (queue 2) of a flush that also holds input gradients go into one grid with the
+ * first input-gradient launch (qlmx_pair_begin / qlmx_pair_end): neither fills the device to the end of its last
+ * round of tiles, and in one grid the one's tiles take the compute units the other leaves. */
 static bool q2_reads_what_the_flush_writes(void){
     /* the reference issues queue 0, 1, 2 in order on one stream (cudalm.cu:3243), so there a weight-gradient
-     * problem may read an output of the same flush; side by side that would race, so such a flush runs in order */
+     * problem may read an output of the same flush; in one grid that would race, so such a flush runs in order */
     const size_t asz = g_mg_act == QLMX_ACT_BF16 ? 2 : 4;
     auto overlaps = [](const void *p, size_t n, const void *q, size_t m){
         const uintptr_t a = (uintptr_t)p, b = (uintptr_t)q;
@@ -514,11 +515,10 @@ static bool q2_reads_what_the_flush_writes(void){
 }
 void mg_flush(void){
     mg_run_dual();
-    void *side = NULL;
-    const bool beside = !g_q[2].empty() && (!g_q[0].empty() || !g_q[1].empty()) && !q2_reads_what_the_flush_writes()
-                     && qlmx_side_fork(NULL, &side) == QLMX_OK;
-    if(beside) mg_run(g_q[2], side);
+    const bool paired = !g_q[2].empty() && (!g_q[0].empty() || !g_q[1].empty()) && !q2_reads_what_the_flush_writes();
+    if(paired && qlmx_pair_begin(NULL) != QLMX_OK){ fprintf(stderr, "mg_flush: %s\n", qlmx_last_error()); exit(1); }
+    if(paired) mg_run(g_q[2]);                 /* held; leaves with the first input-gradient launch */
     mg_run_pairs(); mg_run(g_q[0]); mg_run(g_q[1]);
-    if(beside){ if(qlmx_side_join(NULL) != QLMX_OK){ fprintf(stderr, "mg_flush: %s\n", qlmx_last_error()); exit(1); } }
+    if(paired){ if(qlmx_pair_end(NULL) != QLMX_OK){ fprintf(stderr, "mg_flush: %s\n", qlmx_last_error()); exit(1); } }
     else mg_run(g_q[2]);
 }

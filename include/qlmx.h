@@ -10,7 +10,7 @@
  * library keeps process-wide state -- the table rings of the grouped GEMMs and their staging copies, the chain flags
  * of split contractions, the partial sums of qlmx_sqsum, the decode workspace -- so calls must come from one host
  * thread, and calls whose kernels could overlap on different streams are not supported, except the documented
- * pairing of qlmx_side_fork / qlmx_side_join.
+ * pairing of qlmx_side_fork / qlmx_side_join (qlmx_pair_begin / qlmx_pair_end runs the two on one stream).
  * Every function returns 0 on success and a
  * negative QLMX_E_* code on failure; qlmx_last_error() holds the message of the calling thread's
  * last failure. The reference's print-and-exit(1) behaviour (ck/ckb, cudalm.cu:147-152) is kept by
@@ -67,6 +67,20 @@ int         qlmx_sync(void *stream);
  * capture. */
 int         qlmx_side_fork(void *stream, void **side);
 int         qlmx_side_join(void *stream);
+/* The two grouped GEMMs of a backward flush as ONE kernel launch (no counterpart in the reference, which issues
+ * them one after the other, cudalm.cu:3243-3256). Between qlmx_pair_begin(stream) and qlmx_pair_end(stream) the
+ * library holds back at most one input-gradient launch (qlmx_moe_gemm_tn, _tn_pair, _tn_pair_scatter,
+ * _tn_swiglu_bwd) and one weight-gradient launch (qlmx_moe_gemm_nt), both on bf16 operands with MFMA math and
+ * queued on `stream`, and qlmx_pair_end issues them as one grid: the workgroups of the one kernel first, those of
+ * the other behind them, each tile computed exactly as in its own launch (bit-identical results), so the second
+ * kind's tiles take the compute units as the first kind's last round leaves them -- without the wait between
+ * hardware queues that the side stream costs at its fork and join. The caller promises what it promises for the
+ * side stream: neither of the two reads what the other writes. Everything else keeps its order on the stream:
+ * a second launch of a kind already held, a launch of a shape the two direct-to-LDS kernels do not take, and any
+ * other library call that queues work first issue what is held. One pair at a time; not for use across host
+ * synchronisation (nothing held runs before qlmx_pair_end or one of the calls just named). */
+int         qlmx_pair_begin(void *stream);
+int         qlmx_pair_end(void *stream);
 
 /* ---- host integer helpers: the __host__ __device__ inlines of qlm.cuh:78-111, used by the
  *      reference's checkpoint code and selftest reference (cudalm.cu:10574-10580) ---- */

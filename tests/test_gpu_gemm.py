@@ -591,3 +591,75 @@ def test_side_stream_fork_join(q, orc):
         torch.cuda.synchronize()
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
     assert float(outs[0][1].abs().max()) > 0.0
+
+
+def test_backward_pair_is_one_launch_with_the_same_bits(q, orc):
+    """qlmx_pair_begin / qlmx_pair_end: the input gradient and the weight gradient of a flush held back and issued as
+    one grid give the bits of the two launches one after the other -- plain, with a sliced weight-gradient contraction
+    (chain flags inside the combined grid), with the continued input gradient -- and everything else keeps its order
+    on the stream: a second launch of a held kind, a copy queued between the two, the end without a partner."""
+    import torch
+    cur = torch.cuda.current_stream().cuda_stream
+    for (E, rows, K, N, seed, paired) in [(6, [700, 33, 0, 1290, 256, 64], 256, 512, 17, False),
+                                         (5, [9000, 12, 300, 0, 129], 256, 384, 18, False),
+                                         (4, [513, 64, 1, 2000], 384, 256, 19, True)]:
+        tot = sum(rows); off = np.concatenate([[0], np.cumsum(rows)]).astype(int)
+        d, s, P = make_weights(orc, seed, 2 * E, K, N, 128)      # forward weights [K, N] per expert; dX[rows, K] = dY[rows, N] . W^T
+        dY = orc.bf16_round(orc.normal(tot * N, seed, 10)); dY2 = orc.bf16_round(orc.normal(tot * N, seed, 13)); X = orc.bf16_round(orc.normal(tot * K, seed, 11))
+        dYb, dY2b, Xb = to_bf16_bits(dev(dY)), to_bf16_bits(dev(dY2)), to_bf16_bits(dev(X))
+        dd, ds = dev(d), dev(s)
+        outs = []
+        for pair in (False, True):
+            G = dev(orc.normal(E * K * N, seed, 12, 0.1)); dX = torch.zeros(tot * K, device="cuda")
+            nt = q.problems([(Xb.data_ptr() + off[e] * K * 2, dYb.data_ptr() + off[e] * N * 2, G.data_ptr() + e * K * N * 4, 0, 0, rows[e], 1.0) for e in range(E)])
+            tn = q.problems([(dYb.data_ptr() + off[e] * N * 2, None, dX.data_ptr() + off[e] * K * 4, e * N * K, e * N * K // 128, rows[e], 0.0) for e in range(E)])
+            tn2 = q.problems([(dY2b.data_ptr() + off[e] * N * 2, None, dX.data_ptr() + off[e] * K * 4, (E + e) * N * K, (E + e) * N * K // 128, rows[e], 0.0) for e in range(E)])
+            if pair:
+                q.pair_begin(cur)
+            q.gemm_nt(nt, E, K, N, pkg.ACT_BF16, pkg.MATH_MFMA, cur)
+            if paired:
+                q.gemm_tn_pair(dd, ds, 128, tn, tn2, E, N, K, pkg.ACT_BF16, pkg.MATH_MFMA, cur)
+            else:
+                q.gemm_tn(dd, ds, 128, tn, E, N, K, pkg.ACT_BF16, pkg.MATH_MFMA, cur)
+            if pair:
+                q.pair_end(cur)
+            outs.append((G.clone(), dX.clone()))
+            torch.cuda.synchronize()
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1]), (E, rows)
+        assert float(outs[0][1].abs().max()) > 0.0 and float((outs[0][0] - dev(orc.normal(E * K * N, seed, 12, 0.1))).abs().max()) > 0.0
+    # order: dX = dY . W1^T, then dX += dY2 . W2^T (second launch of the held kind), a copy of dX queued before the end,
+    # and a weight gradient that finds no partner at the end
+    E, rows, K, N, seed = 3, [300, 70, 1025], 256, 256, 23
+    tot = sum(rows); off = np.concatenate([[0], np.cumsum(rows)]).astype(int)
+    d, s, P = make_weights(orc, seed, 2 * E, K, N, 128)
+    dYb = to_bf16_bits(dev(orc.bf16_round(orc.normal(tot * N, seed, 10)))); dY2b = to_bf16_bits(dev(orc.bf16_round(orc.normal(tot * N, seed, 13))))
+    Xb = to_bf16_bits(dev(orc.bf16_round(orc.normal(tot * K, seed, 11))))
+    dd, ds = dev(d), dev(s)
+    res = []
+    for pair in (False, True):
+        G = torch.zeros(E * K * N, device="cuda"); dX = torch.zeros(tot * K, device="cuda"); snap = torch.zeros(tot * K, device="cuda")
+        nt = q.problems([(Xb.data_ptr() + off[e] * K * 2, dYb.data_ptr() + off[e] * N * 2, G.data_ptr() + e * K * N * 4, 0, 0, rows[e], 0.0) for e in range(E)])
+        t1 = q.problems([(dYb.data_ptr() + off[e] * N * 2, None, dX.data_ptr() + off[e] * K * 4, e * N * K, e * N * K // 128, rows[e], 0.0) for e in range(E)])
+        t2 = q.problems([(dY2b.data_ptr() + off[e] * N * 2, None, dX.data_ptr() + off[e] * K * 4, (E + e) * N * K, (E + e) * N * K // 128, rows[e], 1.0) for e in range(E)])
+        if pair:
+            q.pair_begin(cur)
+        q.gemm_tn(dd, ds, 128, t1, E, N, K, pkg.ACT_BF16, pkg.MATH_MFMA, cur)
+        q.gemm_tn(dd, ds, 128, t2, E, N, K, pkg.ACT_BF16, pkg.MATH_MFMA, cur)          # issues t1, is held itself
+        q.call("qlmx_memcpy_d2d", snap, dX, tot * K * 4, cur)                           # issues t2
+        q.gemm_nt(nt, E, K, N, pkg.ACT_BF16, pkg.MATH_MFMA, cur)                        # held, no partner
+        if pair:
+            q.pair_end(cur)
+        torch.cuda.synchronize()
+        res.append((G.clone(), dX.clone(), snap.clone()))
+    for a, b in zip(res[0], res[1]):
+        assert torch.equal(a, b)
+    assert torch.equal(res[1][1], res[1][2]) and float(res[1][0].abs().max()) > 0.0
+    # misuse
+    with pytest.raises(pkg.QlmxError, match="no pair is open"):
+        q.pair_end(cur)
+    q.pair_begin(cur)
+    try:
+        with pytest.raises(pkg.QlmxError, match="already open"):
+            q.pair_begin(cur)
+    finally:
+        q.pair_end(cur)

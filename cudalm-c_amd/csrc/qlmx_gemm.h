@@ -65,16 +65,18 @@ __device__ __forceinline__ int qx_xcd_tile(int b, int grid){
 }
 
 /* Tile of workgroup b for a table whose first nfull tiles are whole-height ones and whose remaining tiles are the
- * problems' last row tiles, tallest first: XCD x takes the x-th contiguous eighth of the first part (tiles that share
- * an expert's rows and weights meet in one L2), then every eighth tile of the second part, so that all XCDs run out
- * of whole tiles and then of tall last tiles at about the same time. 0x7FFFFFFF = no tile. */
-__device__ __forceinline__ int qx_lpt_tile(int b, int nfull, int ntiles){
+ * problems' last row tiles, tallest first, g tiles (one tile row) each: XCD x takes the x-th contiguous eighth of the
+ * first part (tiles that share an expert's rows and weights meet in one L2), then every eighth tile ROW of the second
+ * part -- a row's g tiles read the same activation rows, so they stay on one XCD -- so that all XCDs run out of
+ * whole tiles and then of tall last tiles at about the same time. 0x7FFFFFFF = no tile. */
+__device__ __forceinline__ int qx_lpt_tile(int b, int nfull, int ntiles, int g){
     const int x = b & 7, k = b >> 3, per = (nfull + 7) >> 3;
     if(k < per){ const int t = x * per + k; return t < nfull ? t : 0x7FFFFFFF; }
-    const int t = nfull + (k - per) * 8 + x;
+    const int k2 = k - per, r = k2 / g;
+    const int t = nfull + (r * 8 + x) * g + (k2 - r * g);
     return t < ntiles ? t : 0x7FFFFFFF;
 }
-static inline int qx_lpt_grid(int nfull, int ntiles){ return 8 * ((nfull + 7) / 8 + (ntiles - nfull + 7) / 8); }
+static inline int qx_lpt_grid(int nfull, int ntiles, int g){ return 8 * ((nfull + 7) / 8 + g * (((ntiles - nfull) / g + 7) / 8)); }
 
 /* Weight gradients (tile cost = the expert's row count): every problem owns rp rows of g tiles; a
  * row shares the A-side slab (activations), a column the B-side slab (output gradients).

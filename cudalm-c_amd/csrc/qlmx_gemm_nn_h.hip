@@ -47,7 +47,7 @@ typedef int      i32x4 __attribute__((ext_vector_type(4)));
  *               points at its row indices, out[idx[r], :] = out[idx[r], :] + gate[idx[r]] * y[r, :] (gate NULL: + y[r, :]),
  *               rows with idx[r] < 0 dropped. Within one launch every output row must be named at most once. */
 enum { NH_PLAIN = 0, NH_GATHER = 1, NH_SCATTER = 2 };
-struct NhArgs { const DevProb *pr; int nprob, ntiles, nfull; const signed char *d; const float *s; int gshift; int K, N;
+struct NhArgs { const DevProb *pr; int nprob, ntiles, nfull, tiles_n; const signed char *d; const float *s; int gshift; int K, N;
                 const char *xsrc; float *out; const float *gate; };
 
 /* a row of zeros as long as the longest contraction a gathering launch accepts: what a dropped row reads */
@@ -301,7 +301,7 @@ __device__ __forceinline__ void nh_tile(const NhArgs &a, const DevProb &P, const
 template<int IO>
 __global__ void __launch_bounds__(256, 2) k_gemm_nn_h(NhArgs a){
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * NH_A_BYTES + 2 * NH_B_BYTES];
-    const int t = qx_lpt_tile(blockIdx.x, a.nfull, a.ntiles);
+    const int t = qx_lpt_tile(blockIdx.x, a.nfull, a.ntiles, a.tiles_n);
     if(t >= a.ntiles) return;
     const DevProb P = a.pr[qx_find_problem(a.pr, a.nprob, t)];
     const int lt = t - P.tile0;
@@ -320,7 +320,7 @@ __global__ void __launch_bounds__(256, 2) k_gemm_nn_h(NhArgs a){
 template<int IO>
 __global__ void __launch_bounds__(256, 2) k_gemm_nn_h_swiglu(NhArgs a){
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * NH_A_BYTES + 2 * NH_B_BYTES];
-    const int t = qx_lpt_tile(blockIdx.x, a.nfull, a.ntiles);
+    const int t = qx_lpt_tile(blockIdx.x, a.nfull, a.ntiles, a.tiles_n);
     if(t >= a.ntiles) return;
     const int pi = qx_find_problem(a.pr, a.nprob, t);
     const DevProb P = a.pr[pi];
@@ -345,10 +345,10 @@ int qlmx_gemm_nn_h_launch(const signed char *d, const float *s, int group, const
     const RowBytes rb = {io == NH_GATHER ? sizeof(int) : (size_t)K * 2, io == NH_SCATTER ? sizeof(int) : (size_t)N * 4, 0, 0, 0};
     int rc = qlmx_upload_problems_split(probs, nullptr, nprob, GEMM_NN, K, N, NH_BM, NH_BN, &rb, st, &up, &slot); if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;
-    NhArgs a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.nfull = up.nfull; a.d = d; a.s = s; a.K = K; a.N = N;
+    NhArgs a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.nfull = up.nfull; a.tiles_n = N / NH_BN; a.d = d; a.s = s; a.K = K; a.N = N;
     a.xsrc = (const char *)xsrc; a.out = out; a.gate = gate;
     a.gshift = 0; while((1 << a.gshift) < group) a.gshift++;
-    const int grid = qx_lpt_grid(up.nfull, up.ntiles);
+    const int grid = qx_lpt_grid(up.nfull, up.ntiles, a.tiles_n);
     if(io == NH_GATHER)       hipLaunchKernelGGL(k_gemm_nn_h<NH_GATHER>,  dim3(grid), dim3(256), 0, st, a);
     else if(io == NH_SCATTER) hipLaunchKernelGGL(k_gemm_nn_h<NH_SCATTER>, dim3(grid), dim3(256), 0, st, a);
     else                      hipLaunchKernelGGL(k_gemm_nn_h<NH_PLAIN>,   dim3(grid), dim3(256), 0, st, a);
@@ -366,10 +366,10 @@ int qlmx_gemm_nn_h_swiglu_launch(const signed char *d, const float *s, int group
     const RowBytes rb = {xsrc ? sizeof(int) : (size_t)K * 2, (size_t)N * 4, 0, (size_t)N * 2, (size_t)N * 4};
     int rc = qlmx_upload_problems_split(gate, up_, nprob, GEMM_NN, K, N, NH_BM, NH_BN / 2, &rb, st, &up, &slot); if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;
-    NhArgs a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.nfull = up.nfull; a.d = d; a.s = s; a.K = K; a.N = N;
+    NhArgs a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.nfull = up.nfull; a.tiles_n = N / (NH_BN / 2); a.d = d; a.s = s; a.K = K; a.N = N;
     a.xsrc = (const char *)xsrc; a.out = nullptr; a.gate = nullptr;
     a.gshift = 0; while((1 << a.gshift) < group) a.gshift++;
-    const int grid = qx_lpt_grid(up.nfull, up.ntiles);
+    const int grid = qx_lpt_grid(up.nfull, up.ntiles, a.tiles_n);
     if(xsrc) hipLaunchKernelGGL(k_gemm_nn_h_swiglu<NH_GATHER>, dim3(grid), dim3(256), 0, st, a);
     else     hipLaunchKernelGGL(k_gemm_nn_h_swiglu<NH_PLAIN>,  dim3(grid), dim3(256), 0, st, a);
     QLMX_LAUNCH_CHECK("grouped gemm nn + swiglu (fp16 matrix core) launch");

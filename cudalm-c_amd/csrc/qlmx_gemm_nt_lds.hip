@@ -19,7 +19,12 @@ static void *g_nt3_zeros = nullptr;
  * column tiles of one (problem, tile row, slice); XCD x runs its entries in order, g workgroups each.
  * Returns the grid size, or 0 when the launch does not fit the table. */
 struct Nt3Group { int prob, ti, cost; };
+/* whole problems up to num/den of an XCD's share (QLMX_NT_WHOLE = num, 0 = never). Config-3 step, reads of the two
+ * weight-gradient launches by FETCH_SIZE and their times: never 278 + 436 MiB, 77.7 + 140.6 us; 2/4 185 + 312 MiB,
+ * 82.6 + 137.8; 3/4 159 + 292 MiB, 75.1 + 136.2; 4/4 the same as 3/4 (no expert lies between). */
+static int g_nt3_whole_num = -1, g_nt3_whole_den = 4;
 static int nt3_schedule(DevProb *pr, int n, int K, int N, int BN, int slots_per_cu, int cus, DevUnit *units, int *nflags_out, int *nent_out){
+    if(g_nt3_whole_num < 0){ const char *e = getenv("QLMX_NT_WHOLE"); g_nt3_whole_num = e ? atoi(e) : 3; }
     const int g = N / BN, rp = (K + NT3_BM - 1) / NT3_BM;
     if(rp > 64) return 0;                                              /* the packed entry has 6 bits for the tile row */
     long long work = 0;
@@ -38,16 +43,22 @@ static int nt3_schedule(DevProb *pr, int n, int K, int N, int BN, int slots_per_
         nunits += (long long)nc * rp;
     }
     if(nunits + 8LL * 15 > QLMX_MAX_UNITS) return 0;
+    /* A problem whose whole cost is at most `whole` of an XCD's share stays on one XCD with all its tile rows
+     * (ti = -1): they read the same rows of dY, which then come from HBM once instead of once per tile row. */
     static Nt3Group groups[QLMX_MAX_UNITS];
     int ng = 0;
-    for(int p = 0; p < n; p++) for(int ti = 0; ti < rp; ti++) groups[ng++] = {p, ti, pr[p].M};
+    const long long share = (work + 7) / 8;
+    for(int p = 0; p < n; p++){
+        if(rp > 1 && (long long)pr[p].M * rp * g * g_nt3_whole_den <= share * g_nt3_whole_num) groups[ng++] = {p, -1, pr[p].M * rp};
+        else for(int ti = 0; ti < rp; ti++) groups[ng++] = {p, ti, pr[p].M};
+    }
     std::stable_sort(groups, groups + ng, [](const Nt3Group &x, const Nt3Group &y){ return x.cost > y.cost; });
     static int gx[QLMX_MAX_UNITS];
     long long load[8] = {0, 0, 0, 0, 0, 0, 0, 0}; int len[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     for(int i = 0; i < ng; i++){
         int x = 0;
         for(int y = 1; y < 8; y++) if(load[y] < load[x]) x = y;
-        gx[i] = x; load[x] += (long long)groups[i].cost * g; len[x] += nchunk[groups[i].prob];
+        gx[i] = x; load[x] += (long long)groups[i].cost * g; len[x] += nchunk[groups[i].prob] * (groups[i].ti < 0 ? rp : 1);
     }
     int longest = 0;
     for(int x = 0; x < 8; x++) if(len[x] > longest) longest = len[x];
@@ -62,7 +73,9 @@ static int nt3_schedule(DevProb *pr, int n, int K, int N, int BN, int slots_per_
     int pos[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     for(int i = 0; i < ng; i++){
         const int p = groups[i].prob, x = gx[i], nc = nchunk[p];
-        for(int c = 0; c < nc; c++) units[8 * pos[x]++ + x] = QX_UNIT(p, groups[i].ti, 0, c, nc);
+        const int t0 = groups[i].ti < 0 ? 0 : groups[i].ti, t1 = groups[i].ti < 0 ? rp : groups[i].ti + 1;
+        for(int c = 0; c < nc; c++)                                   /* a slice's tile rows side by side: they share its rows of dY */
+            for(int ti = t0; ti < t1; ti++) units[8 * pos[x]++ + x] = QX_UNIT(p, ti, 0, c, nc);
     }
     *nflags_out = nflags;
     *nent_out = nent;

@@ -51,7 +51,7 @@ struct Tn3Seg { int nseg; long long dA, dW, dS; };
  * (k_scatter_add4 behind the paired input-gradient GEMMs, cudalm.cu:4365-4367), see qx_scatter_tiles */
 /* gp != NULL: k_swiglu_bwd behind the down projection's input gradient (cudalm.cu:4340-4346): the product is d(act);
  * a problem's C field points at its rows of gp, and up, dg, du hold the same rows at the same element offset */
-struct Tn3Args { const DevProb *pr; int nprob, ntiles, nfull; const signed char *d; const float *s; int gshift; int K, N; float *out; const float *gate;
+struct Tn3Args { const DevProb *pr; int nprob, ntiles, nfull, tiles_n; const signed char *d; const float *s; int gshift; int K, N; float *out; const float *gate;
                  const float *gp, *up; unsigned short *dg, *du; };
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -319,7 +319,7 @@ __device__ __forceinline__ void tn3_tile(const Tn3Args &a, const DevProb &P, con
 
 /* one workgroup's tile; bid = its index in the launch */
 __device__ __forceinline__ void tn3_block(const Tn3Args &a, const unsigned bid, unsigned char *lds){
-    const int t = qx_lpt_tile(bid, a.nfull, a.ntiles);
+    const int t = qx_lpt_tile(bid, a.nfull, a.ntiles, a.tiles_n);
     if(t >= a.ntiles) return;
     const int pi = qx_find_problem(a.pr, a.nprob, t);
     const DevProb P = a.pr[pi];

@@ -31,10 +31,10 @@ int qlmx_gemm_tn_lds_launch(const signed char *d, const float *s, int group, con
     int rc = qlmx_upload_problems_split(probs, second, nprob, GEMM_TN, K, N, TN3_BM, TN3_BN, &rb, st, &up, &slot);
     if(rc) return rc;
     if(up.ntiles == 0) return QLMX_OK;
-    Tn3Args a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.nfull = up.nfull; a.d = d; a.s = s; a.K = K; a.N = N; a.out = out; a.gate = gate;
+    Tn3Args a; a.pr = up.dev; a.nprob = up.nprob; a.ntiles = up.ntiles; a.nfull = up.nfull; a.tiles_n = N / TN3_BN; a.d = d; a.s = s; a.K = K; a.N = N; a.out = out; a.gate = gate;
     a.gp = gp; a.up = up_; a.dg = (unsigned short *)dg; a.du = (unsigned short *)du;
     a.gshift = 0; while((1 << a.gshift) < group) a.gshift++;
-    const int grid = qx_lpt_grid(up.nfull, up.ntiles);
+    const int grid = qx_lpt_grid(up.nfull, up.ntiles, a.tiles_n);
     bool held;
     rc = qlmx_pair_hold_tn(a, grid, slot, st, &held); if(rc) return rc;
     return held ? QLMX_OK : qlmx_gemm_tn_lds_issue(a, grid, slot, st);

@@ -513,13 +513,16 @@ def bench_c5(torch, q, args, L=8, E=64, D=2048, F=1408, tokens=32768, topk=4):
     return {
         "workload": "C5 whole stack: %d layers x (E=%d top-%d D=%d F=%d), %d bf16 tokens -> %d expert rows per layer, Zipf(1.1) load per layer "
                     "(max/min rows %s); fwd+dgrad+wgrad = %d grouped GEMMs in %d launches, then one Integer AdamW step over %d weights"
-                    % (L, E, topk, D, F, tokens, rows, "/".join("%d:%d" % x for x in loads[:2]) + "...", 9 * L, 6 * L, nq),
-        "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tg["wall_ms"] + ta["wall_ms"], "dtype": "bf16",
+                    % (L, E, topk, D, F, tokens, rows, "/".join("%d:%d" % x for x in loads[:2]) + "...", 9 * L, (4 if args.bwd == "pair" else 6) * L, nq),
+        "bwd": args.bwd,
+        "metric": "QLM expert dequant-GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": tg["wall_ms"] + ta["wall_ms"],
+        "dtype": "bf16" if args.fwd_math == "bf16x2" else "bf16 (fwd: fp16 MFMA)",
         "steps": steps, "warmup": warmup,
         "gemm": {"ms": tg["event_ms_avg"], "tflops": tf, "tflop_per_step": flops / 1e12},
         "adamw": {"ms": ta["event_ms_avg"], "gbs": gbs, "weights": nq, "weights_per_s": nq / (ta["event_ms_avg"] * 1e-3), "bytes_per_weight": bytes_per_w},
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "kernel": "k_gemm_nn_lds, k_gemm_tn_lds, k_gemm_nt_lds (all %d launches)" % (6 * L)},
+                     "traffic": None, "kernel": "k_gemm_nn_h, k_gemm_tn_lds, k_gemm_nt_lds (all %d launches)" % ((4 if args.bwd == "pair" else 6) * L),
+                     "note": "the device holds 1.33-1.39 GHz under this load (profiles/k_gemm_lds_train_c5.txt); the peak is that of 2.4 GHz"},
         "roofline_adamw": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
                            "kernel": "k_qlmx_step<adam>, one launch over all %d weights" % nq},
     }
@@ -892,11 +895,12 @@ def cpu_decode(args, E=32, D=768, F=2048, topk=2, T=16, layers=2):
 
 # HBM bytes from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the 1 GiB copy calibration); the runs,
 # counter values and scale factors are in profiles/*.txt. adamw: per launch. train: per step, i.e. summed over
-# the step's 6 launches (1177 MiB read + 1086 MiB written). decode: per launch = per layer at T=16
-# (64.1 MiB read + 5.1 MiB written). The figures are constants of the code state they were measured at; that
-# state is named in the JSON line so that a reader can tell a stale one.
-PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.373e9, "decode": 7.39e7}
-PROFILED_AT = "git e24a32b (train), ef06021 (decode), 771b539 (adamw)"
+# the step's 4 launches (1035.9 MiB read + 1086.2 MiB written). c5: per step over the 32 GEMM launches of the 8
+# layers (104.4 GiB read + 49.0 GiB written). decode: per launch = per layer at T=16 (64.1 MiB read + 5.1 MiB
+# written). train and c5 are those of the default --bwd pair. The figures are constants of the code state they
+# were measured at; that state is named in the JSON line so that a reader can tell a stale one.
+PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.225e9, "c5": 1.648e11, "decode": 7.39e7}
+PROFILED_AT = "git bd3f2f6 (train, c5), ef06021 (decode), 87b8442 (adamw)"
 
 
 def main():
@@ -929,7 +933,8 @@ def main():
         "device": q.call("qlmx_device_name").decode(),
     }
     for w in results:
-        if results[w]["roofline"].get("traffic") is None and PROFILED_TRAFFIC.get(w) and not (w == "adamw" and args.render_p):
+        if results[w]["roofline"].get("traffic") is None and PROFILED_TRAFFIC.get(w) and not (w == "adamw" and args.render_p) \
+                and not (w in ("train", "c5") and (args.bwd != "pair" or args.fwd_math != "f16")):
             results[w]["roofline"]["traffic"] = PROFILED_TRAFFIC[w]
             results[w]["roofline"]["traffic_source"] = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, summaries in profiles/, measured at " + PROFILED_AT
     if not args.no_cpu:

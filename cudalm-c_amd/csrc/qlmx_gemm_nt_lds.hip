@@ -108,7 +108,8 @@ static int nt3_submit(int BN, const Nt3Args &a, int grid, int slot, bool units, 
         int rc = qlmx_pair_hold_nt(a, grid, slot, units, st, &held); if(rc) return rc;
         return held ? QLMX_OK : qlmx_gemm_nt_lds_issue(a, grid, slot, units, st);
     }
-    int rc = nt3_launch_any(BN, a, grid, st); if(rc) return rc;
+    int rc = qlmx_pair_flush(); if(rc) return rc;          /* the wide tile is never held: what is held goes first */
+    rc = nt3_launch_any(BN, a, grid, st); if(rc) return rc;
     QLMX_LAUNCH_CHECK("grouped gemm nt (direct-to-LDS) launch");
     return units ? qlmx_unit_done(slot, st) : qlmx_upload_done(slot, st);
 }

@@ -124,7 +124,7 @@ def test_f32_c1_single_expert(q, orc):
 def test_f32_c1_whole_chain_into_the_integer_step(q, orc):
     """BASELINE config 1 as one chain on its own two matrices: X fp32 [1024,512] ~ N(0,1), W_up [512,1536] and W_down
     [1536,512] from 0.02 N(0,1) through encode; H = X.W_up, Y = H.W_down; dH = dY.W_down^T, dX = dH.W_up^T;
-    dW_down = H^T.dY, dW_up = X^T.dH with dY ~ N(0,1) (SURVEY's statement of the config: no activation between the two);
+    dW_down = H^T.dY, dW_up = X^T.dH with dY ~ N(0,1) (the configuration as the reference's test states it: no activation between the two);
     then one Integer AdamW step, t = 1, from fresh state (m8 = v8 = 0, moment scales 0) on both matrices with the weight
     gradients scaled to the config's 1e-3 (the device clip scalar: gsp). Every GEMM against the oracle's at 1e-5; the
     step byte for byte against the oracle's step fed the same gradient bits (the step's parity is defined on equal
@@ -654,6 +654,25 @@ def test_backward_pair_is_one_launch_with_the_same_bits(q, orc):
     for a, b in zip(res[0], res[1]):
         assert torch.equal(a, b)
     assert torch.equal(res[1][1], res[1][2]) and float(res[1][0].abs().max()) > 0.0
+    # a weight gradient on the wide tile is never held: it goes behind a held one (it accumulates into the same output)
+    res = []
+    for pair in (False, True):
+        G = torch.zeros(E * K * N, device="cuda")
+        n0 = q.problems([(Xb.data_ptr() + off[e] * K * 2, dYb.data_ptr() + off[e] * N * 2, G.data_ptr() + e * K * N * 4, 0, 0, rows[e], 0.0) for e in range(E)])
+        n1 = q.problems([(Xb.data_ptr() + off[e] * K * 2, dY2b.data_ptr() + off[e] * N * 2, G.data_ptr() + e * K * N * 4, 0, 0, rows[e], 1.0) for e in range(E)])
+        if pair:
+            q.pair_begin(cur)
+        q.gemm_nt(n0, E, K, N, pkg.ACT_BF16, pkg.MATH_MFMA, cur)
+        q.call("qlmx_nt_tile", 256)
+        try:
+            q.gemm_nt(n1, E, K, N, pkg.ACT_BF16, pkg.MATH_MFMA, cur)
+        finally:
+            q.call("qlmx_nt_tile", 128)
+        if pair:
+            q.pair_end(cur)
+        torch.cuda.synchronize()
+        res.append(G.clone())
+    assert torch.equal(res[0], res[1]) and float(res[0].abs().max()) > 0.0
     # misuse
     with pytest.raises(pkg.QlmxError, match="no pair is open"):
         q.pair_end(cur)

@@ -44,7 +44,8 @@ def parse():
     ap.add_argument("--bwd", default="pair", choices=["pair", "serial", "streams"],
                     help="train, c5: the two grouped GEMMs of every backward flush as one launch (qlmx_pair_begin / qlmx_pair_end), "
                          "one after the other, or the weight gradient on the library's side stream beside the input gradient")
-    ap.add_argument("--step-only", action="store_true", help="train: skip the per-launch repetitions, so that a kernel trace holds nothing but steps")
+    ap.add_argument("--step-only", action="store_true", help="train: skip the per-launch repetitions, so that a kernel trace holds nothing but steps; "
+                    "layer: time the merged layer only (no pass-by-pass forms, no glue-only run)")
     ap.add_argument("--adamw-weights", type=int, default=120 * 2 ** 20)
     ap.add_argument("--render-p", type=int, default=0, help="adamw: also write the fp32 view P (4 B/weight more)")
     return ap.parse_args()
@@ -354,8 +355,9 @@ def bench_layer(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2):
 
     steps, warmup = max(5, args.steps // 4), max(2, args.warmup // 4)
     per_pass, one_list = Lists(False), Lists(True)
-    t_sep = timed(torch, lambda: layer(per_pass, False, False), steps, warmup)
-    t_fus = timed(torch, lambda: layer(per_pass, True, False), steps, warmup)
+    nil = {"event_ms_avg": None}
+    t_sep = nil if args.step_only else timed(torch, lambda: layer(per_pass, False, False), steps, warmup)
+    t_fus = nil if args.step_only else timed(torch, lambda: layer(per_pass, True, False), steps, warmup)
     t_mrg = timed(torch, lambda: layer(one_list, True, True), steps, warmup)
     spread = step_spread(torch, lambda: layer(one_list, True, True), steps)
 
@@ -368,7 +370,7 @@ def bench_layer(torch, q, args, E=32, D=768, F=2048, tokens=8192, topk=2):
         q.moe_gather(x, L.tok, Xp, L.R, D, ACT_BF16, stream)
         q.moe_dgate_merged(dout, yp, L.perm, gate, dgate, dyp, N, K, D, ACT_BF16, stream)
         q.moe_combine(dXp, L.inv, None, dx, N, K, D, stream)
-    t_glue = timed(torch, glue_only, steps, warmup)
+    t_glue = nil if args.step_only else timed(torch, glue_only, steps, warmup)
     flops = K * 12 * 2.0 * N * D * F                       # per pass: 3 forward GEMMs, 3 recomputed in the backward, 3 dgrad, 3 wgrad
     tf = flops / (t_mrg["event_ms_avg"] * 1e-3) / 1e12
     return {"workload": "C3 whole expert layer, forward + backward with the recomputed forward (%d tokens top-%d, E=%d D=%d F=%d): GEMMs and glue" % (N, K, E, D, F),
@@ -897,10 +899,11 @@ def cpu_decode(args, E=32, D=768, F=2048, topk=2, T=16, layers=2):
 # counter values and scale factors are in profiles/*.txt. adamw: per launch. train: per step, i.e. summed over
 # the step's 4 launches (1035.9 MiB read + 1086.2 MiB written). c5: per step over the 32 GEMM launches of the 8
 # layers (104.4 GiB read + 49.0 GiB written). decode: per launch = per layer at T=16 (64.1 MiB read + 5.1 MiB
-# written). train and c5 are those of the default --bwd pair. The figures are constants of the code state they
+# written). layer: per step of the merged layer, all its kernels (2442.1 MiB read + 1393.2 MiB written). train and c5
+# are those of the default --bwd pair. The figures are constants of the code state they
 # were measured at; that state is named in the JSON line so that a reader can tell a stale one.
-PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.225e9, "c5": 1.648e11, "decode": 7.39e7}
-PROFILED_AT = "git bd3f2f6 (train, c5), ef06021 (decode), 87b8442 (adamw)"
+PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.225e9, "layer": 4.022e9, "c5": 1.648e11, "decode": 7.39e7}
+PROFILED_AT = "git bd3f2f6 (train, layer, c5), ef06021 (decode), 87b8442 (adamw)"
 
 
 def main():

@@ -62,6 +62,9 @@ SIGNATURES = {
     "qlmx_side_join": (c_i, [c_vp]),
     "qlmx_pair_begin": (c_i, [c_vp]),
     "qlmx_pair_end": (c_i, [c_vp]),
+    "qlmx_prof_mark": (c_i, [C.c_char_p, c_vp]),
+    "qlmx_prof_report": (c_i, [C.c_char_p, C.c_size_t, C.POINTER(c_i)]),
+    "qlmx_prof_reset": (c_i, []),
     "qlmx_qhashu": (C.c_uint, [c_u64]),
     "qlmx_qsri": (c_i, [c_f, c_u64, c_u64]),
     "qlmx_qclmp": (c_i, [c_i, c_i, c_i]),
@@ -281,6 +284,16 @@ class Qlmx:
 
     def side_join(self, stream=None):
         self.call("qlmx_side_join", stream)
+
+    def prof_mark(self, label, stream=None):
+        """An event on `stream`; the GPU time since the previous mark is charged to `label` (qlmx_prof_mark)."""
+        self.call("qlmx_prof_mark", label.encode(), stream)
+
+    def prof_report(self):
+        """(text of the table, number of labels) of qlmx_prof_report"""
+        buf = C.create_string_buffer(8192); n = C.c_int(0)
+        self.call("qlmx_prof_report", buf, len(buf), C.byref(n))
+        return buf.value.decode(), int(n.value)
 
     def pair_begin(self, stream=None):
         """Hold back the next input-gradient and weight-gradient launches on `stream` (qlmx_pair_begin)."""

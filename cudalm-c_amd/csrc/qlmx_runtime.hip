@@ -140,3 +140,78 @@ extern "C" void qlmx_qd_set_host(signed char *d, unsigned long long i, int v, in
     *b = (unsigned char)((i & 1ULL) ? ((*b & 0x0Fu) | (nib << 4)) : ((*b & 0xF0u) | nib));
 }
 extern "C" unsigned long long qlmx_qd_bytes(unsigned long long nq, int packed){ return packed ? (nq + 1) / 2 : nq; }
+
+/* ---- label timing without synchronisation (prof_ev / prof_flush / prof_report, cudalm.cu:806-840) ----
+ * qlmx_prof_mark(label, stream) records an event on `stream`; a label is charged the GPU time between the mark
+ * before it and its own, so marks are placed BEHIND the work they name, as the reference places kchk(). `drained`
+ * counts the marks that found the previous mark's event already complete: the GPU had run out of queued work and
+ * the host was the bottleneck at that point. Events live in a ring that is drained (one wait for the newest event)
+ * when it is full and by the report. Host-side state only; the marks are ordinary event records. */
+#define PROF_LABELS 48
+#define PROF_EVENTS 1024
+struct ProfLabel { char name[40]; double ms; long n, drained; };
+static ProfLabel g_pl[PROF_LABELS];
+static int g_pl_n = 0;
+static hipEvent_t g_pe[PROF_EVENTS];
+static short g_pe_label[PROF_EVENTS];
+static int g_pe_n = 0;
+static bool g_pe_made = false;
+static int prof_label(const char *what){
+    for(int i = 0; i < g_pl_n; i++) if(!strncmp(g_pl[i].name, what, sizeof g_pl[i].name - 1)) return i;
+    if(g_pl_n == PROF_LABELS) return PROF_LABELS - 1;                     /* the table is full: the last entry takes the rest */
+    memset(&g_pl[g_pl_n], 0, sizeof g_pl[0]);
+    snprintf(g_pl[g_pl_n].name, sizeof g_pl[0].name, "%s", what);
+    return g_pl_n++;
+}
+static int prof_drain(void){
+    if(g_pe_n < 2) return QLMX_OK;
+    QLMX_HIP(hipEventSynchronize(g_pe[g_pe_n - 1]), "label timing: wait for the newest mark");
+    for(int i = 1; i < g_pe_n; i++){
+        float ms = 0.0f;
+        QLMX_HIP(hipEventElapsedTime(&ms, g_pe[i - 1], g_pe[i]), "label timing: elapsed time");
+        g_pl[g_pe_label[i]].ms += ms; g_pl[g_pe_label[i]].n++;
+    }
+    const hipEvent_t last = g_pe[g_pe_n - 1];                             /* the newest mark starts the next interval */
+    g_pe[g_pe_n - 1] = g_pe[0]; g_pe[0] = last; g_pe_n = 1;
+    return QLMX_OK;
+}
+extern "C" int qlmx_prof_mark(const char *label, void *stream){
+    int rc = qlmx_check_ready(); if(rc) return rc;
+    QLMX_REQUIRE(label && label[0], "qlmx_prof_mark: empty label");
+    if(!g_pe_made){
+        for(int i = 0; i < PROF_EVENTS; i++) QLMX_HIP(hipEventCreate(&g_pe[i]), "label timing: event");
+        g_pe_made = true;
+    }
+    const int k = prof_label(label);
+    if(g_pe_n > 0 && hipEventQuery(g_pe[g_pe_n - 1]) == hipSuccess) g_pl[k].drained++;
+    (void)hipGetLastError();                                              /* hipErrorNotReady from the query is not an error */
+    QLMX_HIP(hipEventRecord(g_pe[g_pe_n], (hipStream_t)stream), "label timing: record");
+    g_pe_label[g_pe_n++] = (short)k;
+    return g_pe_n == PROF_EVENTS ? prof_drain() : QLMX_OK;
+}
+/* Writes the table, largest total first, one line per label: name, ms, share, count, drained (the format of
+ * prof_report, cudalm.cu:826-840), and returns the number of labels through *nlabels (may be NULL). The text is
+ * cut at cap - 1 characters. */
+extern "C" int qlmx_prof_report(char *out, size_t cap, int *nlabels){
+    int rc = prof_drain(); if(rc) return rc;
+    QLMX_REQUIRE(out && cap > 0, "qlmx_prof_report: no buffer");
+    int order[PROF_LABELS];
+    double tot = 0.0;
+    for(int i = 0; i < g_pl_n; i++){ order[i] = i; tot += g_pl[i].ms; }
+    for(int i = 0; i < g_pl_n; i++) for(int j = i + 1; j < g_pl_n; j++) if(g_pl[order[j]].ms > g_pl[order[i]].ms){ const int t = order[i]; order[i] = order[j]; order[j] = t; }
+    size_t at = 0;
+    out[0] = 0;
+    auto put = [&](const char *fmt, auto... v){ if(at + 1 < cap){ const int w = snprintf(out + at, cap - at, fmt, v...); if(w > 0) at = at + (size_t)w < cap ? at + (size_t)w : cap - 1; } };
+    put("[prof] per-label totals (%.3f ms tracked, GPU time between marks)\n", tot);
+    for(int i = 0; i < g_pl_n; i++){
+        const ProfLabel &e = g_pl[order[i]];
+        put("  %-22s %9.3f ms  %5.1f%%   x%ld   drained %ld\n", e.name, e.ms, tot > 0.0 ? 100.0 * e.ms / tot : 0.0, e.n, e.drained);
+    }
+    if(nlabels) *nlabels = g_pl_n;
+    return QLMX_OK;
+}
+extern "C" int qlmx_prof_reset(void){
+    int rc = prof_drain(); if(rc) return rc;
+    g_pl_n = 0; g_pe_n = 0;
+    return QLMX_OK;
+}

@@ -178,9 +178,12 @@ static void step_groups(Qlm *q, float *P, const float *G, int gi0, int ng, float
 void qlm_gpu_update(Qlm *q, float *P, float *G, float lr, float b1, float b2, float wd,
                     float bc1, float bc2, int t, const float *gs){
     step_groups(q, P, G, 0, (int)q->ngrp, lr, b1, b2, wd, 1.0f, gs, bc1, bc2, t, getenv("CUDALM_QLM_DIAG") ? q->statD : NULL);
+    kchk("qlm step", -1);                                              /* cudalm.cu:6089 */
     const bool servo_due = q->servo_every > 0 && t % q->servo_every == 0;
-    if(servo_due)
+    if(servo_due){
         ck(qlmx_servo(q->d, q->r, q->s, q->spanD, q->nspan, q->group, q->dmax, q->f_hi, q->f_lo, q->packed, (int)q->ngrp, NULL), "qlm servo");
+        kchk("qlm servo", -1);                                         /* cudalm.cu:6101 */
+    }
 }
 
 /* cudalm.cu:6110-6135 without the float spans' AdamW and the diagnostics */
@@ -521,4 +524,80 @@ void mg_flush(void){
     mg_run_pairs(); mg_run(g_q[0]); mg_run(g_q[1]);
     if(paired){ if(qlmx_pair_end(NULL) != QLMX_OK){ fprintf(stderr, "mg_flush: %s\n", qlmx_last_error()); exit(1); } }
     else mg_run(g_q[2]);
+}
+
+/* ---- kchk / prof_report (cudalm.cu:787-855) ---- */
+namespace {
+struct LabelTime { std::string name; double ms = 0.0; long n = 0; };
+struct CheckState {
+    int debug = -1, prof = -1;                 /* -1: not read yet */
+    double tdr = 2.0, prev = 0.0, max_ms = 0.0;
+    std::string max_what = "(none)";
+    std::vector<LabelTime> tab;                /* waiting modes; the event mode's table lives in the library */
+};
+CheckState g_chk;
+double wall_seconds(){
+    struct timespec ts; clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+}
+void chk_levels_from_env(){
+    if(g_chk.debug >= 0) return;
+    const char *d = getenv("CUDALM_DEBUG"), *p = getenv("CUDALM_PROF");
+    g_chk.debug = (d && atoi(d) != 0) ? 1 : 0;
+    g_chk.prof = p ? atoi(p) : 0;
+    g_chk.prev = wall_seconds();
+}
+}
+void kchk_levels(int debug, int prof, double tdr_seconds){
+    g_chk.debug = debug ? 1 : 0; g_chk.prof = prof; g_chk.tdr = tdr_seconds > 0.0 ? tdr_seconds : 2.0;
+    g_chk.prev = wall_seconds(); g_chk.max_ms = 0.0; g_chk.max_what = "(none)"; g_chk.tab.clear();
+    qlmx_prof_reset();
+}
+void kchk(const char *what, int l){
+    chk_levels_from_env();
+    if(!g_chk.debug && !g_chk.prof) return;
+    if(g_chk.prof >= 3 && !g_chk.debug){
+        if(qlmx_prof_mark(what, NULL) != QLMX_OK){ fprintf(stderr, "kchk: %s\n", qlmx_last_error()); exit(1); }
+        return;
+    }
+    if(qlmx_sync(NULL) != QLMX_OK){
+        fprintf(stderr, "\n[FAULT] after %s (layer %d): %s\n", what, l, qlmx_last_error());
+        exit(1);
+    }
+    const double now = wall_seconds(), ms = (now - g_chk.prev) * 1000.0;
+    g_chk.prev = now;
+    if(g_chk.prof){
+        size_t i = 0;
+        while(i < g_chk.tab.size() && g_chk.tab[i].name != what) i++;
+        if(i == g_chk.tab.size()){ g_chk.tab.emplace_back(); g_chk.tab.back().name = what; }
+        g_chk.tab[i].ms += ms; g_chk.tab[i].n++;
+    }
+    if(ms > g_chk.max_ms){
+        g_chk.max_ms = ms;
+        char buf[128]; snprintf(buf, sizeof buf, "%s (layer %d)", what, l);
+        g_chk.max_what = buf;
+    }
+    if(g_chk.debug && ms > g_chk.tdr * 1000.0 * 0.25)
+        fprintf(stderr, "[WARN] %s (layer %d) took %.0f ms - %.0f%% of the %.0fs TDR budget\n", what, l, ms, 100.0 * ms / (g_chk.tdr * 1000.0), g_chk.tdr);
+}
+const char *kchk_slowest(double *ms){ if(ms) *ms = g_chk.max_ms; return g_chk.max_what.c_str(); }
+void prof_report(void){
+    chk_levels_from_env();
+    if(!g_chk.prof) return;
+    if(g_chk.prof >= 3 && !g_chk.debug){
+        static char text[8192];
+        int n = 0;
+        if(qlmx_prof_report(text, sizeof text, &n) != QLMX_OK){ fprintf(stderr, "prof_report: %s\n", qlmx_last_error()); exit(1); }
+        if(n) printf("\n%s", text);
+        fflush(stdout);
+        return;
+    }
+    if(g_chk.tab.empty()) return;
+    std::vector<LabelTime> t = g_chk.tab;
+    std::stable_sort(t.begin(), t.end(), [](const LabelTime &a, const LabelTime &b){ return a.ms > b.ms; });
+    double tot = 0.0;
+    for(const LabelTime &e : t) tot += e.ms;
+    printf("\n[prof] per-kernel totals over the run (%.0f ms tracked)\n", tot);
+    for(const LabelTime &e : t) printf("  %-22s %9.1f ms  %5.1f%%   x%ld\n", e.name.c_str(), e.ms, 100.0 * e.ms / tot, e.n);
+    fflush(stdout);
 }

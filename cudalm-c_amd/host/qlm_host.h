@@ -112,4 +112,16 @@ void mg_atb(const void *A, const void *B, float *C, int M, int K, int N);       
  * item: gp = A.B1, up = A.B3 (fp32, kept for the backward pass), ap = bf16(SwiGLU(gp, up)) */
 void mg_ab_swiglu(const void *A, const float *B1, const float *B3, float *gp, float *up, void *ap, int M, int K, int N);
 void mg_flush(void);                                                                      /* cudalm.cu:3243 */
+
+/* Label timing and fault localisation at the reference's check points (kchk, cudalm.cu:842-855; hooks e.g. at 4336,
+ * 4366, 6089). Levels as the reference reads them from the environment (cudalm.cu:10764-10765): CUDALM_DEBUG != 0 or
+ * CUDALM_PROF = 1, 2: wait for the device at every label, report a fault by label and layer and exit(1), charge the
+ * wall time since the previous label to this one, warn when one label took more than a quarter of the watchdog
+ * budget; CUDALM_PROF >= 3 (and no debug): no wait -- an event per label, GPU time between events, and a count of the
+ * labels at which the GPU had already run dry. Neither set: kchk returns at once. prof_report prints the table
+ * (cudalm.cu:826-840); kchk_slowest returns the label that took longest in the waiting modes. */
+void kchk(const char *what, int l);
+void prof_report(void);
+const char *kchk_slowest(double *ms);
+void kchk_levels(int debug, int prof, double tdr_seconds);        /* instead of the environment (tests, hosts with flags) */
 #endif

@@ -40,7 +40,8 @@ static std::vector<unsigned char> slurp(const char *path){
  * cudalm.cu:6454 forms them; the gradient of step t is the t-th block of np floats in QLM_TEST_GRADS; when
  * QLM_TEST_CLIP is set the step takes its clip multiplier from a device scalar holding that value). The servo
  * period, the optimizer and the LR mode come from the environment as in the reference. OUT gets, raw and in this
- * order: d, r, m8, v8 (Adam only), s, m8s, v8s (Adam only), sref per span, the fp32 view P. */
+ * order: d, r, m8, v8 (Adam only), s, m8s, v8s (Adam only), sref per span, the fp32 view P. With CUDALM_PROF or
+ * CUDALM_DEBUG set the driver's check points (kchk) time its labels and the table is printed at the end. */
 static int tool(int argc, char **argv){
     if(argc < 7){ fprintf(stderr, "usage: %s optq|sref|update IN OUT PREFIX GAP N0 [N1 ...]\n", argv[0]); return 2; }
     size_t np = 0;
@@ -112,6 +113,9 @@ static int tool(int argc, char **argv){
         if(!okw){ fprintf(stderr, "update: short write to %s\n", argv[3]); return 1; }
         printf("update: %d steps, %d servo passes, adam %d lrmode %d group %d dmax %d, %llu weights %llu groups\n",
                steps, servo_passes, q.adam, q.lrmode, q.group, q.dmax, q.nq, q.ngrp);
+        prof_report();                                     /* the table of the driver's kchk labels when CUDALM_PROF is set */
+        double slow_ms = 0.0; const char *slow = kchk_slowest(&slow_ms);
+        if(getenv("CUDALM_DEBUG") && atoi(getenv("CUDALM_DEBUG"))) printf("slowest label: %s, %.3f ms\n", slow, slow_ms);
         return 0;
     }
     fprintf(stderr, "unknown mode %s\n", argv[1]); return 2;

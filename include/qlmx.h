@@ -81,6 +81,17 @@ int         qlmx_side_join(void *stream);
  * synchronisation (nothing held runs before qlmx_pair_end or one of the calls just named). */
 int         qlmx_pair_begin(void *stream);
 int         qlmx_pair_end(void *stream);
+/* Label timing without synchronisation: prof_ev / prof_flush / prof_report behind kchk, cudalm.cu:806-840.
+ * qlmx_prof_mark(label, stream) records an event on `stream` and charges the GPU time since the previous mark to
+ * `label` (marks stand BEHIND the work they name, as the reference places kchk); a mark that finds the previous
+ * mark's event already complete counts as `drained`: the GPU had no queued work left and the host was the bottleneck
+ * there. Up to 48 labels (the rest share the last entry); events are drained every 1024 marks and by the report.
+ * qlmx_prof_report writes the table (largest total first: name, ms, share, count, drained) into out[cap] and the number
+ * of labels into *nlabels (may be NULL); qlmx_prof_reset forgets everything. The waiting modes of kchk (fault
+ * localisation, wall time per label) live in the host mirror (cudalm-c_amd/host/qlm_host.h: kchk, prof_report). */
+int         qlmx_prof_mark(const char *label, void *stream);
+int         qlmx_prof_report(char *out, size_t cap, int *nlabels);
+int         qlmx_prof_reset(void);
 
 /* ---- host integer helpers: the __host__ __device__ inlines of qlm.cuh:78-111, used by the
  *      reference's checkpoint code and selftest reference (cudalm.cu:10574-10580) ---- */

@@ -274,3 +274,56 @@ def test_host_mirror_update_driver_equals_the_oracle(orc, tmp_path, opt, lrmode,
         assert np.array_equal(got[at: at + wb.size], wb), "%s differs after %d steps (%d groups rescaled on the way)" % (name, steps, rescaled)
         at += wb.size
     assert at == got.size
+
+
+@pytest.mark.parametrize("prof,debug", [(3, 0), (1, 0), (0, 1)])
+def test_host_mirror_check_points_time_their_labels(orc, tmp_path, prof, debug):
+    """kchk / prof_report (cudalm.cu:787-855) at the optimizer driver's check points (cudalm.cu:6089, 6101): with
+    CUDALM_PROF=3 an event per label and the GPU time between them, with CUDALM_PROF=1 a wait per label and wall time,
+    with CUDALM_DEBUG=1 the slowest label; four steps with a servo pass after every second one give four `qlm step`
+    and two `qlm servo` entries."""
+    sizes = [128 * 12]
+    np_ = 4 + sizes[0] + 2
+    src, gsrc, dst = str(tmp_path / "P.f32"), str(tmp_path / "G.f32"), str(tmp_path / "state.bin")
+    orc.normal(np_, 7, 1, 0.02).tofile(src)
+    np.concatenate([orc.normal(np_, 7, 10 + t, 2e-2) for t in range(4)]).tofile(gsrc)
+    env = dict(os.environ, QLM_SERVO="2", QLM_TEST_STEPS="4", QLM_TEST_GRADS=gsrc, CUDALM_PROF=str(prof), CUDALM_DEBUG=str(debug))
+    p = subprocess.run([os.path.join(PKG_DIR, "qlm_selftest"), "update", src, dst, "4", "0"] + [str(n) for n in sizes],
+                       env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert p.returncode == 0, p.stdout
+    if prof:
+        assert "[prof]" in p.stdout, p.stdout
+        step = [l for l in p.stdout.splitlines() if l.strip().startswith("qlm step")][0]
+        servo = [l for l in p.stdout.splitlines() if l.strip().startswith("qlm servo")][0]
+        # the first mark of the event mode only starts the clock: three of the four steps are intervals
+        assert (" x3 " in step + " " or " x4" in step) and " x2" in servo, p.stdout
+        if prof >= 3:                                   # GPU time to a microsecond; the waiting mode prints tenths of a millisecond
+            assert float(step.split()[2]) > 0.0 and float(servo.split()[2]) > 0.0 and "drained" in step, p.stdout
+        else:
+            assert float(step.split()[2]) >= float(servo.split()[2]) >= 0.0, p.stdout
+    if debug:
+        assert "slowest label: qlm " in p.stdout, p.stdout
+
+
+def test_label_timing_through_the_c_abi(q):
+    """qlmx_prof_mark / qlmx_prof_report: a long fill and a short one behind their marks; the long one's label takes
+    more GPU time, counts add up, the report is sorted, qlmx_prof_reset forgets."""
+    import torch
+    cur = torch.cuda.current_stream().cuda_stream
+    big = torch.empty(1 << 28, dtype=torch.uint8, device="cuda"); small = torch.empty(1 << 12, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    q.call("qlmx_prof_reset")
+    q.prof_mark("start", cur)
+    for rep in range(5):
+        q.call("qlmx_memset", big, rep, big.numel(), cur); q.prof_mark("big fill", cur)
+        q.call("qlmx_memset", small, rep, small.numel(), cur); q.prof_mark("small fill", cur)
+    text, n = q.prof_report()
+    assert n == 3, text
+    lines = [l.split() for l in text.splitlines()[1:]]
+    got = {" ".join(l[:-6]): (float(l[-6]), int(l[-3][1:]), int(l[-1])) for l in lines}    # name, ms, "ms", share, xN, "drained", count
+    assert got["big fill"][1] == 5 and got["small fill"][1] == 5 and got["start"][1] == 0, text
+    assert got["big fill"][0] > 5 * got["small fill"][0] > 0.0, text
+    assert lines[0][0] == "big", text                       # largest total first
+    q.call("qlmx_prof_reset")
+    text, n = q.prof_report()
+    assert n == 0, text

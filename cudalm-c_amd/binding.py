@@ -93,6 +93,7 @@ SIGNATURES = {
     "qlmx_decode_math": (c_i, [c_i]),
     "qlmx_test_sqrt_form": (c_i, [C.c_uint, c_u64, c_vp, c_vp]),
     "qlmx_test_div_form": (c_i, [c_u64, c_u64, c_vp, c_vp]),
+    "qlmx_test_step_wide": (c_i, [c_i]),
     "qlmx_step_touched": (c_i, [c_vp] * 10 + [c_i, c_i, c_i, c_f, c_f, c_f, c_f, c_f, c_f, c_f, c_u64, c_u64, c_vp, c_i, c_vp]),
     "qlmx_sqsum": (c_i, [c_vp, c_u64, c_vp, c_vp]),
     "qlmx_gnorm": (c_i, [c_vp, c_i, c_i, c_vp, c_vp]),

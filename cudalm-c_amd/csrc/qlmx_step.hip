@@ -110,6 +110,14 @@ __device__ __forceinline__ float qx_row16_max_nonneg(float f){
         "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf" : "+v"(v));
     return __uint_as_float(v);
 }
+/* the same over the 8 lanes of a half row (lanes 0-7 and 8-15 of every row of 16 separately) */
+__device__ __forceinline__ float qx_row8_max_nonneg(float f){
+    uint32_t v = __float_as_uint(f);
+    asm("s_nop 1\n\tv_max_u32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf" : "+v"(v));
+    return __uint_as_float(v);
+}
 /* byte `B` of `word` = low byte of a - b, the other bytes kept (a sub-dword destination instead of a subtract and
  * a funnel shift) */
 template<int B> __device__ __forceinline__ void qx_sub_to_byte(uint32_t &word, int a, int b){
@@ -280,14 +288,141 @@ __device__ __forceinline__ bool step_row8_mid(const StepParams &a, const GroupCt
     return true;
 }
 
+/* The same for a group spread over 8 lanes: a lane owns two runs of 8 weights, elements 8 l .. 8 l + 7 and
+ * 64 + 8 l .. 64 + 8 l + 7 of its group, so that every access of a half row still covers 256 contiguous bytes of G
+ * (64 of the byte arrays), a wavefront steps 8 groups, and what a lane works out once per group -- the span, the
+ * addresses, the scales, the learning-rate quotient, the new scales and their reciprocals -- is spread over 16
+ * weights instead of 8. Same arithmetic per element and the same guards as step_row8_mid, hence the same bytes;
+ * qg, pofg, gofg are the positions of the group's first weight in the byte arrays, in P and in G. */
+template<bool HASP, bool V4>
+__device__ __forceinline__ bool step_row16_mid(const StepParams &a, const GroupCtx &c, int gi, int lane8, uint64_t qg, uint64_t pofg, uint64_t gofg,
+                                               uint64_t kt, uint64_t ktm, uint64_t ktv){
+    float mn[2][8], rv[2][8], uu[2][8];
+    uint32_t dw[2]; uint2 rw[2];
+    float vmin = 3.0e38f, amin = 3.0e38f, am = 0.0f, vm = 0.0f;
+#pragma unroll
+    for(int h = 0; h < 2; h++){
+        const uint64_t e = (uint64_t)(h * 64 + lane8 * 8);
+        const float4 h0 = *(const float4 *)(a.G + gofg + e), h1 = *(const float4 *)(a.G + gofg + e + 4);
+        const uint2 mw = *(const uint2 *)(a.m8 + qg + e), vw = *(const uint2 *)(a.v8 + qg + e);
+        dw[h] = *(const uint32_t *)(a.d + ((qg + e) >> 1));
+        rw[h] = *(const uint2 *)(a.r + qg + e);
+        const float gv[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
+#pragma unroll
+        for(int k = 0; k < 8; k++){
+            const uint32_t mword = k < 4 ? mw.x : mw.y, vword = k < 4 ? vw.x : vw.y;
+            const int sh = 8 * (k & 3);
+            const float gr = gv[k] * c.gs;
+            const float mv = (float)(int)(signed char)(mword >> sh) * c.ms_old;
+            float sv = (float)((vword >> sh) & 0xFFu) * c.vs_old; if(V4) sv = sv * sv;
+            mn[h][k] = c.b1 * mv + c.omb1 * gr;
+            rv[h][k] = c.b2 * (sv * sv) + c.omb2 * gr * gr;                /* the second moment; its root below */
+            vmin = fminf(vmin, rv[h][k]);
+            amin = fminf(amin, fabsf(mn[h][k])); am = fmaxf(am, fabsf(mn[h][k]));
+        }
+    }
+    if(__builtin_amdgcn_ballot_w64(!(vmin >= 0x1p-96f)) != 0) return false;        /* NaN compares false */
+#pragma unroll
+    for(int h = 0; h < 2; h++)
+#pragma unroll
+        for(int k = 0; k < 8; k++){
+            rv[h][k] = qx_sqrt_above_2m96(rv[h][k]);
+            const float u = qx_div_mid(mn[h][k] * c.inv_bc1, rv[h][k] * c.inv_sqrt_bc2 + c.veps);
+            uu[h][k] = __builtin_amdgcn_fmed3f(u, -8.0f, 8.0f);
+            vm = fmaxf(vm, rv[h][k]);                    /* the guard wants the plain root also when V4 */
+        }
+    {
+        const float nlo = amin * c.inv_bc1, nhi = am * c.inv_bc1;
+        const bool lane_ok = vm <= 0x1p25f && nlo >= 0x1p-40f && nhi <= 0x1p40f && am >= 0x1p-32f && am <= 0x1p40f && c.veps <= 0x1p20f;
+        if(__builtin_amdgcn_ballot_w64(!lane_ok) != 0) return false;
+    }
+    if(V4){
+        vm = 0.0f;
+#pragma unroll
+        for(int h = 0; h < 2; h++)
+#pragma unroll
+            for(int k = 0; k < 8; k++){ rv[h][k] = qx_sqrt_above_2m96(rv[h][k]); vm = fmaxf(vm, rv[h][k]); }
+    }
+    /* ---- digits and residuals (qlm.cuh:230-242) ---- */
+    uint64_t ki = QLMX_KI;
+    asm volatile("" : "+s"(ki));
+    int dlo = -c.dmax, dhi = c.dmax;
+    asm volatile("" : "+v"(dlo), "+v"(dhi));
+    uint64_t key0[2];
+#pragma unroll
+    for(int h = 0; h < 2; h++){
+        const uint64_t e = (uint64_t)(h * 64 + lane8 * 8), q = qg + e;
+        key0[h] = q * QLMX_KI + 0x9E3779B97F4A7C15ULL;                   /* the hash's own additive constant rides along */
+        float pv[8];
+        uint32_t dnew = 0, rn0 = 0, rn1 = 0;
+        uint64_t key = key0[h] + kt;
+#pragma unroll
+        for(int k = 0; k < 8; k++){
+            const uint32_t rword = k < 4 ? rw[h].x : rw[h].y;
+            const int rold = (int)(signed char)(rword >> (8 * (k & 3)));
+            const int dd = qx_nib(dw[h], k);
+            const float v = -(c.L * uu[h][k] + c.dec * (float)dd);
+            const float fl = floorf(v);
+            const int rr0 = rold + (int)fl + (qx_hash_unit(key) < (v - fl) ? 1 : 0);
+            const int cyv = rr0 + 63 - (rr0 >> 31);
+            const int cy = cyv >> 7;                                       /* qx_carry(rr0) */
+            if(k == 0) qx_sub_to_byte<0>(rn0, rr0, cyv & 0x80); if(k == 1) qx_sub_to_byte<1>(rn0, rr0, cyv & 0x80);
+            if(k == 2) qx_sub_to_byte<2>(rn0, rr0, cyv & 0x80); if(k == 3) qx_sub_to_byte<3>(rn0, rr0, cyv & 0x80);
+            if(k == 4) qx_sub_to_byte<0>(rn1, rr0, cyv & 0x80); if(k == 5) qx_sub_to_byte<1>(rn1, rr0, cyv & 0x80);
+            if(k == 6) qx_sub_to_byte<2>(rn1, rr0, cyv & 0x80); if(k == 7) qx_sub_to_byte<3>(rn1, rr0, cyv & 0x80);
+            const int dn = qx_med3i(dd + cy, dlo, dhi);
+            if(HASP) pv[k] = c.sg * (float)dn;
+            dnew = __builtin_amdgcn_alignbit((uint32_t)dn, dnew, 4);
+            key += ki;
+        }
+        *(uint32_t *)(a.d + (q >> 1)) = dnew;
+        *(uint2 *)(a.r + q) = make_uint2(rn0, rn1);
+        if(HASP){
+            typedef float f4 __attribute__((ext_vector_type(4)));
+            f4 p0 = {pv[0], pv[1], pv[2], pv[3]}, p1 = {pv[4], pv[5], pv[6], pv[7]};
+            __builtin_nontemporal_store(p0, (f4 *)(a.P + pofg + e));
+            __builtin_nontemporal_store(p1, (f4 *)(a.P + pofg + e + 4));
+        }
+    }
+    /* ---- fresh scales and the re-quantised moments (qlm.cuh:244-278); both maxima are positive here ---- */
+    am = qx_row8_max_nonneg(am); vm = qx_row8_max_nonneg(vm);
+    const float ms = qx_div_mid(am, 127.0f), vs = qx_div_mid(vm, 255.0f);
+    const float ym = qx_div_mid(1.0f, ms), yv = qx_div_mid(1.0f, vs);
+    if(lane8 == 0){ a.m8s[gi] = ms; a.v8s[gi] = vs; }
+#pragma unroll
+    for(int h = 0; h < 2; h++){
+        const uint64_t q = qg + (uint64_t)(h * 64 + lane8 * 8);
+        uint32_t mo0 = 0, mo1 = 0, vo0 = 0, vo1 = 0;
+        uint64_t keym = key0[h] + ktm, keyv = key0[h] + ktv;
+#pragma unroll
+        for(int k = 0; k < 8; k++){
+            const float t = mn[h][k] * ym;
+            const float qm = __builtin_amdgcn_fmed3f(fmaf(fmaf(-t, ms, mn[h][k]), ym, t), -127.0f, 127.0f);
+            const float w = rv[h][k] * yv, qv = fmaf(fmaf(-w, vs, rv[h][k]), yv, w);
+            {
+                const float fl = floorf(qm);
+                const int mq = (int)fl + (qx_hash_unit(keym) < (qm - fl) ? 1 : 0);
+                if(k < 4) mo0 = __builtin_amdgcn_alignbit((uint32_t)mq, mo0, 8); else mo1 = __builtin_amdgcn_alignbit((uint32_t)mq, mo1, 8);
+            }
+            {
+                const float fl = floorf(qv);
+                const float vq = fmaxf(fl + (qx_hash_unit(keyv) < (qv - fl) ? 1.0f : 0.0f), 1.0f);
+                if(k < 4) vo0 = __builtin_amdgcn_cvt_pk_u8_f32(vq, k & 3, vo0); else vo1 = __builtin_amdgcn_cvt_pk_u8_f32(vq, k & 3, vo1);
+            }
+            keym += ki; keyv += ki;
+        }
+        *(uint2 *)(a.m8 + q) = make_uint2(mo0, mo1);
+        *(uint2 *)(a.v8 + q) = make_uint2(vo0, vo1);
+    }
+    return true;
+}
+
 /* STAT: the four counters are kept; HASP: the fp32 view is written; V4: the second moment is stored as its
  * fourth root (a.v4). All are fixed per launch, so they are template parameters and the usual launch (none of
  * them) carries no trace of them: as a run-time flag, v4 made the compiler compute the second square root of
  * every element and select (18 of 186 vector instructions per weight). */
 template<bool ADAM, bool STAT, bool HASP, bool V4>
-__global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
-    const int lane16 = threadIdx.x & 15;
-    const int team = (int)((blockIdx.x * (unsigned)blockDim.x + threadIdx.x) >> 4);
+__device__ __forceinline__ void step_team(const StepParams &a, const int team, const int lane16){
     if(team >= a.ng) return;                       /* whole rows leave together */
     const int gi = a.touched ? a.touched[team] : a.gi_base + team;
     const qlmx_span S = a.touched ? a.one : a.sp[qx_span_of(a.sp, a.nspan, gi)];
@@ -535,6 +670,47 @@ __global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
     }
 }
 
+/* one group per row of 16 lanes: every shape, every option */
+template<bool ADAM, bool STAT, bool HASP, bool V4>
+__global__ void __launch_bounds__(256) k_qlmx_step(StepParams a){
+    step_team<ADAM, STAT, HASP, V4>(a, (int)((blockIdx.x * (unsigned)blockDim.x + threadIdx.x) >> 4), threadIdx.x & 15);
+}
+/* Adam on packed groups of 128 without statistics (what a training step launches): one group per 8 lanes, eight
+ * groups per wavefront, through step_row16_mid when all eight are whole, aligned groups with operands in the middle
+ * of the range -- a choice per wavefront, made before anything is stored; otherwise the wavefront's groups go through
+ * the code above, four at a time. */
+template<bool HASP, bool V4>
+__global__ void __launch_bounds__(256) k_qlmx_step_wide(StepParams a){
+    const int lane = threadIdx.x & 63;
+    const int g0 = (int)((blockIdx.x * (unsigned)blockDim.x + threadIdx.x) >> 6) * 8;       /* first group of the wavefront */
+    if(g0 >= a.ng) return;
+    if(g0 + 8 <= a.ng){
+        const int gi = a.gi_base + g0 + (lane >> 3);
+        const qlmx_span S = a.sp[qx_span_of(a.sp, a.nspan, gi)];
+        const uint64_t j0 = (uint64_t)(gi - S.gi0) * 128u;
+        const uint64_t pof = S.pof + j0, qi0 = S.qi0 + j0, gof = S.gof + j0;
+        const bool whole = S.n - j0 >= 128u && ((pof | qi0 | gof) & 7ULL) == 0;
+        if(__builtin_amdgcn_ballot_w64(!whole) == 0){
+            GroupCtx c;
+            c.gs = a.gsp ? *a.gsp : a.gscale;
+            c.sg = a.s[gi];
+            c.L = a.lr * 128.0f / (a.lrmode ? c.sg : S.sref);
+            c.dec = a.lr * a.wd * 128.0f;
+            c.ms_old = a.m8s[gi];
+            c.vs_old = a.v8s[gi];
+            { float q1 = 1.0f * c.vs_old; if(V4) q1 = q1 * q1; c.veps = fmaxf(q1, 1e-8f); }
+            c.b1 = a.b1; c.b2 = a.b2; c.omb1 = 1.0f - a.b1; c.omb2 = 1.0f - a.b2;
+            c.inv_bc1 = a.inv_bc1; c.inv_sqrt_bc2 = a.inv_sqrt_bc2;
+            c.dmax = a.dmax; c.v4 = V4;
+            const uint64_t kt = a.t * QLMX_KT;
+            if(step_row16_mid<HASP, V4>(a, c, gi, lane & 7, qi0, pof, gof, kt, kt + 0x5EEDULL * QLMX_KT, kt + 0xBEEFULL * QLMX_KT)) return;
+            asm volatile("" ::: "memory");         /* nothing was stored; the general code loads its operands itself */
+        }
+    }
+#pragma unroll 1
+    for(int p = 0; p < 2; p++) step_team<true, false, HASP, V4>(a, g0 + 4 * p + (lane >> 4), lane & 15);
+}
+
 template<bool ADAM, bool V4> static void step_launch_opt(const StepParams &a, unsigned blocks, hipStream_t st){
     const bool stat = a.stat != nullptr, hasp = a.P != nullptr;
     if(stat && hasp)  hipLaunchKernelGGL((k_qlmx_step<ADAM, true, true, V4>),   dim3(blocks), dim3(256), 0, st, a);
@@ -548,6 +724,7 @@ static void step_launch(const StepParams &a, bool adam, unsigned blocks, hipStre
     else step_launch_opt<false, false>(a, blocks, st);
 }
 
+static bool g_step_wide = true;
 /* qlm_step_launch (qlm.cuh:377-397) */
 extern "C" int qlmx_step(float *P, const float *G, signed char *d, signed char *r, const float *s,
               signed char *m8, float *m8s, unsigned char *v8, float *v8s,
@@ -574,12 +751,24 @@ extern "C" int qlmx_step(float *P, const float *G, signed char *d, signed char *
     a.mid_ok = inv_sqrt_bc2 >= 0.0f && inv_sqrt_bc2 <= 1024.0f;
     a.vec_ok = (((uintptr_t)P | (uintptr_t)G) & 15) == 0 && (((uintptr_t)r | (uintptr_t)m8 | (uintptr_t)v8) & 7) == 0
                && ((uintptr_t)d & 3) == 0;
-    const unsigned blocks = (unsigned)((ng + 15) / 16);
     hipStream_t st = (hipStream_t)stream;
-    step_launch(a, adam != 0, blocks, st);
+    if(adam && !stat && packed && group == 128 && a.mid_ok && a.vec_ok && g_step_wide){
+        /* a training step's launch: eight groups per wavefront (k_qlmx_step_wide) */
+        const unsigned wblocks = (unsigned)((ng + 31) / 32);
+        if(v4){ if(P) hipLaunchKernelGGL((k_qlmx_step_wide<true, true>), dim3(wblocks), dim3(256), 0, st, a);
+                else  hipLaunchKernelGGL((k_qlmx_step_wide<false, true>), dim3(wblocks), dim3(256), 0, st, a); }
+        else  { if(P) hipLaunchKernelGGL((k_qlmx_step_wide<true, false>), dim3(wblocks), dim3(256), 0, st, a);
+                else  hipLaunchKernelGGL((k_qlmx_step_wide<false, false>), dim3(wblocks), dim3(256), 0, st, a); }
+    } else {
+        const unsigned blocks = (unsigned)((ng + 15) / 16);
+        step_launch(a, adam != 0, blocks, st);
+    }
     QLMX_LAUNCH_CHECK("qlmx_step launch");
     return QLMX_OK;
 }
+/* Test hook: 0 sends every launch through the one-group-per-16-lanes kernel (the two kernels must agree byte for
+ * byte), 1 (the default) lets training-shaped launches take the eight-groups-per-wavefront kernel. */
+extern "C" int qlmx_test_step_wide(int on){ g_step_wide = on != 0; return QLMX_OK; }
 
 /* k_ng_q4_step (cudalm.cu:4472-4520; CPU twin cpu_kern.h:620-648): the step restricted to a list of
  * touched groups of ONE packed 4-bit span that starts at element 0 of d/r/m8/v8/P (the n-gram

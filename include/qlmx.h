@@ -410,6 +410,10 @@ int qlmx_test_sqrt_form(unsigned first_bits, unsigned long long count, unsigned 
  * instructions, which do nothing there. This compares that form with `/` on the device for `count` pseudo-random
  * operand pairs of that range (derived from `seed`) and adds the number of differing results to *mismatches_dev. */
 int qlmx_test_div_form(unsigned long long seed, unsigned long long count, unsigned long long *mismatches_dev, void *stream);
+/* Test hook. qlmx_step has two kernels: one group per 16 lanes (every shape and option) and, for Adam on packed groups
+ * of 128 without statistics, eight groups per wavefront with 16 weights per lane. They must leave the same bytes;
+ * on = 0 sends every later launch through the first, on = 1 (the default) restores the choice. */
+int qlmx_test_step_wide(int on);
 
 /* =====================================================================================
  * q4n wire format (host only, no device needed): quantize_params / dequantize_params with qtype 3

@@ -338,6 +338,48 @@ def test_step_operands_at_the_edges_of_the_mid_range_forms(q, orc, v4, render, i
         assert beq(got, want), nm
 
 
+@pytest.mark.parametrize("v4,render", [(0, False), (1, True)])
+def test_step_eight_groups_per_wavefront_equals_one_per_row(q, orc, v4, render):
+    """The training step's kernel (eight groups per wavefront, 16 weights per lane) against the general one (a group
+    per row of 16 lanes) and the oracle: two spans, the first with a short last group in the middle of a wavefront, a
+    shifted gradient offset on the second, a group count that is no multiple of 8, and a sub-range launch that starts
+    inside a wavefront's worth of groups; three steps, every byte."""
+    import torch
+    group, dmax = 128, 7
+    tab, nq, ng = make_spans([128 * 203 + 40, 128 * 118], group)
+    tab[1]["gof"] = tab[1]["pof"] + 8
+    tab["sref"] = [0.0086, 0.0091]
+    npar = nq + 8
+    st0 = dict(hd=orc.digits(nq, 31, 20), hr=orc.int8(nq, 31, 21, -64, 64), hm8=orc.int8(nq, 31, 22, -127, 127), hv8=orc.u8(nq, 31, 23, 1, 255),
+               hs=orc.uniform(ng, 31, 24, 0.5, 1.5) * f32(0.02 * 3 / 7), hm8s=orc.uniform(ng, 31, 25, 0.5, 1.5) * f32(3e-3 / 127),
+               hv8s=orc.uniform(ng, 31, 26, 0.5, 1.5) * f32(3e-3 / 255))
+    grads = [orc.normal(npar, 31, 30 + t, 1e-3) for t in range(1, 4)]
+    ranges = [(0, ng), (5, ng - 11), (0, ng)]                 # the second step over a sub-range
+    results = []
+    for wide in (1, 0):
+        q.call("qlmx_test_step_wide", wide)
+        try:
+            d, r, m8, v8, s, m8s, v8s = (dev(st0[k].copy()) for k in ("hd", "hr", "hm8", "hv8", "hs", "hm8s", "hv8s"))
+            P = torch.zeros(npar, device="cuda") if render else None
+            for t in range(1, 4):
+                bc1 = f32(1) - f32(0.9) ** f32(t); bc2 = f32(1) - f32(0.95) ** f32(t)
+                hp = (3e-4, 0.9, 0.95, 0.1, 1.0, None, float(f32(1) / bc1), float(f32(1) / np.sqrt(bc2)), 0, t, 1, None, 1) + ranges[t - 1]
+                q.step(P, dev(grads[t - 1]), d, r, s, m8, m8s, v8, v8s, dev(tab), 2, group, dmax, *hp, v4)
+            results.append([host(x) for x in (d, r, m8, v8, m8s, v8s)] + ([host(P)] if render else []))
+        finally:
+            q.call("qlmx_test_step_wide", 1)
+    h = {k: v.copy() for k, v in st0.items()}
+    hP = np.zeros(npar, f32) if render else None
+    for t in range(1, 4):
+        bc1 = f32(1) - f32(0.9) ** f32(t); bc2 = f32(1) - f32(0.95) ** f32(t)
+        hp = (3e-4, 0.9, 0.95, 0.1, 1.0, None, float(f32(1) / bc1), float(f32(1) / np.sqrt(bc2)), 0, t, 1, None, 1) + ranges[t - 1]
+        orc.step(hP, grads[t - 1], h["hd"], h["hr"], h["hs"], h["hm8"], h["hm8s"], h["hv8"], h["hv8s"], tab, group, dmax, *hp, v4)
+    want = [h["hd"], h["hr"], h["hm8"], h["hv8"], h["hm8s"], h["hv8s"]] + ([hP] if render else [])
+    for i, nm in enumerate(["d", "r", "m8", "v8", "m8s", "v8s"] + (["P"] if render else [])):
+        assert np.array_equal(results[0][i].view(np.uint8), results[1][i].view(np.uint8)), nm
+        assert np.array_equal(results[0][i].view(np.uint8), np.asarray(want[i]).view(np.uint8)), nm
+
+
 def test_argument_errors(q):
     import torch
     x = torch.zeros(256, device="cuda")

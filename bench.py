@@ -654,7 +654,7 @@ def bench_adamw(torch, q, args):
         "metric": "int-AdamW GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": tm["wall_ms"], "dtype": "u8+f32",
         "kernel_ms": tm, "weights_per_s": nq / (tm["event_ms_avg"] * 1e-3),
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                     "traffic": None, "kernel": "k_qlmx_step<adam>", "bytes_per_weight": bytes_per_w},
+                     "traffic": None, "kernel": "k_qlmx_step_wide (Adam, eight groups per wavefront)", "bytes_per_weight": bytes_per_w},
     }
 
 
@@ -902,8 +902,8 @@ def cpu_decode(args, E=32, D=768, F=2048, topk=2, T=16, layers=2):
 # written). layer: per step of the merged layer, all its kernels (2442.1 MiB read + 1393.2 MiB written). train and c5
 # are those of the default --bwd pair. The figures are constants of the code state they
 # were measured at; that state is named in the JSON line so that a reader can tell a stale one.
-PROFILED_TRAFFIC = {"adamw": 1.416e9, "train": 2.225e9, "layer": 4.022e9, "c5": 1.648e11, "decode": 7.39e7}
-PROFILED_AT = "git bd3f2f6 (train, layer, c5), ef06021 (decode), 87b8442 (adamw)"
+PROFILED_TRAFFIC = {"adamw": 1.405e9, "train": 2.225e9, "layer": 4.022e9, "c5": 1.648e11, "decode": 7.39e7}
+PROFILED_AT = "git bd3f2f6 (train, layer, c5), ef06021 (decode), 497f628 (adamw)"
 
 
 def main():

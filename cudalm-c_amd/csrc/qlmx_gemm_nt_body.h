@@ -10,7 +10,7 @@
  * 128 of dY -- so that
  *   * every 16-byte piece goes from global memory to LDS without passing through registers
  *     (lane l of a wave instruction lands at base + 16*l; which piece a lane fetches is free, and
- *     that freedom is the XOR swizzle below), three tiles deep, one barrier per step;
+ *     that freedom is the XOR swizzle below), three tiles deep (four in the wide form), one barrier per step;
  *   * an MFMA operand is two ds_read_b64_tr_b16: within 16 lanes, lane i receives element (i & 3)
  *     of the 8-byte pieces addressed by lanes 4v + (i >> 2), v = 0..3; pointing lane 4v + q at
  *     (row r0 + v, columns c0 + 4q .. +3) therefore hands lane i the four consecutive rows
@@ -28,15 +28,14 @@ typedef short  s16x8  __attribute__((ext_vector_type(8)));
 typedef float  f32x16 __attribute__((ext_vector_type(16)));
 
 /* Two tile shapes, one kernel body (template parameters BN = columns of dY per tile, NW = wavefronts):
- *   256 x 128: four wavefronts of 128 x 64, two workgroups per CU (256 registers each);
- *   256 x 256: eight wavefronts of 128 x 64, one workgroup per CU: a third fewer bytes brought into LDS per
- *              multiplication, but all eight wavefronts meet at one barrier per step, so the two on a SIMD read
- *              their operands at the same time instead of one multiplying while the other reads, and nothing
- *              else is resident to cover the prologue and the epilogue. Not faster as measured (see
- *              nt3_pick_bn); opt-in. */
+ *   256 x 128: four wavefronts of 128 x 64, two workgroups per CU (256 registers each), three tiles in LDS;
+ *   256 x 256: eight wavefronts of 128 x 64, one workgroup per CU, four tiles in LDS (128 KB): a third fewer bytes
+ *              brought into LDS per multiplication and a tile more on its way, but all eight wavefronts meet at one
+ *              barrier per step, so the two on a SIMD read their operands at the same time instead of one
+ *              multiplying while the other reads, and nothing else is resident to cover the prologue and the
+ *              epilogue. Faster for experts of a few thousand rows, slower for short ones (see nt3_pick_bn); opt-in. */
 #define NT3_BM 256
 #define NT3_BK 32
-#define NT3_STAGES 3
 #define NT3_A_BYTES (NT3_BK * NT3_BM * 2)      /* 16384 */
 template<int BN, int NW> struct Nt3Shape {
     static constexpr int NT = NW * 64;                       /* threads */
@@ -47,7 +46,8 @@ template<int BN, int NW> struct Nt3Shape {
     static constexpr int B_BYTES = NT3_BK * BN * 2;
     static constexpr int STAGE_BYTES = NT3_A_BYTES + B_BYTES;
     static constexpr int NREQ = NA + NB;                     /* requests per thread and tile */
-    static constexpr int LDS_BYTES = NT3_STAGES * STAGE_BYTES;
+    static constexpr int STAGES = NW == 8 ? 4 : 3;           /* tiles in LDS; STAGES - 1 of them on their way while one is multiplied */
+    static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
     static constexpr int WG_PER_CU = BN == 128 ? 2 : 1;
 };
 
@@ -196,18 +196,18 @@ __device__ __forceinline__ void nt3_block(const Nt3Args &a, const unsigned bid){
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
     constexpr int R0 = SH::NREQ / 2;                        /* requests issued behind the first slice's multiplications */
     auto addrs = [&](int st, uint32_t (&adA)[4], uint32_t (&adB)[NJ]){
-        const uint32_t sb = lds_base + (uint32_t)(st % NT3_STAGES) * SH::STAGE_BYTES;
+        const uint32_t sb = lds_base + (uint32_t)(st % SH::STAGES) * SH::STAGE_BYTES;
 #pragma unroll
         for(int i = 0; i < 4; i++) adA[i] = sb + offA[i];
 #pragma unroll
         for(int j = 0; j < NJ; j++) adB[j] = sb + offB[j];
     };
-    issue(0, 0);
-    issue(1, 1);
+#pragma unroll
+    for(int t = 0; t < SH::STAGES - 1; t++) issue(t, t);
     for(int st = 0; st < steps; st++){
-        /* tile st has landed once at most the requests of tile st+1 are still in flight */
-        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(SH::NREQ) : "memory");
-        __builtin_amdgcn_s_barrier();                       /* everybody's pieces are in; stage (st+2)%3 is free again */
+        /* tile st has landed once at most the requests of the STAGES - 2 tiles behind it are still in flight */
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"((SH::STAGES - 2) * SH::NREQ) : "memory");
+        __builtin_amdgcn_s_barrier();                       /* everybody's pieces are in; the stage read in the step before is free again */
         uint32_t adA[4], adB[NJ];
         addrs(st, adA, adB);
         Nt3Ops<NJ> o0, o1;
@@ -217,7 +217,7 @@ __device__ __forceinline__ void nt3_block(const Nt3Args &a, const unsigned bid){
         /* The requests of tile st+2 go out between the multiplications, one after every row of them:
          * a request can wait a hundred cycles for the address unit when eight wavefronts ask at once, and
          * behind an MFMA that wait costs nothing. The fences keep the compiler from gathering them again. */
-        const int nt = st + 2, ns = (st + 2) % NT3_STAGES;
+        const int nt = st + SH::STAGES - 1, ns = nt % SH::STAGES;
 #pragma unroll
         for(int i = 0; i < 4; i++){
 #pragma unroll

@@ -114,11 +114,13 @@ static int nt3_submit(int BN, const Nt3Args &a, int grid, int slot, bool units, 
     return units ? qlmx_unit_done(slot, st) : qlmx_upload_done(slot, st);
 }
 
-/* Which tile. The wide one is built and correct but not faster on this GPU. Uniform experts, K=768 N=2048,
- * TFLOP/s at 512 / 2048 / 8192 rows per expert: 128 columns 733 / 931 / 932; 256 columns 690 / 972 / 872 (on
- * four wavefronts of 128 x 128 it was 636 / 935 / 824); the config-5 step is the same with either (870 and
- * 872 TFLOP/s). So the wide tile is only taken on request: QLMX_NT_TILE=256 in the environment (read at the
- * first call) or qlmx_nt_tile(256). */
+/* Which tile. Uniform experts, K=768 N=2048, TFLOP/s at 512 / 2048 / 8192 rows per expert (8 experts at 8192, which
+ * leaves the wide form 192 tiles for 256 CUs): 128 columns 778 / 950 / 934; 256 columns on eight wavefronts with four
+ * tiles in LDS 724 / 1036 / 905 (with three 690 / 972 / 872, with five 719 / 1003 / 892; on four wavefronts of
+ * 128 x 128 and three tiles 636 / 935 / 824). The wide form wins where experts have a few thousand rows and the
+ * device is not held back by its power limit; the config-3 step has 512-row experts and the config-5 step runs at
+ * the clock its load allows (861.6 against 863.3 TFLOP/s), so the wide tile is only taken on request:
+ * QLMX_NT_TILE=256 in the environment (read at the first call) or qlmx_nt_tile(256). */
 static int g_nt3_forced = -1;
 static int nt3_pick_bn(int N){
     if(g_nt3_forced < 0){ const char *e = getenv("QLMX_NT_TILE"); g_nt3_forced = e ? atoi(e) : 0; }

@@ -492,7 +492,7 @@ __device__ __forceinline__ float df_stage_f32(const float (&v)[DF_NG][DF_MB], bo
 }
 
 /* One task: which slice of which matrix, for which problem. list 0 = none. */
-struct DfT { u64 wq, wg; int list, N, k0, rows, chunk, M, prob, mat, sl; };
+struct DfT { u64 wq, wg; int list, N, k0, rows, chunk, M, prob, mat, sl, ngl; };   /* ngl: scale groups of the chunk that lie inside the row (1 or 2) */
 
 /* first DF_BATCH steps of a task's digits into W (the caller keeps them in flight across the end of
  * the previous task) */
@@ -774,7 +774,7 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
     const int nc1 = nslot > 0 ? (lim1 - slot0 + nslot - 1) / nslot : 0, nc2 = nslot > 0 ? (lim2 - slot0 + nslot - 1) / nslot : 0;
     const int c1 = nc1 > 0 ? nc1 : 0, c2 = nc2 > 0 ? nc2 : 0;           /* candidates of the two lists */
     {
-        DfT t; t.list = 0; t.wq = 0; t.wg = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = 0;
+        DfT t; t.list = 0; t.wq = 0; t.wg = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = t.ngl = 0;
         if(tid < c1){
             const int q = slot0 + tid * nslot;
             /* slot q of this XCD: first its whole groups, then its pieces of the groups left over */
@@ -786,6 +786,7 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
                 const int g = whole ? vg : full1 + gp, part = whole ? 0 : vg - gp * parts1, cl = df_div(sub, a.S1, rS1);
                 t.list = 1; t.prob = g >> 1; t.mat = g & 1; t.chunk = part * cpp1 + cl; t.sl = sub - cl * a.S1;
                 t.N = a.F; t.k0 = t.sl * a.R1; t.rows = min(a.R1, a.D - t.k0); t.M = mt.p_M[t.prob];
+                t.ngl = (ng == 2 && t.N - t.chunk * DF_CW > a.group) ? 2 : 1;
                 const int ex = mt.p_e[t.prob];
                 t.wq = (t.mat ? a.w3q : a.w1q) + (u64)ex * DF;
                 t.wg = (t.mat ? a.w3g : a.w1g) + (u64)ex * a.dfg;
@@ -800,6 +801,7 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
                 const int prob = whole ? vg : full2 + gp, part = whole ? 0 : vg - gp * parts2, cl = df_div(sub, a.S2, rS2);
                 t.list = 2; t.prob = prob; t.mat = 0; t.chunk = part * cpp2 + cl; t.sl = sub - cl * a.S2;
                 t.N = a.D; t.k0 = t.sl * a.R2; t.rows = min(a.R2, a.F - t.k0); t.M = mt.p_M[prob];
+                t.ngl = (ng == 2 && t.N - t.chunk * DF_CW > a.group) ? 2 : 1;
                 const int ex = mt.p_e[prob];
                 t.wq = a.w2q + (u64)ex * DF;
                 t.wg = a.w2g + (u64)ex * a.dfg;
@@ -824,11 +826,11 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
     const int ntasks = min(DF_MAXTASKS, wcount[0] + wcount[1] + wcount[2] + wcount[3]);
     int ti = 0;
     auto fetch = [&]() -> DfT {
-        DfT t; t.list = 0; t.wq = 0; t.wg = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = 0;
+        DfT t; t.list = 0; t.wq = 0; t.wg = 0; t.N = t.k0 = t.rows = t.chunk = t.M = t.prob = t.mat = t.sl = t.ngl = 0;
         if(ti < ntasks){
             const DfT &s = tasks[ti++];
             t.list = df_uni(s.list); t.N = df_uni(s.N); t.k0 = df_uni(s.k0); t.rows = df_uni(s.rows); t.chunk = df_uni(s.chunk);
-            t.M = df_uni(s.M); t.prob = df_uni(s.prob); t.mat = df_uni(s.mat); t.sl = df_uni(s.sl);
+            t.M = df_uni(s.M); t.prob = df_uni(s.prob); t.mat = df_uni(s.mat); t.sl = df_uni(s.sl); t.ngl = df_uni(s.ngl);
             t.wq = ((u64)(unsigned)df_uni((int)(s.wq >> 32)) << 32) | (unsigned)df_uni((int)(unsigned)s.wq);
             t.wg = ((u64)(unsigned)df_uni((int)(s.wg >> 32)) << 32) | (unsigned)df_uni((int)(unsigned)s.wg);
         }
@@ -849,7 +851,7 @@ __global__ void __launch_bounds__(DF_THREADS, 4) k_decode_fused(DfArgs a){
     auto scales_ahead = [&](const DfT &t, float (&sc)[DF_NG]){
         const float *sp = scales_of(t) + (size_t)min(tid, t.rows - 1) * (t.list == 1 ? gprF : gprD);
 #pragma unroll
-        for(int gg = 0; gg < DF_NG; gg++) sc[gg] = sp[(gg < ng && t.chunk * DF_CW + gg * a.group < t.N) ? gg : 0];   /* a group past the row's end re-reads the first */
+        for(int gg = 0; gg < DF_NG; gg++) sc[gg] = sp[gg < t.ngl ? gg : 0];   /* a group past the row's end re-reads the first */
     };
     float csc[DF_NG];
     DF_STAMP(20);
